@@ -1,0 +1,129 @@
+/*
+ * ma_hip.h - C ABI of libma_hip.so: the MonarchAttention forward pass on one
+ * MI355X (gfx950), hand-written HIP kernels.
+ *
+ * This is the boundary a host binding attaches to.  It replaces the body of
+ * the reference's implementation function
+ *
+ *     monarch_attention_torch(q, k, v, attn_mask, T, B, pre_pad) -> Tensor
+ *         (ma/ma_torch.py:65-108; registered through register_impl,
+ *          ma/monarch_attention.py:15-22, called from
+ *          MonarchAttention.forward, ma/monarch_attention.py:50-59)
+ *
+ * Plain pointers and sizes only: no torch types, no C++ in the signatures.
+ * The library never allocates, frees or synchronises device memory in the
+ * entry points below; every buffer belongs to the caller and all work is
+ * enqueued on the stream that is passed in.  Return value of every int
+ * function: 0 = ok, < 0 = ma_status, > 0 = hipError_t of a failed launch.
+ *
+ * Tensor conventions (the reference's, ma/ma_torch.py:74-90):
+ *   q, k : (E, H, N, D)   v : (E, H, N, Dv)   out : (E, H, N, Dv) in v's dtype
+ *   mask : (E, N) bytes, non-zero = keep the key/query token, or NULL
+ *   B block size, M = ceil(N / B) blocks, Np = M * B; zero padding at the
+ *   front (pre_pad != 0) or the back; T alternating steps.
+ * Strides are in ELEMENTS for the dims (e, h, n); the innermost dim must be
+ * contiguous (stride 1).
+ */
+#ifndef MA_HIP_H_
+#define MA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MA_ABI_VERSION 1
+
+typedef enum ma_dtype { MA_F32 = 0, MA_F16 = 1, MA_BF16 = 2 } ma_dtype;
+
+typedef enum ma_variant {
+    MA_VARIANT_AUTO = 0,    /* fastest variant that supports the problem            */
+    MA_VARIANT_GENERIC = 1, /* FMA kernels, 2T(+T-1) launches: any dtype/shape/stride */
+    MA_VARIANT_STAGED = 2,  /* MFMA kernels, one launch per half step (2T launches)  */
+    MA_VARIANT_FUSED = 3    /* MFMA, all T steps in ONE launch                       */
+} ma_variant;
+
+typedef enum ma_status {
+    MA_OK = 0,
+    MA_ERR_NULL = -1,        /* a required pointer is NULL                        */
+    MA_ERR_SHAPE = -2,       /* a dimension, B or T is < 1 (or overflows int32)   */
+    MA_ERR_DTYPE = -3,       /* unknown ma_dtype                                  */
+    MA_ERR_STRIDE = -4,      /* a stride is < 0 or rows overlap                   */
+    MA_ERR_WORKSPACE = -5,   /* workspace missing, misaligned or too small        */
+    MA_ERR_UNSUPPORTED = -6, /* the requested variant cannot run this problem     */
+    MA_ERR_VARIANT = -7,     /* unknown ma_variant                                */
+    MA_ERR_DEVICE = -8       /* no usable gfx950 device / device query failed     */
+} ma_status;
+
+/* Arguments of one forward call; replaces the argument list of
+ * monarch_attention_torch (ma/ma_torch.py:65-73). */
+typedef struct ma_fwd_params {
+    const void* q;           /* device pointers                                   */
+    const void* k;
+    const void* v;
+    const uint8_t* mask;     /* (E, N) or NULL (ma/ma_torch.py:96-98)             */
+    void* out;               /* (E, H, N, Dv), dtype_v                            */
+    void* workspace;         /* >= ma_fwd_workspace_bytes(), 256-byte aligned     */
+    uint64_t workspace_bytes;
+    int32_t E, H, N, D, Dv;
+    int32_t B;               /* block size  (reference argument B)               */
+    int32_t T;               /* num_steps   (reference argument T)               */
+    int32_t pre_pad;         /* pad at the front instead of the back             */
+    int32_t dtype_qk;        /* ma_dtype of q and k                              */
+    int32_t dtype_v;         /* ma_dtype of v and out                            */
+    int32_t variant;         /* ma_variant                                       */
+    int32_t reserved;        /* must be 0                                        */
+    int64_t q_stride[3];     /* element strides of (e, h, n)                     */
+    int64_t k_stride[3];
+    int64_t v_stride[3];
+    int64_t out_stride[3];
+    int64_t mask_stride[2];  /* element (byte) strides of (e, n)                 */
+    float eps;               /* 1e-12 in the reference (ma/ma_torch.py:10,38)    */
+    int32_t reserved2;       /* must be 0                                        */
+} ma_fwd_params;
+
+/* Byte offsets of the per-call state inside the workspace.  The arrays have
+ * exactly the shapes and element types of the reference's intermediates
+ * (ma/ma_torch.py:88-104), so a stage can be checked on its own:
+ *   aR (E,H,M,B,D) dtype_qk   cR (E,H,M,B) f32   [inputs of the R step]
+ *   aL (E,H,B,M,D) dtype_qk   cL (E,H,B,M) f32   Y (E,H,B,M,Dv) dtype_v
+ *   stats: scratch of the generic L step; sync: counters of the fused kernel */
+typedef struct ma_ws_layout {
+    uint64_t aR, cR, aL, cL, Y, stats, sync, total;
+} ma_ws_layout;
+
+int ma_abi_version(void);
+const char* ma_strerror(int status);
+
+/* Validates the problem (pointers may be NULL here) and reports the workspace
+ * it needs.  ma_fwd_workspace_bytes returns 0 for an invalid problem. */
+int ma_fwd_workspace_layout(const ma_fwd_params* p, ma_ws_layout* layout);
+uint64_t ma_fwd_workspace_bytes(const ma_fwd_params* p);
+
+/* The variant MA_VARIANT_AUTO resolves to for this problem (a ma_variant), or
+ * a negative ma_status. */
+int ma_fwd_select_variant(const ma_fwd_params* p);
+
+/* Whole forward pass: replaces monarch_attention_torch (ma/ma_torch.py:65-108).
+ * `stream` is a hipStream_t (NULL = the default stream). */
+int ma_fwd(const ma_fwd_params* p, void* stream);
+
+/* One stage on the state held in the workspace (stage-level parity tests;
+ * variants GENERIC and STAGED).
+ *   ma_r_step  replaces al_cl_ref (ma/ma_torch.py:10-23) and, with with_v != 0,
+ *              al_y_cl_ref (:38-52).  first != 0: take aR = Q, cR = 1 straight
+ *              from q (the state before the first step, :88-89) instead of the
+ *              workspace.  Writes aL, cL (and Y).
+ *   ma_l_step  replaces ar_cr_ref (:26-35): reads aL, cL, writes aR, cR.
+ *   ma_z_step  replaces z_ref (:55-62) and the final slice (:106-108): reads
+ *              aL, cL, Y, writes the N real rows of out. */
+int ma_r_step(const ma_fwd_params* p, int first, int with_v, void* stream);
+int ma_l_step(const ma_fwd_params* p, void* stream);
+int ma_z_step(const ma_fwd_params* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MA_HIP_H_ */

@@ -1,0 +1,209 @@
+// C-ABI layer of libma_hip.so: argument validation, workspace layout, variant
+// selection and the launch sequence of one forward call.  The sequence mirrors
+// the driver of the reference, monarch_attention_torch (ma/ma_torch.py:100-108):
+// (T-1) x [R step, L step], the R step that also forms Y, then the Z step.
+#include "ma_common.h"
+
+#include <cmath>
+#include <cstring>
+
+namespace ma {
+namespace {
+
+constexpr uint64_t kAlign = 256;
+
+uint64_t align_up(uint64_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
+int elt_size(int dt) { return dt == MA_F32 ? 4 : 2; }
+bool dtype_ok(int dt) { return dt == MA_F32 || dt == MA_F16 || dt == MA_BF16; }
+
+// Shape-level validation: everything that can be checked without touching the
+// device.  Pointers are checked separately (layout queries pass NULLs).
+int check_shape(const ma_fwd_params* p) {
+    if (p == nullptr) return MA_ERR_NULL;
+    if (p->E < 1 || p->H < 1 || p->N < 1 || p->D < 1 || p->Dv < 1 || p->B < 1 || p->T < 1) return MA_ERR_SHAPE;
+    if (!dtype_ok(p->dtype_qk) || !dtype_ok(p->dtype_v)) return MA_ERR_DTYPE;
+    if (p->variant < MA_VARIANT_AUTO || p->variant > MA_VARIANT_FUSED) return MA_ERR_VARIANT;
+    const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+    const long long Np = M * p->B;
+    // every launch grid and every in-kernel int index must stay inside int32
+    const long long eh = static_cast<long long>(p->E) * p->H;
+    if (Np > (1LL << 30) || eh > (1LL << 30)) return MA_ERR_SHAPE;
+    if (eh * Np > (1LL << 31) - 1) return MA_ERR_SHAPE;
+    if (M > 16384) return MA_ERR_UNSUPPORTED;  // LDS tile of the generic L step
+    if (p->B > 12288) return MA_ERR_UNSUPPORTED;
+    for (int i = 0; i < 3; ++i)
+        if (p->q_stride[i] < 0 || p->k_stride[i] < 0 || p->v_stride[i] < 0 || p->out_stride[i] < 0) return MA_ERR_STRIDE;
+    if (p->q_stride[2] < p->D || p->k_stride[2] < p->D) {
+        if (p->N > 1) return MA_ERR_STRIDE;  // rows of q / k overlap
+    }
+    if (p->N > 1 && (p->v_stride[2] < p->Dv || p->out_stride[2] < p->Dv)) return MA_ERR_STRIDE;
+    if (p->mask_stride[0] < 0 || p->mask_stride[1] < 0) return MA_ERR_STRIDE;
+    if (!(p->eps >= 0.0f)) return MA_ERR_SHAPE;
+    return MA_OK;
+}
+
+int layout_of(const ma_fwd_params* p, ma_ws_layout* L) {
+    const int st = check_shape(p);
+    if (st != MA_OK) return st;
+    const uint64_t M = (static_cast<uint64_t>(p->N) + p->B - 1) / p->B;
+    const uint64_t rows = static_cast<uint64_t>(p->E) * p->H * M * p->B;  // E*H*Np
+    const uint64_t sq = elt_size(p->dtype_qk), sv = elt_size(p->dtype_v);
+    uint64_t off = 0;
+    L->aR = off; off = align_up(off + rows * p->D * sq);
+    L->cR = off; off = align_up(off + rows * 4);
+    L->aL = off; off = align_up(off + rows * p->D * sq);
+    L->cL = off; off = align_up(off + rows * 4);
+    L->Y = off; off = align_up(off + rows * p->Dv * sv);
+    L->stats = off; off = align_up(off + rows * 8);
+    L->sync = off; off = align_up(off + 4096);
+    L->total = off;
+    return MA_OK;
+}
+
+int check_buffers(const ma_fwd_params* p, const ma_ws_layout& L) {
+    if (!p->q || !p->k || !p->v || !p->out) return MA_ERR_NULL;
+    if (!p->workspace) return MA_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(p->workspace) % kAlign) return MA_ERR_WORKSPACE;
+    if (p->workspace_bytes < L.total) return MA_ERR_WORKSPACE;
+    const uintptr_t aq = elt_size(p->dtype_qk), av = elt_size(p->dtype_v);
+    if (reinterpret_cast<uintptr_t>(p->q) % aq || reinterpret_cast<uintptr_t>(p->k) % aq ||
+        reinterpret_cast<uintptr_t>(p->v) % av || reinterpret_cast<uintptr_t>(p->out) % av)
+        return MA_ERR_STRIDE;
+    return MA_OK;
+}
+
+Problem make_problem(const ma_fwd_params* p, const ma_ws_layout& L) {
+    Problem P;
+    std::memset(&P, 0, sizeof(P));
+    char* ws = static_cast<char*>(p->workspace);
+    P.q = static_cast<const char*>(p->q);
+    P.k = static_cast<const char*>(p->k);
+    P.v = static_cast<const char*>(p->v);
+    P.mask = p->mask;
+    P.out = static_cast<char*>(p->out);
+    P.aR = ws + L.aR;
+    P.cR = reinterpret_cast<float*>(ws + L.cR);
+    P.aL = ws + L.aL;
+    P.cL = reinterpret_cast<float*>(ws + L.cL);
+    P.Y = ws + L.Y;
+    P.stats = reinterpret_cast<float*>(ws + L.stats);
+    P.sync = reinterpret_cast<unsigned*>(ws + L.sync);
+    P.E = p->E; P.H = p->H; P.N = p->N; P.D = p->D; P.Dv = p->Dv; P.B = p->B; P.T = p->T;
+    P.M = (p->N + p->B - 1) / p->B;
+    P.pad_off = p->pre_pad ? P.M * p->B - p->N : 0;  // ma_torch.py:92
+    for (int i = 0; i < 3; ++i) {
+        P.qs[i] = p->q_stride[i]; P.ks[i] = p->k_stride[i];
+        P.vs[i] = p->v_stride[i]; P.os[i] = p->out_stride[i];
+    }
+    P.ms[0] = p->mask_stride[0]; P.ms[1] = p->mask_stride[1];
+    // sm_scale = 1/sqrt(D) as a Python float, used as an fp32 scalar (ma_torch.py:79)
+    P.sm_scale = static_cast<float>(1.0 / std::sqrt(static_cast<double>(p->D)));
+    P.eps = p->eps;
+    return P;
+}
+
+// The variant a problem resolves to.  Only the generic kernels exist in this
+// build of the library; the MFMA variants report MA_ERR_UNSUPPORTED.
+int select_variant(const ma_fwd_params* p) {
+    if (p->variant == MA_VARIANT_AUTO || p->variant == MA_VARIANT_GENERIC) return MA_VARIANT_GENERIC;
+    return MA_ERR_UNSUPPORTED;
+}
+
+struct Prepared {
+    Problem P;
+    int variant;
+};
+
+int prepare(const ma_fwd_params* p, Prepared* out) {
+    ma_ws_layout L;
+    int st = layout_of(p, &L);
+    if (st != MA_OK) return st;
+    st = check_buffers(p, L);
+    if (st != MA_OK) return st;
+    const int v = select_variant(p);
+    if (v < 0) return v;
+    out->P = make_problem(p, L);
+    out->variant = v;
+    return MA_OK;
+}
+
+}  // namespace
+}  // namespace ma
+
+using namespace ma;
+
+extern "C" {
+
+int ma_abi_version(void) { return MA_ABI_VERSION; }
+
+const char* ma_strerror(int status) {
+    switch (status) {
+        case MA_OK: return "ok";
+        case MA_ERR_NULL: return "a required pointer is NULL";
+        case MA_ERR_SHAPE: return "invalid shape: every dimension, B and T must be >= 1 and E*H*Np must fit int32";
+        case MA_ERR_DTYPE: return "unknown dtype (expected MA_F32, MA_F16 or MA_BF16)";
+        case MA_ERR_STRIDE: return "invalid stride or misaligned tensor pointer";
+        case MA_ERR_WORKSPACE: return "workspace missing, not 256-byte aligned or smaller than ma_fwd_workspace_bytes()";
+        case MA_ERR_UNSUPPORTED: return "the requested variant does not support this problem";
+        case MA_ERR_VARIANT: return "unknown variant";
+        case MA_ERR_DEVICE: return "no usable gfx950 device";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
+    return "unknown status";
+}
+
+int ma_fwd_workspace_layout(const ma_fwd_params* p, ma_ws_layout* layout) {
+    if (layout == nullptr) return MA_ERR_NULL;
+    return layout_of(p, layout);
+}
+
+uint64_t ma_fwd_workspace_bytes(const ma_fwd_params* p) {
+    ma_ws_layout L;
+    return layout_of(p, &L) == MA_OK ? L.total : 0;
+}
+
+int ma_fwd_select_variant(const ma_fwd_params* p) {
+    const int st = check_shape(p);
+    if (st != MA_OK) return st;
+    return select_variant(p);
+}
+
+int ma_r_step(const ma_fwd_params* p, int first, int with_v, void* stream) {
+    Prepared pr;
+    const int st = prepare(p, &pr);
+    if (st != MA_OK) return st;
+    return launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, first != 0, with_v != 0, static_cast<hipStream_t>(stream));
+}
+
+int ma_l_step(const ma_fwd_params* p, void* stream) {
+    Prepared pr;
+    const int st = prepare(p, &pr);
+    if (st != MA_OK) return st;
+    return launch_generic_l(pr.P, p->dtype_qk, static_cast<hipStream_t>(stream));
+}
+
+int ma_z_step(const ma_fwd_params* p, void* stream) {
+    Prepared pr;
+    const int st = prepare(p, &pr);
+    if (st != MA_OK) return st;
+    return launch_generic_z(pr.P, p->dtype_qk, p->dtype_v, static_cast<hipStream_t>(stream));
+}
+
+int ma_fwd(const ma_fwd_params* p, void* stream) {
+    Prepared pr;
+    int st = prepare(p, &pr);
+    if (st != MA_OK) return st;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int t = 0; t < p->T - 1; ++t) {
+        st = launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, t == 0, false, s);
+        if (st) return st;
+        st = launch_generic_l(pr.P, p->dtype_qk, s);
+        if (st) return st;
+    }
+    st = launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, p->T == 1, true, s);
+    if (st) return st;
+    return launch_generic_z(pr.P, p->dtype_qk, p->dtype_v, s);
+}
+
+}  // extern "C"

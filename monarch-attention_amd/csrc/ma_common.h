@@ -1,0 +1,54 @@
+// Internal declarations shared by the kernels and the C-ABI layer of libma_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ma_hip.h"
+
+namespace ma {
+
+using f16 = _Float16;
+using bf16 = __bf16;
+
+// Device-side view of one forward call.  Indices follow the reference
+// (ma/ma_torch.py:74-90): token p = m*B + j of the PADDED sequence is block m,
+// in-block position j; the real token is t = p - pad_off, valid iff 0 <= t < N.
+struct Problem {
+    const char* q;
+    const char* k;
+    const char* v;
+    const uint8_t* mask;
+    char* out;
+    char* aR;      // (E,H,M,B,D)  q/k dtype
+    char* aL;      // (E,H,B,M,D)  q/k dtype
+    char* Y;       // (E,H,B,M,Dv) v dtype
+    float* cR;     // (E,H,M,B)
+    float* cL;     // (E,H,B,M)
+    float* stats;  // (E,H,B,M,2)  row max / row sum of the generic L step
+    unsigned* sync;
+    int E, H, N, D, Dv, B, M, T, pad_off;
+    long long qs[3], ks[3], vs[3], os[3], ms[2];
+    float sm_scale, eps;
+};
+
+__device__ __forceinline__ bool token_ok(const Problem& P, int e, int t) {
+    if (t < 0 || t >= P.N) return false;
+    return P.mask == nullptr || P.mask[e * P.ms[0] + t * P.ms[1]] != 0;
+}
+
+template <class T>
+__device__ __forceinline__ float to_f(T x) { return static_cast<float>(x); }
+template <class T>
+__device__ __forceinline__ T from_f(float x) { return static_cast<T>(x); }  // round to nearest even
+template <class T>
+__device__ __forceinline__ float round_to(float x) { return to_f<T>(from_f<T>(x)); }
+template <>
+__device__ __forceinline__ float round_to<float>(float x) { return x; }
+
+// Launchers (defined next to their kernels).  All return a hipError_t.
+int launch_generic_r(const Problem& P, int dt_qk, int dt_v, bool first, bool with_v, hipStream_t s);
+int launch_generic_l(const Problem& P, int dt_qk, hipStream_t s);
+int launch_generic_z(const Problem& P, int dt_qk, int dt_v, hipStream_t s);
+
+}  // namespace ma

@@ -1,0 +1,326 @@
+// Generic stage kernels: plain fp32 FMA arithmetic, every dtype / shape /
+// stride / mask the operator accepts.  They are the correctness backbone (the
+// fp32 path with its 1e-5 bound, ragged and odd shapes, Dv != D, an fp32 V
+// with 16-bit q/k) and the on-device cross-check for the MFMA kernels.
+//
+// Stage -> reference function:
+//   r_step_kernel   al_cl_ref (ma/ma_torch.py:10-23) / al_y_cl_ref (:38-52)
+//   l_stats_kernel + l_accum_kernel   ar_cr_ref (:26-35)
+//   z_step_kernel   z_ref (:55-62) + the final slice (:106-108)
+// The rounding points of the reference are kept: every matmul result is rounded
+// to the operand dtype before the fp32 softmax math, probabilities are rounded
+// to the operand dtype before the second matmul, and sm_scale is applied to aL
+// after that rounding.
+#include "ma_common.h"
+
+namespace ma {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+constexpr float kTiny = 1.17549435e-38f;  // finfo(float32).tiny, ma_torch.py:18
+
+__device__ __forceinline__ float wave_max(float x) {
+    for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o));
+    return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+
+// Row pointer of a padded-sequence token in q / k / v, or nullptr for a pad row.
+template <class T>
+__device__ __forceinline__ const T* tok_row(const char* base, const long long* st, int e, int h, int t, int N) {
+    if (t < 0 || t >= N) return nullptr;
+    return reinterpret_cast<const T*>(base) + e * st[0] + h * st[1] + static_cast<long long>(t) * st[2];
+}
+
+template <class TA, class TB>
+__device__ __forceinline__ float dot_rows(const TA* a, const TB* b, int D) {
+    float acc = 0.f;
+    if (a == nullptr || b == nullptr) return acc;
+    for (int d = 0; d < D; ++d) acc = fmaf(to_f(a[d]), to_f(b[d]), acc);
+    return acc;
+}
+
+// ---------------------------------------------------------------- R step
+// One workgroup: TJ query rows j of one key block (e,h,m).  LDS: S[TJ][B].
+template <class TQ, class TV>
+__global__ __launch_bounds__(kThreads) void r_step_kernel(Problem P, int TJ, int first, int with_v) {
+    extern __shared__ float lds[];
+    const int B = P.B, M = P.M, D = P.D, Dv = P.Dv;
+    const int jt_count = (B + TJ - 1) / TJ;
+    int w = blockIdx.x;
+    const int jt = w % jt_count; w /= jt_count;
+    const int m = w % M; w /= M;
+    const int h = w % P.H;
+    const int e = w / P.H;
+    const int j0 = jt * TJ;
+    const int rows = min(TJ, B - j0);
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const TQ* aR = reinterpret_cast<const TQ*>(P.aR) + (eh * M + m) * B * D;
+    const float* cR = P.cR + (eh * M + m) * B;
+
+    // logits (ma_torch.py:11-13)
+    for (int idx = threadIdx.x; idx < rows * B; idx += kThreads) {
+        const int jj = idx / B, i = idx % B, j = j0 + jj;
+        const TQ* x = first ? tok_row<TQ>(P.q, P.qs, e, h, m * B + j - P.pad_off, P.N) : aR + j * D;
+        const int ti = m * B + i - P.pad_off;
+        const TQ* kr = tok_row<TQ>(P.k, P.ks, e, h, ti, P.N);
+        float s = P.sm_scale * round_to<TQ>(dot_rows(x, kr, D));
+        const float c = first ? 1.0f : cR[j];
+        s = s / (c + P.eps);
+        if (!token_ok(P, e, ti)) s = -INFINITY;
+        lds[jj * B + i] = s;
+    }
+    __syncthreads();
+
+    // clamped-max softmax, tiny clamp, cL = sum r log r (ma_torch.py:14-20)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int jj = wave; jj < rows; jj += kWaves) {
+        float* S = lds + jj * B;
+        float mx = -INFINITY;
+        for (int i = lane; i < B; i += 64) mx = fmaxf(mx, S[i]);
+        mx = fmaxf(wave_max(mx), P.eps);
+        float sum = 0.f;
+        for (int i = lane; i < B; i += 64) {
+            const float p = expf(S[i] - mx);
+            S[i] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum) + P.eps;
+        float ent = 0.f;
+        for (int i = lane; i < B; i += 64) {
+            const float r = fmaxf(S[i] / sum, kTiny);
+            S[i] = r;
+            ent += r * logf(r);
+        }
+        ent = wave_sum(ent);
+        if (lane == 0) P.cL[(eh * B + (j0 + jj)) * M + m] = ent;
+    }
+    __syncthreads();
+
+    // aL = sm_scale * round(R) K, Y = round(R) V  (ma_torch.py:21, :49-50)
+    TQ* aL = reinterpret_cast<TQ*>(P.aL);
+    for (int idx = threadIdx.x; idx < rows * D; idx += kThreads) {
+        const int jj = idx / D, d = idx % D;
+        const float* S = lds + jj * B;
+        float acc = 0.f;
+        for (int i = 0; i < B; ++i) {
+            const TQ* kr = tok_row<TQ>(P.k, P.ks, e, h, m * B + i - P.pad_off, P.N);
+            if (kr) acc = fmaf(round_to<TQ>(S[i]), to_f(kr[d]), acc);
+        }
+        aL[((eh * B + (j0 + jj)) * M + m) * D + d] = from_f<TQ>(P.sm_scale * round_to<TQ>(acc));
+    }
+    if (with_v) {
+        TV* Y = reinterpret_cast<TV*>(P.Y);
+        for (int idx = threadIdx.x; idx < rows * Dv; idx += kThreads) {
+            const int jj = idx / Dv, d = idx % Dv;
+            const float* S = lds + jj * B;
+            float acc = 0.f;
+            for (int i = 0; i < B; ++i) {
+                const TV* vr = tok_row<TV>(P.v, P.vs, e, h, m * B + i - P.pad_off, P.N);
+                if (vr) acc = fmaf(round_to<TV>(S[i]), to_f(vr[d]), acc);
+            }
+            Y[((eh * B + (j0 + jj)) * M + m) * static_cast<long long>(Dv) + d] = from_f<TV>(acc);
+        }
+    }
+}
+
+// ---------------------------------------------------------------- L / Z logits
+// U[ll][k] = round(Qt[j,l,:] . aL[j,k,:]) - cL[j,k] for TL query blocks l.
+template <class TQ>
+__device__ __forceinline__ void lz_logits(const Problem& P, float* U, int e, int h, int j, int l0, int rows) {
+    const int M = P.M, D = P.D;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const TQ* aL = reinterpret_cast<const TQ*>(P.aL) + (eh * P.B + j) * M * D;
+    const float* cL = P.cL + (eh * P.B + j) * M;
+    for (int idx = threadIdx.x; idx < rows * M; idx += kThreads) {
+        const int ll = idx / M, kk = idx % M;
+        const TQ* qr = tok_row<TQ>(P.q, P.qs, e, h, (l0 + ll) * P.B + j - P.pad_off, P.N);
+        U[ll * M + kk] = round_to<TQ>(dot_rows(qr, aL + kk * D, D)) - cL[kk];
+    }
+}
+
+__device__ __forceinline__ void decode_bj(const Problem& P, int tiles, int& e, int& h, int& j, int& tile) {
+    int w = blockIdx.x;
+    tile = w % tiles; w /= tiles;
+    j = w % P.B; w /= P.B;
+    h = w % P.H;
+    e = w / P.H;
+}
+
+// L step, pass 1: softmax statistics over key blocks k for every query block l.
+template <class TQ>
+__global__ __launch_bounds__(kThreads) void l_stats_kernel(Problem P, int TL) {
+    extern __shared__ float lds[];
+    const int M = P.M;
+    int e, h, j, lt;
+    decode_bj(P, (M + TL - 1) / TL, e, h, j, lt);
+    const int l0 = lt * TL, rows = min(TL, M - l0);
+    lz_logits<TQ>(P, lds, e, h, j, l0, rows);
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    for (int ll = wave; ll < rows; ll += kWaves) {
+        const float* U = lds + ll * M;
+        float mx = -INFINITY;
+        for (int k = lane; k < M; k += 64) mx = fmaxf(mx, U[k]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int k = lane; k < M; k += 64) sum += expf(U[k] - mx);
+        sum = wave_sum(sum);
+        if (lane == 0) {
+            float* st = P.stats + ((eh * P.B + j) * M + (l0 + ll)) * 2;
+            st[0] = mx;
+            st[1] = sum;
+        }
+    }
+}
+
+// L step, pass 2: TK key blocks k of one (e,h,j): L[k,l] for all l, then
+// cR[k,j] = sum_l L, aR[k,j,:] = round(L) Qt   (ma_torch.py:29-33).  LDS: Pl[M][TK].
+template <class TQ>
+__global__ __launch_bounds__(kThreads) void l_accum_kernel(Problem P, int TK) {
+    extern __shared__ float lds[];
+    const int M = P.M, D = P.D, B = P.B;
+    int e, h, j, kt;
+    decode_bj(P, (M + TK - 1) / TK, e, h, j, kt);
+    const int k0 = kt * TK, cols = min(TK, M - k0);
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const TQ* aL = reinterpret_cast<const TQ*>(P.aL) + (eh * B + j) * M * D;
+    const float* cL = P.cL + (eh * B + j) * M;
+    const float* st = P.stats + (eh * B + j) * M * 2;
+    for (int idx = threadIdx.x; idx < M * cols; idx += kThreads) {
+        const int l = idx / cols, kk = idx % cols;
+        const int t = l * B + j - P.pad_off;
+        const TQ* qr = tok_row<TQ>(P.q, P.qs, e, h, t, P.N);
+        const float u = round_to<TQ>(dot_rows(qr, aL + (k0 + kk) * D, D)) - cL[k0 + kk];
+        float p = expf(u - st[2 * l]) / st[2 * l + 1];
+        if (!token_ok(P, e, t)) p = 0.f;  // query mask after the softmax (:30)
+        lds[l * TK + kk] = p;
+    }
+    __syncthreads();
+    TQ* aR = reinterpret_cast<TQ*>(P.aR);
+    for (int idx = threadIdx.x; idx < cols * (D + 1); idx += kThreads) {
+        const int kk = idx / (D + 1), d = idx % (D + 1);
+        float acc = 0.f;
+        if (d == D) {
+            for (int l = 0; l < M; ++l) acc += lds[l * TK + kk];
+            P.cR[(eh * M + (k0 + kk)) * B + j] = acc;
+        } else {
+            for (int l = 0; l < M; ++l) {
+                const TQ* qr = tok_row<TQ>(P.q, P.qs, e, h, l * B + j - P.pad_off, P.N);
+                if (qr) acc = fmaf(round_to<TQ>(lds[l * TK + kk]), to_f(qr[d]), acc);
+            }
+            aR[((eh * M + (k0 + kk)) * B + j) * D + d] = from_f<TQ>(acc);
+        }
+    }
+}
+
+// Z step: TL query blocks l of one (e,h,j); writes the real output rows.
+template <class TQ, class TV>
+__global__ __launch_bounds__(kThreads) void z_step_kernel(Problem P, int TL) {
+    extern __shared__ float lds[];
+    const int M = P.M, Dv = P.Dv, B = P.B;
+    int e, h, j, lt;
+    decode_bj(P, (M + TL - 1) / TL, e, h, j, lt);
+    const int l0 = lt * TL, rows = min(TL, M - l0);
+    lz_logits<TQ>(P, lds, e, h, j, l0, rows);
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int ll = wave; ll < rows; ll += kWaves) {
+        float* U = lds + ll * M;
+        float mx = -INFINITY;
+        for (int k = lane; k < M; k += 64) mx = fmaxf(mx, U[k]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int k = lane; k < M; k += 64) {
+            const float p = expf(U[k] - mx);
+            U[k] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum);
+        for (int k = lane; k < M; k += 64) U[k] = U[k] / sum;
+    }
+    __syncthreads();
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const TV* Y = reinterpret_cast<const TV*>(P.Y) + (eh * B + j) * M * static_cast<long long>(Dv);
+    TV* out = reinterpret_cast<TV*>(P.out) + e * P.os[0] + h * P.os[1];
+    for (int idx = threadIdx.x; idx < rows * Dv; idx += kThreads) {
+        const int ll = idx / Dv, d = idx % Dv;
+        const int t = (l0 + ll) * B + j - P.pad_off;
+        if (t < 0 || t >= P.N) continue;  // padded query rows are dropped (:108)
+        const float* U = lds + ll * M;
+        float acc = 0.f;
+        for (int k = 0; k < M; ++k) acc = fmaf(round_to<TV>(U[k]), to_f(Y[k * static_cast<long long>(Dv) + d]), acc);
+        out[static_cast<long long>(t) * P.os[2] + d] = from_f<TV>(acc);
+    }
+}
+
+// rows per workgroup so that rows * width floats fit the LDS budget
+int tile_rows(int width, int want) {
+    const long long budget = 48 * 1024 / 4;
+    long long r = budget / (width > 0 ? width : 1);
+    if (r < 1) r = 1;
+    return static_cast<int>(r < want ? r : want);
+}
+
+template <class F>
+int dispatch_qk(int dt, F&& f) {
+    switch (dt) {
+        case MA_F32: return f(float{});
+        case MA_F16: return f(f16{});
+        default: return f(bf16{});
+    }
+}
+
+}  // namespace
+
+int launch_generic_r(const Problem& P, int dt_qk, int dt_v, bool first, bool with_v, hipStream_t s) {
+    const int TJ = tile_rows(P.B, 16);
+    const long long grid = static_cast<long long>(P.E) * P.H * P.M * ((P.B + TJ - 1) / TJ);
+    const size_t lds = static_cast<size_t>(TJ) * P.B * sizeof(float);
+    return dispatch_qk(dt_qk, [&](auto tq) {
+        using TQ = decltype(tq);
+        return dispatch_qk(dt_v, [&](auto tv) {
+            using TV = decltype(tv);
+            hipLaunchKernelGGL((r_step_kernel<TQ, TV>), dim3(grid), dim3(kThreads), lds, s, P, TJ, first ? 1 : 0,
+                               with_v ? 1 : 0);
+            return static_cast<int>(hipGetLastError());
+        });
+    });
+}
+
+int launch_generic_l(const Problem& P, int dt_qk, hipStream_t s) {
+    const int TL = tile_rows(P.M, 16);
+    const int TK = tile_rows(P.M, 16);
+    const long long ehb = static_cast<long long>(P.E) * P.H * P.B;
+    return dispatch_qk(dt_qk, [&](auto tq) {
+        using TQ = decltype(tq);
+        hipLaunchKernelGGL((l_stats_kernel<TQ>), dim3(ehb * ((P.M + TL - 1) / TL)), dim3(kThreads),
+                           static_cast<size_t>(TL) * P.M * sizeof(float), s, P, TL);
+        int err = static_cast<int>(hipGetLastError());
+        if (err) return err;
+        hipLaunchKernelGGL((l_accum_kernel<TQ>), dim3(ehb * ((P.M + TK - 1) / TK)), dim3(kThreads),
+                           static_cast<size_t>(TK) * P.M * sizeof(float), s, P, TK);
+        return static_cast<int>(hipGetLastError());
+    });
+}
+
+int launch_generic_z(const Problem& P, int dt_qk, int dt_v, hipStream_t s) {
+    const int TL = tile_rows(P.M, 16);
+    const long long grid = static_cast<long long>(P.E) * P.H * P.B * ((P.M + TL - 1) / TL);
+    const size_t lds = static_cast<size_t>(TL) * P.M * sizeof(float);
+    return dispatch_qk(dt_qk, [&](auto tq) {
+        using TQ = decltype(tq);
+        return dispatch_qk(dt_v, [&](auto tv) {
+            using TV = decltype(tv);
+            hipLaunchKernelGGL((z_step_kernel<TQ, TV>), dim3(grid), dim3(kThreads), lds, s, P, TL);
+            return static_cast<int>(hipGetLastError());
+        });
+    });
+}
+
+}  // namespace ma

@@ -1,0 +1,116 @@
+"""Host side of the HIP implementation: marshals torch tensors into the C ABI.
+
+``monarch_attention_hip`` has the signature of the reference's implementation
+functions (``MonarchAttentionFn``, ma/monarch_attention.py:11-13; the torch
+one is ``monarch_attention_torch``, ma/ma_torch.py:65-73):
+
+    fn(q, k, v, attn_mask, T, B, pre_pad) -> Tensor
+
+q, k ``(E, H, N, D)``; v ``(E, H, N, Dv)`` (its dtype is the output dtype and
+may differ from q/k, as in ``get_matrix``); ``attn_mask`` ``(E, N)`` bool /
+int / float, truthy = keep, or ``None``.  Inputs may be arbitrary strided views
+with a contiguous last dimension (models pass permuted ``(E, N, H, D)``
+buffers); nothing is padded or copied on the host - the kernels apply the
+reference's zero padding (ma/ma_torch.py:81-86) by index arithmetic and write
+only the N real rows.  PyTorch provides the device buffers (output, workspace)
+and the stream; all arithmetic happens in libma_hip.so.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _hip_lib as L
+
+Tensor = torch.Tensor
+
+_DTYPES = {torch.float32: L.MA_F32, torch.float16: L.MA_F16, torch.bfloat16: L.MA_BF16}
+
+# default variant of monarch_attention_hip; tests and the benchmark switch it
+# per call through the `variant` keyword
+DEFAULT_VARIANT = "auto"
+
+
+def _check_inputs(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int) -> None:
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+        if t.dim() != 4:
+            raise ValueError(f"{name} must have shape (E, H, N, D), got {tuple(t.shape)}")
+    if q.shape != k.shape:
+        raise ValueError(f"q and k must have the same shape, got {tuple(q.shape)} and {tuple(k.shape)}")
+    if v.shape[:3] != q.shape[:3]:
+        raise ValueError(f"v must share (E, H, N) with q, got {tuple(v.shape)} vs {tuple(q.shape)}")
+    if q.dtype != k.dtype:
+        raise TypeError(f"q and k must have the same dtype, got {q.dtype} and {k.dtype}")
+    if q.dtype not in _DTYPES or v.dtype not in _DTYPES:
+        raise TypeError(f"supported dtypes are float32, float16, bfloat16; got q {q.dtype}, v {v.dtype}")
+    if not (q.device == k.device == v.device):
+        raise ValueError("q, k and v must be on the same device")
+    if min(q.shape) < 1 or v.shape[-1] < 1:
+        raise ValueError(f"empty tensors are not supported, got q {tuple(q.shape)}, v {tuple(v.shape)}")
+    if not isinstance(B, int) or B < 1:
+        raise ValueError(f"block size B must be a positive int, got {B!r}")
+    if not isinstance(T, int) or T < 1:
+        raise ValueError(f"number of steps T must be a positive int, got {T!r}")
+    if attn_mask is not None:
+        if attn_mask.shape != (q.shape[0], q.shape[2]):
+            raise ValueError(f"attn_mask must have shape (E, N) = {(q.shape[0], q.shape[2])}, "
+                             f"got {tuple(attn_mask.shape)}")
+        if attn_mask.device != q.device:
+            raise ValueError("attn_mask must be on the same device as q")
+    if q.device.type != "cuda":
+        raise ValueError(f"the 'hip' implementation needs tensors on a GPU, got {q.device}")
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        raise NotImplementedError("the 'hip' implementation is forward-only: call it under torch.no_grad() "
+                                  "or detach the inputs")
+
+
+def _inner_contiguous(t: Tensor) -> Tensor:
+    return t if t.stride(-1) == 1 or t.shape[-1] == 1 else t.contiguous()
+
+
+def make_params(q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B: int, pre_pad: bool,
+                variant: str = "auto", eps: float = 1e-12) -> L.FwdParams:
+    """Fill a ``ma_fwd_params`` (workspace fields left empty)."""
+    if variant not in L.VARIANTS:
+        raise ValueError(f"unknown variant {variant!r}; available: {', '.join(L.VARIANTS)}")
+    E, H, N, D = q.shape
+    p = L.FwdParams()
+    p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    p.mask = mask_u8.data_ptr() if mask_u8 is not None else None
+    p.E, p.H, p.N, p.D, p.Dv = E, H, N, D, v.shape[-1]
+    p.B, p.T, p.pre_pad = B, T, int(bool(pre_pad))
+    p.dtype_qk, p.dtype_v = _DTYPES[q.dtype], _DTYPES[v.dtype]
+    p.variant = L.VARIANTS[variant]
+    for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("out_stride", out)):
+        s = t.stride()
+        setattr(p, name, (L.C.c_int64 * 3)(s[0], s[1], s[2]))
+    if mask_u8 is not None:
+        p.mask_stride = (L.C.c_int64 * 2)(*mask_u8.stride())
+    p.eps = eps
+    return p
+
+
+def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, T: int, B: int,
+                          pre_pad: bool, *, variant: str | None = None) -> Tensor:
+    """MonarchAttention forward on the current HIP stream; returns a new
+    contiguous ``(E, H, N, Dv)`` tensor of ``v.dtype``."""
+    _check_inputs(q, k, v, attn_mask, T, B)
+    lib = L.load()
+    q, k, v = _inner_contiguous(q), _inner_contiguous(k), _inner_contiguous(v)
+    mask_u8 = None
+    if attn_mask is not None:
+        # truthiness, as torch.logical_and sees it (ma/ma_torch.py:98)
+        mask_u8 = (attn_mask != 0).to(torch.uint8)
+    E, H, N, _ = q.shape
+    with torch.cuda.device(q.device):
+        out = torch.empty((E, H, N, v.shape[-1]), dtype=v.dtype, device=q.device)
+        p = make_params(q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
+        nbytes = lib.ma_fwd_workspace_bytes(p)
+        if nbytes == 0:
+            L.check(lib.ma_fwd_workspace_layout(p, L.WsLayout()), "monarch_attention_hip")
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+        p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        L.check(lib.ma_fwd(p, stream), "ma_fwd")
+    return out

@@ -1,0 +1,137 @@
+"""C-ABI checks that need no GPU: the library loads, exports every symbol the
+header declares, its structs match the ctypes mirror, and invalid calls are
+rejected with the documented status before anything is launched."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+
+from ma import _hip_lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ma_hip.h")
+
+
+def declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"^\s*(?:const\s+char\s*\*|int|uint64_t)\s+(ma_\w+)\s*\(", src, flags=re.M)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    assert set(L.EXPORTS) <= set(names), names
+    assert "ma_fwd" in names and "ma_r_step" in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = L.load()
+    for name in declared_functions():
+        assert hasattr(lib, name), f"libma_hip.so does not export {name}"
+    assert lib.ma_abi_version() == L.ABI_VERSION
+
+
+def test_struct_layout_matches_header(tmp_path):
+    prog = tmp_path / "sz.c"
+    prog.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "ma_hip.h"\n'
+        "int main(void){printf(\"%zu %zu %zu %zu %zu %zu\\n\", sizeof(ma_fwd_params), offsetof(ma_fwd_params,E),"
+        " offsetof(ma_fwd_params,q_stride), offsetof(ma_fwd_params,mask_stride), offsetof(ma_fwd_params,eps),"
+        " sizeof(ma_ws_layout)); return 0;}\n")
+    exe = tmp_path / "sz"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(prog), "-o", str(exe)],
+                   check=True)
+    got = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
+    F = L.FwdParams
+    assert got == [C.sizeof(F), F.E.offset, F.q_stride.offset, F.mask_stride.offset, F.eps.offset,
+                   C.sizeof(L.WsLayout)]
+
+
+def good_params(**kw):
+    p = L.FwdParams()
+    p.E, p.H, p.N, p.D, p.Dv, p.B, p.T = 2, 3, 50, 16, 16, 8, 2
+    p.dtype_qk = p.dtype_v = L.MA_F16
+    for name, inner in (("q_stride", 16), ("k_stride", 16), ("v_stride", 16), ("out_stride", 16)):
+        setattr(p, name, (C.c_int64 * 3)(3 * 50 * inner, 50 * inner, inner))
+    p.eps = 1e-12
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_workspace_layout_is_ordered_and_aligned():
+    lib = L.load()
+    p = good_params()
+    lay = L.WsLayout()
+    assert lib.ma_fwd_workspace_layout(p, lay) == L.MA_OK
+    offs = [lay.aR, lay.cR, lay.aL, lay.cL, lay.Y, lay.stats, lay.sync, lay.total]
+    assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
+    rows = 2 * 3 * 7 * 8                       # E*H*Np with Np = ceil(50/8)*8
+    assert lay.cR - lay.aR >= rows * 16 * 2 and lay.aL - lay.cR >= rows * 4
+    assert lib.ma_fwd_workspace_bytes(p) == lay.total
+
+
+@pytest.mark.parametrize("field,value,status", [
+    ("E", 0, L.MA_ERR_SHAPE), ("N", -3, L.MA_ERR_SHAPE), ("B", 0, L.MA_ERR_SHAPE), ("T", 0, L.MA_ERR_SHAPE),
+    ("Dv", 0, L.MA_ERR_SHAPE), ("dtype_qk", 7, L.MA_ERR_DTYPE), ("dtype_v", -1, L.MA_ERR_DTYPE),
+    ("variant", 9, L.MA_ERR_VARIANT),
+])
+def test_invalid_problem_is_rejected(field, value, status):
+    lib = L.load()
+    p = good_params(**{field: value})
+    assert lib.ma_fwd_workspace_layout(p, L.WsLayout()) == status
+    assert lib.ma_fwd_workspace_bytes(p) == 0
+    assert lib.ma_fwd(p, None) == status
+    assert L.strerror(status)
+
+
+def test_overlapping_rows_and_negative_strides_are_rejected():
+    lib = L.load()
+    p = good_params()
+    p.q_stride = (C.c_int64 * 3)(2400, 800, 8)       # row stride < D
+    assert lib.ma_fwd_workspace_bytes(p) == 0
+    assert lib.ma_fwd(p, None) == L.MA_ERR_STRIDE
+    p = good_params()
+    p.v_stride = (C.c_int64 * 3)(-1, 800, 16)
+    assert lib.ma_fwd(p, None) == L.MA_ERR_STRIDE
+
+
+def test_pointer_and_workspace_checks_precede_any_launch():
+    lib = L.load()
+    p = good_params()
+    assert lib.ma_fwd(p, None) == L.MA_ERR_NULL                      # q/k/v/out NULL
+    p.q = p.k = p.v = p.out = 0x10000
+    assert lib.ma_fwd(p, None) == L.MA_ERR_WORKSPACE                 # no workspace
+    need = lib.ma_fwd_workspace_bytes(p)
+    p.workspace, p.workspace_bytes = 0x100000, need - 1
+    assert lib.ma_fwd(p, None) == L.MA_ERR_WORKSPACE                 # too small
+    p.workspace, p.workspace_bytes = 0x100010, need
+    assert lib.ma_fwd(p, None) == L.MA_ERR_WORKSPACE                 # misaligned
+    p.workspace = 0x100000
+    p.q = 0x10001                                                    # fp16 pointer must be 2-byte aligned
+    assert lib.ma_fwd(p, None) == L.MA_ERR_STRIDE
+    for fn in (lib.ma_l_step, lib.ma_z_step):
+        assert fn(good_params(), None) == L.MA_ERR_NULL
+    assert lib.ma_r_step(good_params(), 1, 0, None) == L.MA_ERR_NULL
+    assert lib.ma_fwd(None, None) == L.MA_ERR_NULL
+
+
+def test_select_variant_reports_a_known_variant():
+    lib = L.load()
+    v = lib.ma_fwd_select_variant(good_params())
+    assert v in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["fused"])
+    p32 = good_params(dtype_qk=L.MA_F32, dtype_v=L.MA_F32)
+    assert lib.ma_fwd_select_variant(p32) == L.VARIANTS["generic"]
+
+
+def test_check_maps_status_to_python_exceptions():
+    with pytest.raises(ValueError):
+        L.check(L.MA_ERR_SHAPE, "x")
+    with pytest.raises(NotImplementedError):
+        L.check(L.MA_ERR_UNSUPPORTED, "x")
+    with pytest.raises(RuntimeError):
+        L.check(L.MA_ERR_WORKSPACE, "x")
+    L.check(L.MA_OK, "x")

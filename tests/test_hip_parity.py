@@ -1,0 +1,320 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle and with the
+committed golden vectors.  Runs on a MI355X only (``-m gpu``).
+
+Gate: fp32 max-abs <= 1e-5; fp16/bf16 <= 2e-2 relative (max-norm and Frobenius)
+plus the reference's own ``allclose(atol = rtol = 1e-2 | 5e-2)``
+(ma/tests/test_ma.py:64-65).  Every variant of the library is checked; a
+variant that does not support a problem must say so (NotImplementedError), it
+must not fall back silently.
+"""
+import pytest
+import torch
+
+from helpers import (DT, assert_parity, block_safe_mask, err_metrics, golden_names, load_golden, seeded_qkv)
+from ma import _hip_lib as L
+from ma.ma_hip import make_params, monarch_attention_hip
+from ma.monarch_attention import MonarchAttention, PadType
+from oracle.ma_oracle import OracleTrace, monarch_attention_oracle, monarch_matrix_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+VARIANTS = ["generic", "staged", "fused", "auto"]
+
+
+def run_hip(q, k, v, mask, T, B, pre, variant):
+    try:
+        out = monarch_attention_hip(q, k, v, mask, T, B, pre, variant=variant)
+    except NotImplementedError as ex:
+        if variant in ("auto", "generic"):
+            raise
+        pytest.skip(f"variant {variant}: {ex}")
+    torch.cuda.synchronize()
+    return out
+
+
+def to_dev(*ts):
+    return tuple(None if t is None else t.to(DEV) for t in ts)
+
+
+# ---------------------------------------------------------------- golden vectors
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("name", golden_names())
+def test_golden_vectors(name, variant):
+    g = load_golden(name)
+    q, k, v, mask = to_dev(g["q"], g["k"], g["v"], g["mask"])
+    out = run_hip(q, k, v, mask, g["T"], g["B"], g["pre"], variant)
+    assert out.shape == g["out"].shape and out.dtype == g["out"].dtype and out.is_contiguous()
+    assert_parity(out.cpu(), g["out"], g["dt"], f"{name}/{variant}")
+
+
+# ---------------------------------------------------------------- the reference's parameter tables, against the oracle
+MATCH = [  # (E, H, N, D, B, T, pre_pad, dtype)   ma/tests/test_ma.py:34-48
+    (1, 1, 16, 16, 4, 2, False, "f16"), (1, 1, 16, 16, 4, 2, True, "f16"), (1, 4, 16, 16, 8, 3, False, "f16"),
+    (1, 1, 19, 16, 4, 2, False, "f16"), (1, 1, 19, 16, 4, 2, True, "f16"), (2, 4, 32, 32, 8, 2, False, "f16"),
+    (2, 1, 24, 16, 8, 3, False, "f16"), (2, 4, 16, 32, 4, 2, False, "bf16"), (1, 1, 16, 32, 4, 2, True, "bf16"),
+    (1, 1, 24, 16, 8, 2, False, "bf16"),
+]
+MASKED = [  # ma/tests/test_ma.py:70-80
+    (1, 1, 16, 16, 4, 2, False, "f16"), (1, 1, 16, 16, 4, 2, True, "f16"), (1, 1, 19, 16, 4, 2, False, "f16"),
+    (1, 4, 19, 16, 4, 3, True, "f16"), (1, 1, 32, 16, 8, 2, False, "f16"), (2, 4, 32, 32, 8, 2, False, "f16"),
+    (1, 1, 16, 16, 4, 2, True, "bf16"), (2, 4, 16, 32, 4, 2, False, "bf16"),
+]
+T1 = [  # (E, H, N, D, B, pre_pad, dtype)   ma/tests/test_ma.py:105-109,125-133
+    (1, 1, 16, 16, 4, False, "f16"), (2, 4, 19, 32, 8, True, "bf16"), (1, 1, 16, 16, 4, True, "f16"),
+    (2, 4, 32, 32, 8, False, "f16"), (1, 1, 19, 16, 4, False, "f16"), (1, 1, 19, 16, 4, True, "f16"),
+    (2, 4, 16, 32, 4, False, "bf16"),
+]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt", MATCH)
+def test_reference_match_table(E, H, N, D, B, T, pre, dt, variant):
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt])
+    ref = monarch_attention_oracle(q, k, v, None, T, B, pre)
+    out = run_hip(*to_dev(q, k, v), None, T, B, pre, variant)
+    assert_parity(out.cpu(), ref, dt)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt", MASKED)
+def test_reference_mask_table(E, H, N, D, B, T, pre, dt, variant):
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt])
+    mask = block_safe_mask(E, N, B)
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre)
+    out = run_hip(*to_dev(q, k, v, mask), T, B, pre, variant)
+    assert not torch.isnan(out).any()
+    assert_parity(out.cpu(), ref, dt)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("E,H,N,D,B,pre,dt", T1)
+def test_reference_t1_table(E, H, N, D, B, pre, dt, variant):
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt])
+    ref = monarch_attention_oracle(q, k, v, None, 1, B, pre)
+    out = run_hip(*to_dev(q, k, v), None, 1, B, pre, variant)
+    assert out.shape == (E, H, N, D)
+    assert_parity(out.cpu(), ref, dt)
+
+
+# ---------------------------------------------------------------- benchmark configurations (reduced batch where the CPU oracle is slow)
+CONFIGS = [  # name, E, H, N, D, B, T, pre, dt, scale
+    ("c1", 1, 1, 256, 64, 16, 1, False, "f32", 1.0),
+    ("c2a_pre", 4, 12, 197, 64, 16, 2, True, "f16", 0.125),
+    ("c2a_post", 4, 12, 197, 64, 16, 2, False, "f16", 0.125),
+    ("c2b", 4, 12, 256, 64, 16, 2, False, "f16", 0.125),
+    ("c3", 4, 12, 512, 64, 32, 2, False, "bf16", 1.0),
+    ("c4", 2, 16, 1024, 72, 32, 3, False, "f16", 1.0),
+    ("cM_T1", 1, 16, 4096, 64, 64, 1, False, "f16", 1.0),
+    ("cM_T2", 1, 16, 4096, 64, 64, 2, False, "f16", 1.0),
+    ("cM_T3", 1, 16, 4096, 64, 64, 3, False, "f16", 1.0),
+    ("c5", 1, 4, 16384, 64, 128, 3, False, "f16", 1.0),
+    ("c3_f32", 1, 4, 512, 64, 32, 2, False, "f32", 1.0),
+    ("bart8k", 1, 2, 8192, 64, 64, 2, False, "bf16", 1.0),
+    ("gps", 1, 2, 7600, 48, 128, 2, False, "f32", 1.0),
+    ("vit_b14", 2, 12, 197, 64, 14, 2, True, "f16", 0.125),
+    ("roberta_b24", 2, 12, 384, 64, 24, 1, False, "f16", 1.0),
+]
+
+
+_ORACLE_CACHE = {}
+
+
+def _config_case(name, E, H, N, D, B, T, pre, dt, scale):
+    """Seeded inputs and the oracle's output for a named configuration (the
+    oracle runs once per configuration, not once per variant)."""
+    if name not in _ORACLE_CACHE:
+        q, k, v = seeded_qkv(E, H, N, D, DT[dt], scale=scale)
+        _ORACLE_CACHE[name] = (q, k, v, monarch_attention_oracle(q, k, v, None, T, B, pre, upcast=True))
+    return _ORACLE_CACHE[name]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("name,E,H,N,D,B,T,pre,dt,scale", CONFIGS)
+def test_benchmark_shapes_against_oracle(name, E, H, N, D, B, T, pre, dt, scale, variant):
+    q, k, v, ref = _config_case(name, E, H, N, D, B, T, pre, dt, scale)
+    out = run_hip(*to_dev(q, k, v), None, T, B, pre, variant)
+    assert_parity(out.cpu(), ref, dt, f"{name}/{variant}")
+
+
+# ---------------------------------------------------------------- stage-level parity (workspace state against the oracle trace)
+def _stage_setup(E, H, N, D, Dv, B, T, pre, dt, vdt, variant, with_mask):
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt], Dv=Dv)
+    v = v.to(DT[vdt])
+    mask = block_safe_mask(E, N, B) if with_mask else None
+    tr = OracleTrace()
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, trace=tr)
+    lib = L.load()
+    qd, kd, vd, md = to_dev(q, k, v, mask)
+    m8 = None if md is None else (md != 0).to(torch.uint8)
+    out = torch.zeros(E, H, N, Dv, dtype=DT[vdt], device=DEV)
+    p = make_params(qd, kd, vd, m8, out, T, B, pre, variant)
+    lay = L.WsLayout()
+    L.check(lib.ma_fwd_workspace_layout(p, lay), "layout")
+    ws = torch.zeros(lay.total, dtype=torch.uint8, device=DEV)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), lay.total
+    keep = (qd, kd, vd, m8, out, ws)
+    M = -(-N // B)
+
+    def view(off, shape, dtype):
+        n = 1
+        for s in shape:
+            n *= s
+        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        return ws[off:off + nbytes].view(dtype).view(*shape)
+
+    state = dict(aR=view(lay.aR, (E, H, M, B, D), DT[dt]), cR=view(lay.cR, (E, H, M, B), torch.float32),
+                 aL=view(lay.aL, (E, H, B, M, D), DT[dt]), cL=view(lay.cL, (E, H, B, M), torch.float32),
+                 Y=view(lay.Y, (E, H, B, M, Dv), DT[vdt]))
+    return lib, p, state, tr, ref, out, keep
+
+
+def _call(fn, *args):
+    st = fn(*args)
+    if st == L.MA_ERR_UNSUPPORTED:
+        pytest.skip("variant does not expose stage entry points for this problem")
+    L.check(st, "stage")
+    torch.cuda.synchronize()
+
+
+STAGE_CASES = [  # E,H,N,D,Dv,B,T,pre,dt,vdt,mask
+    (1, 2, 64, 16, 16, 8, 3, False, "f32", "f32", False),
+    (2, 2, 50, 16, 24, 8, 3, True, "f32", "f32", True),
+    (1, 2, 128, 64, 64, 16, 2, False, "f16", "f16", False),
+    (1, 2, 197, 64, 64, 16, 3, True, "f16", "f16", True),
+    (1, 2, 256, 64, 64, 32, 2, False, "bf16", "bf16", False),
+    (1, 1, 1024, 64, 64, 64, 2, False, "f16", "f16", False),
+    (1, 2, 40, 32, 40, 8, 2, False, "f16", "f32", False),
+]
+
+
+@pytest.mark.parametrize("variant", ["generic", "staged"])
+@pytest.mark.parametrize("E,H,N,D,Dv,B,T,pre,dt,vdt,with_mask", STAGE_CASES)
+def test_stages_against_oracle_trace(E, H, N, D, Dv, B, T, pre, dt, vdt, with_mask, variant):
+    lib, p, st, tr, ref, out, keep = _stage_setup(E, H, N, D, Dv, B, T, pre, dt, vdt, variant, with_mask)
+    tol = dict(f32=(2e-6, 1e-5), f16=(2e-3, 4e-3), bf16=(1.6e-2, 3e-2))[dt]
+
+    def close(got, want, what, scale=1.0):
+        want = want.to(DEV)
+        assert torch.allclose(got.float(), want.float(), atol=tol[0] * scale, rtol=tol[1]), \
+            (what, err_metrics(got, want))
+
+    # every stage is fed the ORACLE's inputs so that differences do not compound
+    for t, step in enumerate(tr.steps):
+        last = t == len(tr.steps) - 1
+        if t > 0:
+            st["aR"].copy_(step["aR"].to(DEV))
+            st["cR"].copy_(step["cR"].to(DEV))
+        _call(lib.ma_r_step, p, int(t == 0), int(last), None)
+        close(st["aL"], step["aL"], f"aL[{t}]")
+        close(st["cL"], step["cL"], f"cL[{t}]", scale=10.0)
+        if last:
+            vt = dict(f32=1.0, f16=1.0, bf16=1.0)[vdt]
+            close(st["Y"], step["Y"], "Y", scale=vt if vdt == dt else 1000.0)
+            break
+        st["aL"].copy_(step["aL"].to(DEV))
+        st["cL"].copy_(step["cL"].to(DEV))
+        _call(lib.ma_l_step, p, None)
+        nxt = tr.steps[t + 1]
+        close(st["cR"], nxt["cR"], f"cR[{t}]", scale=10.0)
+        # aR rows scale with cR; compare on that scale
+        close(st["aR"], nxt["aR"], f"aR[{t}]", scale=4.0)
+    st["aL"].copy_(tr.steps[-1]["aL"].to(DEV))
+    st["cL"].copy_(tr.steps[-1]["cL"].to(DEV))
+    st["Y"].copy_(tr.steps[-1]["Y"].to(DEV))
+    _call(lib.ma_z_step, p, None)
+    assert_parity(out.cpu(), ref, dt if dt == vdt else dt, "Z")
+
+
+# ---------------------------------------------------------------- caller-side layouts and masks
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+def test_permuted_views_as_models_pass_them(dt, variant):
+    """(E,H,N,D) views of an (E,N,H,D) buffer, as every model in the reference
+    passes them (experiments/vit/model.py:73-79)."""
+    E, H, N, D, B, T = 2, 3, 197, 64, 16, 2
+    g = torch.Generator().manual_seed(0)
+    buf = [(0.2 * torch.randn(E, N, H, D, generator=g)).to(DT[dt]) for _ in range(3)]
+    q, k, v = (b.permute(0, 2, 1, 3) for b in buf)
+    assert not q.is_contiguous()
+    ref = monarch_attention_oracle(q, k, v, None, T, B, True, upcast=True)
+    qd, kd, vd = (b.to(DEV).permute(0, 2, 1, 3) for b in buf)
+    out = run_hip(qd, kd, vd, None, T, B, True, variant)
+    assert_parity(out.cpu(), ref, dt)
+    assert torch.equal(qd.cpu(), q)       # inputs are not modified
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("kind", ["bool", "int64", "float"])
+def test_mask_dtypes(kind, variant):
+    E, H, N, D, B, T = 2, 2, 384, 64, 32, 2
+    q, k, v = seeded_qkv(E, H, N, D, torch.float16)
+    keep = torch.arange(N)[None] < torch.tensor([N, N - 131])[:, None]
+    mask = dict(bool=keep, int64=keep.long(), float=keep.float())[kind]
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, False, upcast=True)
+    out = run_hip(*to_dev(q, k, v, mask), T, B, False, variant)
+    assert_parity(out.cpu(), ref, "f16")
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_dead_key_block_gives_no_nan(variant):
+    E, H, N, D, B, T = 1, 2, 256, 64, 32, 2
+    q, k, v = seeded_qkv(E, H, N, D, torch.float16)
+    mask = torch.ones(E, N, dtype=torch.bool)
+    mask[:, 64:96] = False
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, False, upcast=True)
+    out = run_hip(*to_dev(q, k, v, mask), T, B, False, variant)
+    assert torch.isfinite(out.float()).all()
+    assert_parity(out.cpu(), ref, "f16")
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+def test_get_matrix_through_the_module(dt):
+    E, H, N, D, B, T = 1, 2, 96, 32, 16, 2
+    q, k, _ = seeded_qkv(E, H, N, D, DT[dt])
+    mod = MonarchAttention(B, T, PadType.post)
+    A = mod.get_matrix(q.to(DEV), k.to(DEV))
+    ref = monarch_matrix_oracle(q, k, None, T, B, False)
+    assert A.dtype == torch.float32 and A.shape == (E, H, N, N)
+    assert_parity(A.cpu(), ref, dt)
+    assert torch.allclose(A.sum(-1).cpu(), torch.ones(E, H, N), atol=5e-3)
+
+
+def test_module_forward_pre_and_post_pad():
+    q, k, v = seeded_qkv(2, 12, 197, 64, torch.float16, scale=0.125)
+    for pad in (PadType.pre, "post"):
+        mod = MonarchAttention(14, 2, pad)
+        out = mod(*to_dev(q, k, v))
+        ref = monarch_attention_oracle(q, k, v, None, 2, 14, pad == "pre", upcast=True)
+        assert_parity(out.cpu(), ref, "f16")
+
+
+# ---------------------------------------------------------------- size-independent properties at full benchmark sizes
+FULL = [  # E, H, N, D, B, T, dt
+    (64, 12, 197, 64, 16, 2, "f16"), (16, 12, 512, 64, 32, 2, "bf16"), (8, 16, 1024, 72, 32, 3, "f16"),
+    (1, 16, 4096, 64, 64, 2, "f16"), (1, 16, 16384, 64, 128, 3, "f16"),
+]
+
+
+@pytest.mark.parametrize("variant", ["staged", "fused", "auto"])
+@pytest.mark.parametrize("E,H,N,D,B,T,dt", FULL)
+def test_full_size_properties(E, H, N, D, B, T, dt, variant):
+    """At the full benchmark sizes: finite output, bit-reproducible, a single
+    (e, h) slice equals the full call (batch/head independence), the output is
+    within the convex hull of V per coordinate (rows of A are distributions),
+    and the MFMA variants agree with the generic FMA kernels."""
+    g = torch.Generator(device="cpu").manual_seed(11)
+    scale = 0.125 if N == 197 else 1.0
+    q, k, v = ((scale * torch.randn(E, H, N, D, generator=g)).to(DT[dt]).to(DEV) for _ in range(3))
+    out = run_hip(q, k, v, None, T, B, False, variant)
+    assert torch.isfinite(out.float()).all()
+    again = run_hip(q, k, v, None, T, B, False, variant)
+    assert torch.equal(out, again)
+    e, h = E - 1, H // 2
+    one = run_hip(q[e:e + 1, h:h + 1], k[e:e + 1, h:h + 1], v[e:e + 1, h:h + 1], None, T, B, False, variant)
+    assert torch.equal(one[0, 0], out[e, h])
+    slack = 2e-2 * v.float().abs().max()
+    assert (out.float() <= v.float().amax(dim=2, keepdim=True) + slack).all()
+    assert (out.float() >= v.float().amin(dim=2, keepdim=True) - slack).all()
+    sub = slice(0, min(E, 2))
+    gen = run_hip(q[sub], k[sub], v[sub], None, T, B, False, "generic")
+    assert_parity(out[sub].cpu(), gen.cpu(), dt, "vs generic")
