@@ -102,17 +102,52 @@ Problem make_problem(const ma_fwd_params* p, const ma_ws_layout& L) {
     return P;
 }
 
-// The variant a problem resolves to.  Only the generic kernels exist in this
-// build of the library; the MFMA variants report MA_ERR_UNSUPPORTED.
+// What the MFMA kernels need: 16-bit operands of one dtype, Dv == D, 16-byte
+// row chunks (D % 8 == 0 and every row start 16-byte aligned), and block
+// problems that fit the register / LDS tiles (B, M <= 128, D <= 128).
+// Pointers may be NULL in a layout query; they are then not checked.
+bool mfma_supported(const ma_fwd_params* p) {
+    if (p->dtype_qk == MA_F32 || p->dtype_v != p->dtype_qk) return false;
+    if (p->Dv != p->D || p->D % 8 != 0 || p->D > 128) return false;
+    const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+    if (p->B > 128 || M > 128) return false;
+    for (int i = 0; i < 3; ++i)
+        if (p->q_stride[i] % 8 || p->k_stride[i] % 8 || p->v_stride[i] % 8 || p->out_stride[i] % 4) return false;
+    if (reinterpret_cast<uintptr_t>(p->q) % 16 || reinterpret_cast<uintptr_t>(p->k) % 16 ||
+        reinterpret_cast<uintptr_t>(p->v) % 16 || reinterpret_cast<uintptr_t>(p->out) % 8)
+        return false;
+    return true;
+}
+
+// The variant a problem resolves to (the fused variant is not part of this
+// build of the library).
 int select_variant(const ma_fwd_params* p) {
-    if (p->variant == MA_VARIANT_AUTO || p->variant == MA_VARIANT_GENERIC) return MA_VARIANT_GENERIC;
-    return MA_ERR_UNSUPPORTED;
+    const bool fast = mfma_supported(p);
+    switch (p->variant) {
+        case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
+        case MA_VARIANT_STAGED: return fast ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_FUSED: return MA_ERR_UNSUPPORTED;
+        default: return fast ? MA_VARIANT_STAGED : MA_VARIANT_GENERIC;
+    }
 }
 
 struct Prepared {
     Problem P;
     int variant;
 };
+
+int run_r(const Prepared& pr, const ma_fwd_params* p, bool first, bool with_v, hipStream_t s) {
+    if (pr.variant == MA_VARIANT_GENERIC) return launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, first, with_v, s);
+    return p->dtype_qk == MA_F16 ? launch_mfma_r_f16(pr.P, first, with_v, s) : launch_mfma_r_bf16(pr.P, first, with_v, s);
+}
+int run_l(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
+    if (pr.variant == MA_VARIANT_GENERIC) return launch_generic_l(pr.P, p->dtype_qk, s);
+    return p->dtype_qk == MA_F16 ? launch_mfma_l_f16(pr.P, s) : launch_mfma_l_bf16(pr.P, s);
+}
+int run_z(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
+    if (pr.variant == MA_VARIANT_GENERIC) return launch_generic_z(pr.P, p->dtype_qk, p->dtype_v, s);
+    return p->dtype_qk == MA_F16 ? launch_mfma_z_f16(pr.P, s) : launch_mfma_z_bf16(pr.P, s);
+}
 
 int prepare(const ma_fwd_params* p, Prepared* out) {
     ma_ws_layout L;
@@ -173,21 +208,21 @@ int ma_r_step(const ma_fwd_params* p, int first, int with_v, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    return launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, first != 0, with_v != 0, static_cast<hipStream_t>(stream));
+    return run_r(pr, p, first != 0, with_v != 0, static_cast<hipStream_t>(stream));
 }
 
 int ma_l_step(const ma_fwd_params* p, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    return launch_generic_l(pr.P, p->dtype_qk, static_cast<hipStream_t>(stream));
+    return run_l(pr, p, static_cast<hipStream_t>(stream));
 }
 
 int ma_z_step(const ma_fwd_params* p, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    return launch_generic_z(pr.P, p->dtype_qk, p->dtype_v, static_cast<hipStream_t>(stream));
+    return run_z(pr, p, static_cast<hipStream_t>(stream));
 }
 
 int ma_fwd(const ma_fwd_params* p, void* stream) {
@@ -196,14 +231,14 @@ int ma_fwd(const ma_fwd_params* p, void* stream) {
     if (st != MA_OK) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
     for (int t = 0; t < p->T - 1; ++t) {
-        st = launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, t == 0, false, s);
+        st = run_r(pr, p, t == 0, false, s);
         if (st) return st;
-        st = launch_generic_l(pr.P, p->dtype_qk, s);
+        st = run_l(pr, p, s);
         if (st) return st;
     }
-    st = launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, p->T == 1, true, s);
+    st = run_r(pr, p, p->T == 1, true, s);
     if (st) return st;
-    return launch_generic_z(pr.P, p->dtype_qk, p->dtype_v, s);
+    return run_z(pr, p, s);
 }
 
 }  // extern "C"

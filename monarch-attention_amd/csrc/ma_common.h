@@ -51,4 +51,13 @@ int launch_generic_r(const Problem& P, int dt_qk, int dt_v, bool first, bool wit
 int launch_generic_l(const Problem& P, int dt_qk, hipStream_t s);
 int launch_generic_z(const Problem& P, int dt_qk, int dt_v, hipStream_t s);
 
+// MFMA stage kernels (fp16 / bf16, Dv == D <= 128, D % 8 == 0, B, M <= 128,
+// 16-byte aligned rows).
+int launch_mfma_r_f16(const Problem& P, bool first, bool with_v, hipStream_t s);
+int launch_mfma_l_f16(const Problem& P, hipStream_t s);
+int launch_mfma_z_f16(const Problem& P, hipStream_t s);
+int launch_mfma_r_bf16(const Problem& P, bool first, bool with_v, hipStream_t s);
+int launch_mfma_l_bf16(const Problem& P, hipStream_t s);
+int launch_mfma_z_bf16(const Problem& P, hipStream_t s);
+
 }  // namespace ma

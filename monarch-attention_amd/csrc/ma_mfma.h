@@ -1,0 +1,593 @@
+// MFMA building blocks and the three stage bodies (R, L, Z) for fp16 / bf16 on
+// gfx950.  One wavefront (64 lanes) works on a 16-row strip of a block problem
+// with v_mfma_f32_16x16x32_{f16,bf16}; the four waves of a workgroup share the
+// problem's operand tiles in LDS.
+//
+// Lane naming for the 16x16x32 instruction: r = lane % 16, q = lane / 16.
+//   A operand (16 x 32): lane holds row r,    k = 8q .. 8q+7
+//   B operand (32 x 16): lane holds column r, k = 8q .. 8q+7
+//   C / D     (16 x 16): lane holds column r, rows 4q .. 4q+3
+//
+// Every stage is "GEMM1 -> softmax in registers -> GEMM2":
+//   GEMM1  C[w, x] = sum_d W[w, d] X[x, d]     (both operands row-major in d,
+//          so they load as 16-byte vectors: W from its LDS tile, X from HBM)
+//   softmax over w for every x.  In the R and Z steps x is the lane's column,
+//          so the reduction is in-lane plus two cross-lane steps; the L step
+//          needs the transposed orientation and reduces across 16 lanes (DPP).
+//   GEMM2  out^T[d, x] = sum_w Wv^T[d, w] P[w, x].  P is taken straight from
+//          the C registers as the B operand: the k slots of a lane are mapped
+//          to w = 32g + 16(s/4) + 4q + s%4, exactly the rows the lane already
+//          holds of C tiles 2g and 2g+1.  The transposed A operand comes from
+//          the row-major LDS tile with ds_read_b64_tr_b16 (lane 4e+c of a
+//          16-lane group supplies row e, columns 4c..4c+3 of a 4x16 block;
+//          lane i receives column i of that block).
+//
+// Numerics follow the reference's rounding points (ma/ma_torch.py:11,21,27,33,
+// 39,49,50,56,60): GEMM1 is rounded to the operand dtype before the fp32
+// softmax math, probabilities are rounded to the operand dtype for GEMM2,
+// sm_scale multiplies the rounded aL.  Masked keys, padded tokens and tile
+// tails enter the softmax through a -1e30 bias (exp2 underflows to exactly 0).
+#pragma once
+
+#include "ma_common.h"
+
+namespace ma {
+namespace mfma {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = 64 * kWaves;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegBig = -1.0e30f;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+template <class T>
+struct Ops;
+
+template <>
+struct Ops<f16> {
+    typedef _Float16 v8 __attribute__((ext_vector_type(8)));
+    typedef _Float16 v4 __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ f32x4 mma(v8 a, v8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Ops<bf16> {
+    typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+    typedef __bf16 v4 __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ f32x4 mma(v8 a, v8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+// ---- cross-lane reductions -------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+// all-reduce over the 16 lanes of a DPP row (quad xor 1, xor 2, half mirror, mirror)
+__device__ __forceinline__ float row16_max(float x) {
+    x = fmaxf(x, dpp<0xB1>(x));
+    x = fmaxf(x, dpp<0x4E>(x));
+    x = fmaxf(x, dpp<0x141>(x));
+    x = fmaxf(x, dpp<0x140>(x));
+    return x;
+}
+__device__ __forceinline__ float row16_sum(float x) {
+    x += dpp<0xB1>(x);
+    x += dpp<0x4E>(x);
+    x += dpp<0x141>(x);
+    x += dpp<0x140>(x);
+    return x;
+}
+// all-reduce over the four lanes {r, r+16, r+32, r+48}
+__device__ __forceinline__ float quad_rows_max(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16));
+    x = fmaxf(x, __shfl_xor(x, 32));
+    return x;
+}
+__device__ __forceinline__ float quad_rows_sum(float x) {
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+    return x;
+}
+
+// ---- operand tiles ----------------------------------------------------------
+// LDS tile geometry for a head dim that needs DT 16-wide output tiles:
+// KS 32-wide k steps, row pitch LD elements (the +8 staggers rows over banks).
+template <int DT>
+struct Geom {
+    static constexpr int KS = (DT + 1) / 2;
+    static constexpr int COLS = 32 * KS;
+    static constexpr int LD = COLS + 8;
+};
+
+// Cooperative global -> LDS copy of `rows` rows (zero rows where rowptr gives
+// nullptr, zero columns beyond D).  tix / nth: this thread's index and the
+// number of threads that share the copy.
+template <class T, int DT, class RowPtr>
+__device__ __forceinline__ void load_tile(T* tile, int rows, int D, RowPtr rowptr, int tix, int nth) {
+    constexpr int CH = Geom<DT>::COLS / 8;
+    constexpr int LD = Geom<DT>::LD;
+    for (int c = tix; c < rows * CH; c += nth) {
+        const int row = c / CH, ch = c % CH;
+        u32x4 val = {0u, 0u, 0u, 0u};
+        const T* p = rowptr(row);
+        if (p != nullptr && ch * 8 < D) val = *reinterpret_cast<const u32x4*>(p + ch * 8);
+        *reinterpret_cast<u32x4*>(tile + row * LD + ch * 8) = val;
+    }
+}
+
+// B operand of GEMM1 straight from HBM: row `p` (or zeros), k step ks.
+template <class T, int DT>
+__device__ __forceinline__ void load_x(typename Ops<T>::v8 (&x)[Geom<DT>::KS], const T* p, int D, int q) {
+#pragma unroll
+    for (int ks = 0; ks < Geom<DT>::KS; ++ks) {
+        const int col = 32 * ks + 8 * q;
+        u32x4 val = {0u, 0u, 0u, 0u};
+        if (p != nullptr && col < D) val = *reinterpret_cast<const u32x4*>(p + col);
+        x[ks] = __builtin_bit_cast(typename Ops<T>::v8, val);
+    }
+}
+
+template <class T>
+__device__ __forceinline__ typename Ops<T>::v8 lds_row8(const T* tile_elem) {
+    return __builtin_bit_cast(typename Ops<T>::v8, *reinterpret_cast<const u32x4*>(tile_elem));
+}
+
+// Transposed A operand for k step g of GEMM2 from a row-major LDS tile:
+// returns tile[32g + 16(s/4) + 4q + s%4][col0 + r] for s = 0..7.
+template <class T, int NWT>
+__device__ __forceinline__ typename Ops<T>::v8 lds_tr8(const T* tile, int ld, int g, int col0, int r, int q) {
+    typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
+    const int e = r >> 2, c = r & 3;
+    const T* p0 = tile + (32 * g + 4 * q + e) * ld + col0 + 4 * c;
+    i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+    i16x4 hi = {0, 0, 0, 0};
+    if (2 * g + 1 < NWT) hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 16 * ld));
+    typedef short i16x8 __attribute__((ext_vector_type(8)));
+    i16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(typename Ops<T>::v8, v);
+}
+
+// Natural-order transposed A operand (k slot s <-> row 32g + 8q + s), used by
+// the L step whose B operand is read back from LDS in natural order.
+template <class T>
+__device__ __forceinline__ typename Ops<T>::v8 lds_tr8_natural(const T* tile, int ld, int g, int col0, int r, int q) {
+    typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
+    const int e = r >> 2, c = r & 3;
+    const T* p0 = tile + (32 * g + 8 * q + e) * ld + col0 + 4 * c;
+    i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+    i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 4 * ld));
+    typedef short i16x8 __attribute__((ext_vector_type(8)));
+    i16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(typename Ops<T>::v8, v);
+}
+
+// P (fp32, C layout, NWT tiles) -> B operands of GEMM2, rounded to T.
+template <class T, int NWT>
+__device__ __forceinline__ void pack_p(typename Ops<T>::v8 (&pb)[(NWT + 1) / 2], const f32x4 (&C)[NWT]) {
+#pragma unroll
+    for (int g = 0; g < (NWT + 1) / 2; ++g) {
+        typename Ops<T>::v8 v;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            v[s] = from_f<T>(C[2 * g][s]);
+            v[4 + s] = (2 * g + 1 < NWT) ? from_f<T>(C[2 * g + 1][s]) : from_f<T>(0.f);
+        }
+        pb[g] = v;
+    }
+}
+
+// GEMM2: O[dt][v] = sum_w tile[w][16dt + 4q + v] * P[w][x = lane column]
+template <class T, int DT, int NWT>
+__device__ __forceinline__ void gemm2(f32x4 (&O)[DT], const T* tile, const typename Ops<T>::v8 (&pb)[(NWT + 1) / 2],
+                                      int r, int q) {
+    constexpr int LD = Geom<DT>::LD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int g = 0; g < (NWT + 1) / 2; ++g) acc = Ops<T>::mma(lds_tr8<T, NWT>(tile, LD, g, 16 * dt, r, q), pb[g], acc);
+        O[dt] = acc;
+    }
+}
+
+// 4 consecutive output elements (d = 16dt + 4q .. +3) of one row, 8-byte store
+template <class T>
+__device__ __forceinline__ void store4(T* row, int d0, int D, f32x4 v) {
+    if (row == nullptr || d0 >= D) return;  // D is a multiple of 8, d0 of 4
+    typename Ops<T>::v4 o = {from_f<T>(v[0]), from_f<T>(v[1]), from_f<T>(v[2]), from_f<T>(v[3])};
+    *reinterpret_cast<u32x2*>(row + d0) = __builtin_bit_cast(u32x2, o);
+}
+
+template <class T>
+__device__ __forceinline__ const T* token_row(const char* base, const long long* st, int e, int h, int t, int N) {
+    if (t < 0 || t >= N) return nullptr;
+    return reinterpret_cast<const T*>(base) + e * st[0] + h * st[1] + static_cast<long long>(t) * st[2];
+}
+
+// How a workgroup's four waves are shared among block problems with NT strips:
+// WPP waves per problem, PPW problems per workgroup.
+template <int NT>
+struct Split {
+    static_assert(NT == 1 || NT == 2 || NT == 4 || NT == 8, "strip counts are rounded up to a power of two");
+    static constexpr int WPP = NT < kWaves ? NT : kWaves;
+    static constexpr int PPW = kWaves / WPP;
+};
+
+// LDS bytes of one problem slot of each stage
+template <class T, int DT, int NWT>
+struct Lds {
+    static constexpr int ROWS = 16 * NWT;
+    static constexpr int ROWS2 = 32 * ((NWT + 1) / 2);
+    static constexpr int TILE = ROWS * Geom<DT>::LD;                 // elements
+    static constexpr int TILE2 = ROWS2 * Geom<DT>::LD;
+    static constexpr int LDP = ROWS2 + 8;                            // pitch of the transposed L tile
+    static constexpr size_t R = 2 * TILE * sizeof(T) + ROWS * sizeof(float);
+    static constexpr size_t Z = 2 * TILE * sizeof(T) + ROWS * sizeof(float);
+    static constexpr size_t L = (TILE2 + TILE + ROWS * LDP) * sizeof(T) + (1 + Split<NWT>::WPP) * ROWS * sizeof(float);
+};
+
+// ============================================================================
+// R step for one block problem (e,h,m), run by WPP waves (wig = wave in group).
+// smem: K tile, V tile, key bias.   Reference: al_cl_ref / al_y_cl_ref
+// (ma/ma_torch.py:10-23, :38-52).
+// ============================================================================
+template <class T, int DT, int NWT>
+__device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool active, int e, int h, int m, bool first,
+                                          bool with_v, int wig, int lane) {
+    using G = Geom<DT>;
+    using V8 = typename Ops<T>::v8;
+    constexpr int WPP = Split<NWT>::WPP;
+    constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
+    T* Kt = reinterpret_cast<T*>(smem);
+    T* Vt = Kt + Lds<T, DT, NWT>::TILE;
+    float* kbias = reinterpret_cast<float*>(Vt + Lds<T, DT, NWT>::TILE);
+    const int B = P.B, M = P.M, D = P.D;
+    const int r = lane & 15, q = lane >> 4;
+    const int tix = wig * 64 + lane, nth = WPP * 64;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+
+    if (active) {
+        load_tile<T, DT>(Kt, ROWS, D, [&](int i) { return i < B ? token_row<T>(P.k, P.ks, e, h, m * B + i - P.pad_off, P.N) : nullptr; }, tix, nth);
+        if (with_v)
+            load_tile<T, DT>(Vt, ROWS, D, [&](int i) { return i < B ? token_row<T>(P.v, P.vs, e, h, m * B + i - P.pad_off, P.N) : nullptr; }, tix, nth);
+        for (int i = tix; i < ROWS; i += nth) kbias[i] = (i < B && token_ok(P, e, m * B + i - P.pad_off)) ? 0.f : kNegBig;
+    }
+    __syncthreads();
+    if (active) {
+        for (int strip = wig; strip < NWT; strip += WPP) {
+            const int j = 16 * strip + r;
+            const bool jv = j < B;
+            const long long rowid = (eh * M + m) * B + j;
+            const T* xrow = nullptr;
+            if (jv) xrow = first ? token_row<T>(P.q, P.qs, e, h, m * B + j - P.pad_off, P.N) : reinterpret_cast<const T*>(P.aR) + rowid * D;
+            V8 xb[G::KS];
+            load_x<T, DT>(xb, xrow, D, q);
+            const float cr = (first || !jv) ? 1.0f : P.cR[rowid];
+            const float cj = (P.sm_scale * kLog2e) / (cr + P.eps);  // logits in log2 units
+
+            f32x4 C[NWT];
+#pragma unroll
+            for (int wt = 0; wt < NWT; ++wt) {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(lds_row8<T>(Kt + (16 * wt + r) * G::LD + 32 * ks + 8 * q), xb[ks], acc);
+                const f32x4 kb = *reinterpret_cast<const f32x4*>(kbias + 16 * wt + 4 * q);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[v] = fmaf(round_to<T>(acc[v]), cj, kb[v]);
+                C[wt] = acc;
+            }
+            // clamped row maximum (ma_torch.py:15): max(rowmax, eps), here in log2 units
+            float mx = C[0][0];
+#pragma unroll
+            for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) mx = fmaxf(mx, C[wt][v]);
+            mx = fmaxf(quad_rows_max(mx), P.eps * kLog2e);
+            float sum = 0.f, ent = 0.f;
+#pragma unroll
+            for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float d = C[wt][v] - mx;
+                    const float p = __builtin_amdgcn_exp2f(d);
+                    sum += p;
+                    ent = fmaf(p, d, ent);  // sum p * log2(p)
+                    C[wt][v] = p;
+                }
+            sum = quad_rows_sum(sum);
+            ent = quad_rows_sum(ent);
+            const float den = sum + P.eps;
+            const float inv = 1.0f / den;
+#pragma unroll
+            for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) C[wt][v] *= inv;
+            // cL = sum_i r log r with r = p / den (ma_torch.py:20); rows of tiny r add ~1e-36
+            if (jv && q == 0) P.cL[(eh * B + j) * M + m] = kLn2 * ent * inv - logf(den) * (sum * inv);
+
+            V8 pb[(NWT + 1) / 2];
+            pack_p<T, NWT>(pb, C);
+            T* arow = jv ? reinterpret_cast<T*>(P.aL) + ((eh * B + j) * M + m) * D : nullptr;
+            {
+                f32x4 O[DT];
+                gemm2<T, DT, NWT>(O, Kt, pb, r, q);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) O[dt][v] = P.sm_scale * round_to<T>(O[dt][v]);
+                    store4<T>(arow, 16 * dt + 4 * q, D, O[dt]);
+                }
+            }
+            if (with_v) {
+                T* yrow = jv ? reinterpret_cast<T*>(P.Y) + ((eh * B + j) * M + m) * D : nullptr;
+                f32x4 O[DT];
+                gemm2<T, DT, NWT>(O, Vt, pb, r, q);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) store4<T>(yrow, 16 * dt + 4 * q, D, O[dt]);
+            }
+        }
+    }
+}
+
+// ============================================================================
+// Z step for one column problem (e,h,j).  smem: aL tile, Y tile, cL bias.
+// Reference: z_ref (ma/ma_torch.py:55-62) and the final slice (:106-108).
+// ============================================================================
+template <class T, int DT, int NWT>
+__device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool active, int e, int h, int j, int wig,
+                                          int lane) {
+    using G = Geom<DT>;
+    using V8 = typename Ops<T>::v8;
+    constexpr int WPP = Split<NWT>::WPP;
+    constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
+    T* At = reinterpret_cast<T*>(smem);
+    T* Yt = At + Lds<T, DT, NWT>::TILE;
+    float* cb = reinterpret_cast<float*>(Yt + Lds<T, DT, NWT>::TILE);
+    const int B = P.B, M = P.M, D = P.D;
+    const int r = lane & 15, q = lane >> 4;
+    const int tix = wig * 64 + lane, nth = WPP * 64;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+
+    if (active) {
+        const T* aL = reinterpret_cast<const T*>(P.aL) + (eh * B + j) * M * D;
+        const T* Y = reinterpret_cast<const T*>(P.Y) + (eh * B + j) * M * D;
+        load_tile<T, DT>(At, ROWS, D, [&](int k) { return k < M ? aL + k * D : nullptr; }, tix, nth);
+        load_tile<T, DT>(Yt, ROWS, D, [&](int k) { return k < M ? Y + k * D : nullptr; }, tix, nth);
+        const float* cL = P.cL + (eh * B + j) * M;
+        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * cL[k] : kNegBig;
+    }
+    __syncthreads();
+    if (active) {
+        for (int strip = wig; strip < NWT; strip += WPP) {
+            const int l = 16 * strip + r;
+            const int t = l * B + j - P.pad_off;
+            const bool lv = l < M && t >= 0 && t < P.N;
+            V8 xb[G::KS];
+            load_x<T, DT>(xb, lv ? token_row<T>(P.q, P.qs, e, h, t, P.N) : nullptr, D, q);
+            f32x4 C[NWT];
+#pragma unroll
+            for (int wt = 0; wt < NWT; ++wt) {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(lds_row8<T>(At + (16 * wt + r) * G::LD + 32 * ks + 8 * q), xb[ks], acc);
+                const f32x4 b = *reinterpret_cast<const f32x4*>(cb + 16 * wt + 4 * q);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[v] = fmaf(round_to<T>(acc[v]), kLog2e, b[v]);
+                C[wt] = acc;
+            }
+            float mx = C[0][0];
+#pragma unroll
+            for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) mx = fmaxf(mx, C[wt][v]);
+            mx = quad_rows_max(mx);
+            float sum = 0.f;
+#pragma unroll
+            for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float p = __builtin_amdgcn_exp2f(C[wt][v] - mx);
+                    sum += p;
+                    C[wt][v] = p;
+                }
+            const float inv = 1.0f / quad_rows_sum(sum);
+#pragma unroll
+            for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) C[wt][v] *= inv;
+            V8 pb[(NWT + 1) / 2];
+            pack_p<T, NWT>(pb, C);
+            f32x4 O[DT];
+            gemm2<T, DT, NWT>(O, Yt, pb, r, q);
+            T* orow = lv ? reinterpret_cast<T*>(P.out) + e * P.os[0] + h * P.os[1] + static_cast<long long>(t) * P.os[2] : nullptr;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) store4<T>(orow, 16 * dt + 4 * q, D, O[dt]);
+        }
+    }
+}
+
+// ============================================================================
+// L step for one column problem (e,h,j).  smem: Qt tile (ROWS2 rows), aL tile,
+// transposed L tile PT[k][l], cL bias, per-wave partial cR.
+// Reference: ar_cr_ref (ma/ma_torch.py:26-35).
+// ============================================================================
+template <class T, int DT, int NWT>
+__device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool active, int e, int h, int j, int wig,
+                                          int lane) {
+    using G = Geom<DT>;
+    using V8 = typename Ops<T>::v8;
+    using LS = Lds<T, DT, NWT>;
+    constexpr int WPP = Split<NWT>::WPP;
+    constexpr int ROWS = LS::ROWS, ROWS2 = LS::ROWS2, LDP = LS::LDP, NG = (NWT + 1) / 2;
+    T* Qt = reinterpret_cast<T*>(smem);
+    T* At = Qt + LS::TILE2;
+    T* PT = At + LS::TILE;
+    float* cb = reinterpret_cast<float*>(PT + ROWS * LDP);
+    float* crp = cb + ROWS;  // [WPP][ROWS]
+    const int B = P.B, M = P.M, D = P.D;
+    const int r = lane & 15, q = lane >> 4;
+    const int tix = wig * 64 + lane, nth = WPP * 64;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+
+    if (active) {
+        const T* aL = reinterpret_cast<const T*>(P.aL) + (eh * B + j) * M * D;
+        load_tile<T, DT>(Qt, ROWS2, D, [&](int l) { return l < M ? token_row<T>(P.q, P.qs, e, h, l * B + j - P.pad_off, P.N) : nullptr; }, tix, nth);
+        load_tile<T, DT>(At, ROWS, D, [&](int k) { return k < M ? aL + k * D : nullptr; }, tix, nth);
+        const float* cL = P.cL + (eh * B + j) * M;
+        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * cL[k] : kNegBig;
+        if (ROWS2 > ROWS)  // zero the phantom l columns of PT that phase 2 reads
+            for (int i = tix; i < ROWS * (ROWS2 - ROWS); i += nth) PT[(i / (ROWS2 - ROWS)) * LDP + ROWS + i % (ROWS2 - ROWS)] = from_f<T>(0.f);
+    }
+    __syncthreads();
+    if (active) {
+        // phase 1: L[l, k] for 16-row strips of l; lane holds column k = 16kt + r, rows l0 + 4q + v
+        float crsum[NWT];
+#pragma unroll
+        for (int kt = 0; kt < NWT; ++kt) crsum[kt] = 0.f;
+        for (int strip = wig; strip < NWT; strip += WPP) {
+            const int l0 = 16 * strip;
+            V8 xa[G::KS];
+#pragma unroll
+            for (int ks = 0; ks < G::KS; ++ks) xa[ks] = lds_row8<T>(Qt + (l0 + r) * G::LD + 32 * ks + 8 * q);
+            f32x4 C[NWT];
+#pragma unroll
+            for (int kt = 0; kt < NWT; ++kt) {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(xa[ks], lds_row8<T>(At + (16 * kt + r) * G::LD + 32 * ks + 8 * q), acc);
+                const float b = cb[16 * kt + r];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[v] = fmaf(round_to<T>(acc[v]), kLog2e, b);
+                C[kt] = acc;
+            }
+            f32x4 mx = C[0];
+#pragma unroll
+            for (int kt = 1; kt < NWT; ++kt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) mx[v] = fmaxf(mx[v], C[kt][v]);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) mx[v] = row16_max(mx[v]);
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kt = 0; kt < NWT; ++kt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float p = __builtin_amdgcn_exp2f(C[kt][v] - mx[v]);
+                    sum[v] += p;
+                    C[kt][v] = p;
+                }
+            f32x4 inv;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int l = l0 + 4 * q + v;
+                // padded / masked query tokens are zeroed after the softmax (ma_torch.py:30)
+                const bool ok = l < M && token_ok(P, e, l * B + j - P.pad_off);
+                const float s = row16_sum(sum[v]);
+                inv[v] = ok ? 1.0f / s : 0.f;
+            }
+#pragma unroll
+            for (int kt = 0; kt < NWT; ++kt) {
+                typename Ops<T>::v4 o;
+                float part = 0.f;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float lv = C[kt][v] * inv[v];
+                    part += lv;
+                    o[v] = from_f<T>(lv);
+                }
+                crsum[kt] += part;
+                *reinterpret_cast<u32x2*>(PT + (16 * kt + r) * LDP + l0 + 4 * q) = __builtin_bit_cast(u32x2, o);
+            }
+        }
+#pragma unroll
+        for (int kt = 0; kt < NWT; ++kt) {
+            const float s = quad_rows_sum(crsum[kt]);
+            if (q == 0) crp[wig * ROWS + 16 * kt + r] = s;
+        }
+    }
+    __syncthreads();
+    if (active) {
+        // phase 2: aR[k, :] = sum_l round(L[l,k]) Qt[l, :] for 16-wide tiles of k
+        for (int kt = wig; kt < NWT; kt += WPP) {
+            const int k = 16 * kt + r;
+            const bool kv = k < M;
+            V8 pb[NG];
+#pragma unroll
+            for (int g = 0; g < NG; ++g) pb[g] = lds_row8<T>(PT + k * LDP + 32 * g + 8 * q);
+            T* arow = kv ? reinterpret_cast<T*>(P.aR) + ((eh * M + k) * B + j) * D : nullptr;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int g = 0; g < NG; ++g) acc = Ops<T>::mma(lds_tr8_natural<T>(Qt, G::LD, g, 16 * dt, r, q), pb[g], acc);
+                store4<T>(arow, 16 * dt + 4 * q, D, acc);
+            }
+            if (kv && q == 0) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < WPP; ++w) s += crp[w * ROWS + k];
+                P.cR[(eh * M + k) * B + j] = s;
+            }
+        }
+    }
+}
+
+// ---- staged kernels: one launch per half step ---------------------------------
+template <class T, int DT, int NWT>
+__global__ __launch_bounds__(kThreads) void r_step_mfma(Problem P, int first, int with_v) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int slot = wave / WPP, wig = wave % WPP;
+    const long long total = static_cast<long long>(P.E) * P.H * P.M;
+    long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;
+    const bool active = pid < total;
+    if (!active) pid = 0;
+    const int m = pid % P.M;
+    const int h = (pid / P.M) % P.H;
+    const int e = pid / (static_cast<long long>(P.M) * P.H);
+    r_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::R, active, e, h, m, first != 0, with_v != 0, wig, lane);
+}
+
+template <class T, int DT, int NWT>
+__global__ __launch_bounds__(kThreads) void l_step_mfma(Problem P) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int slot = wave / WPP, wig = wave % WPP;
+    const long long total = static_cast<long long>(P.E) * P.H * P.B;
+    long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;
+    const bool active = pid < total;
+    if (!active) pid = 0;
+    const int j = pid % P.B;
+    const int h = (pid / P.B) % P.H;
+    const int e = pid / (static_cast<long long>(P.B) * P.H);
+    l_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::L, active, e, h, j, wig, lane);
+}
+
+template <class T, int DT, int NWT>
+__global__ __launch_bounds__(kThreads) void z_step_mfma(Problem P) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int slot = wave / WPP, wig = wave % WPP;
+    const long long total = static_cast<long long>(P.E) * P.H * P.B;
+    long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;
+    const bool active = pid < total;
+    if (!active) pid = 0;
+    const int j = pid % P.B;
+    const int h = (pid / P.B) % P.H;
+    const int e = pid / (static_cast<long long>(P.B) * P.H);
+    z_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::Z, active, e, h, j, wig, lane);
+}
+
+}  // namespace mfma
+}  // namespace ma

@@ -1,0 +1,86 @@
+// Host-side dispatch of the staged MFMA kernels over (head-dim tiles DT,
+// strip count NWT).  Included by one .hip file per (dtype, stage) so that the
+// instantiations compile in parallel.
+#pragma once
+
+#include "ma_mfma.h"
+
+namespace ma {
+namespace mfma {
+
+inline int dt_class(int D) { return D <= 32 ? 2 : D <= 64 ? 4 : D <= 80 ? 5 : 8; }
+inline int nt_class(int n) {
+    const int t = (n + 15) / 16;
+    return t <= 1 ? 1 : t <= 2 ? 2 : t <= 4 ? 4 : 8;
+}
+
+template <class K>
+int set_lds_limit(K kernel, size_t bytes) {
+    return static_cast<int>(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+}
+
+// calls f(dt_tag, nt_tag) with integral_constant tags for the problem's classes
+template <class F>
+int for_classes(int dt, int nt, F&& f) {
+#define MA_NT(DTV)                                                                            \
+    switch (nt) {                                                                             \
+        case 1: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 1>{}); \
+        case 2: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 2>{}); \
+        case 4: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 4>{}); \
+        default: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 8>{}); \
+    }
+    switch (dt) {
+        case 2: MA_NT(2)
+        case 4: MA_NT(4)
+        case 5: MA_NT(5)
+        default: MA_NT(8)
+    }
+#undef MA_NT
+}
+
+template <class T>
+int launch_r(const Problem& P, bool first, bool with_v, hipStream_t s) {
+    return for_classes(dt_class(P.D), nt_class(P.B), [&](auto dt, auto nt) {
+        constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
+        constexpr int PPW = Split<NWT>::PPW;
+        constexpr size_t lds = PPW * Lds<T, DT, NWT>::R;
+        static const int attr = set_lds_limit(r_step_mfma<T, DT, NWT>, lds);
+        if (attr) return attr;
+        const long long problems = static_cast<long long>(P.E) * P.H * P.M;
+        hipLaunchKernelGGL((r_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P,
+                           first ? 1 : 0, with_v ? 1 : 0);
+        return static_cast<int>(hipGetLastError());
+    });
+}
+
+template <class T>
+int launch_l(const Problem& P, hipStream_t s) {
+    return for_classes(dt_class(P.D), nt_class(P.M), [&](auto dt, auto nt) {
+        constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
+        constexpr int PPW = Split<NWT>::PPW;
+        constexpr size_t lds = PPW * Lds<T, DT, NWT>::L;
+        static const int attr = set_lds_limit(l_step_mfma<T, DT, NWT>, lds);
+        if (attr) return attr;
+        const long long problems = static_cast<long long>(P.E) * P.H * P.B;
+        hipLaunchKernelGGL((l_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P);
+        return static_cast<int>(hipGetLastError());
+    });
+}
+
+template <class T>
+int launch_z(const Problem& P, hipStream_t s) {
+    return for_classes(dt_class(P.D), nt_class(P.M), [&](auto dt, auto nt) {
+        constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
+        constexpr int PPW = Split<NWT>::PPW;
+        constexpr size_t lds = PPW * Lds<T, DT, NWT>::Z;
+        static const int attr = set_lds_limit(z_step_mfma<T, DT, NWT>, lds);
+        if (attr) return attr;
+        const long long problems = static_cast<long long>(P.E) * P.H * P.B;
+        hipLaunchKernelGGL((z_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P);
+        return static_cast<int>(hipGetLastError());
+    });
+}
+
+}  // namespace mfma
+}  // namespace ma

@@ -1,0 +1,8 @@
+// Z-step MFMA kernels, f16 operands.
+#include <type_traits>
+
+#include "ma_mfma_launch.h"
+
+namespace ma {
+int launch_mfma_z_f16(const Problem& P, hipStream_t s) { return mfma::launch_z<f16>(P, s); }
+}  // namespace ma
