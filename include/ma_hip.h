@@ -57,6 +57,13 @@ typedef enum ma_status {
     MA_ERR_DEVICE = -8       /* no usable gfx950 device / device query failed     */
 } ma_status;
 
+/* ma_fwd_params.flags.  MA_FLAG_SYNC_READY: the caller guarantees that the sync
+ * area of the workspace is zero - true after ma_workspace_init() and after every
+ * completed ma_fwd() on that workspace (the fused kernel leaves it zeroed).
+ * Without the flag the fused variant clears the area with one extra small
+ * launch in front of the forward kernel. */
+#define MA_FLAG_SYNC_READY 1
+
 /* Arguments of one forward call; replaces the argument list of
  * monarch_attention_torch (ma/ma_torch.py:65-73). */
 typedef struct ma_fwd_params {
@@ -74,7 +81,7 @@ typedef struct ma_fwd_params {
     int32_t dtype_qk;        /* ma_dtype of q and k                              */
     int32_t dtype_v;         /* ma_dtype of v and out                            */
     int32_t variant;         /* ma_variant                                       */
-    int32_t reserved;        /* must be 0                                        */
+    int32_t flags;           /* MA_FLAG_* bits, 0 if unsure                      */
     int64_t q_stride[3];     /* element strides of (e, h, n)                     */
     int64_t k_stride[3];
     int64_t v_stride[3];
@@ -89,7 +96,9 @@ typedef struct ma_fwd_params {
  * (ma/ma_torch.py:88-104), so a stage can be checked on its own:
  *   aR (E,H,M,B,D) dtype_qk   cR (E,H,M,B) f32   [inputs of the R step]
  *   aL (E,H,B,M,D) dtype_qk   cL (E,H,B,M) f32   Y (E,H,B,M,Dv) dtype_v
- *   stats: scratch of the generic L step; sync: counters of the fused kernel */
+ *   stats: scratch of the generic L step; sync: counters of the fused kernel,
+ *   always at offset 0 so that it does not move when one workspace serves
+ *   calls of different shapes */
 typedef struct ma_ws_layout {
     uint64_t aR, cR, aL, cL, Y, stats, sync, total;
 } ma_ws_layout;
@@ -102,6 +111,13 @@ const char* ma_strerror(int status);
 int ma_fwd_workspace_layout(const ma_fwd_params* p, ma_ws_layout* layout);
 uint64_t ma_fwd_workspace_bytes(const ma_fwd_params* p);
 
+/* Zero-fills the sync area of p->workspace (one small fill kernel on `stream`);
+ * afterwards calls on that workspace may pass MA_FLAG_SYNC_READY.  The
+ * workspace is used by one forward call at a time: calls that share a
+ * workspace must be ordered on one stream.  No counterpart in the reference
+ * (its intermediates are ordinary tensors, ma/ma_torch.py:100-104). */
+int ma_workspace_init(const ma_fwd_params* p, void* stream);
+
 /* The variant MA_VARIANT_AUTO resolves to for this problem (a ma_variant), or
  * a negative ma_status. */
 int ma_fwd_select_variant(const ma_fwd_params* p);
@@ -111,7 +127,8 @@ int ma_fwd_select_variant(const ma_fwd_params* p);
 int ma_fwd(const ma_fwd_params* p, void* stream);
 
 /* One stage on the state held in the workspace (stage-level parity tests;
- * variants GENERIC and STAGED).
+ * variants GENERIC and STAGED; MA_ERR_UNSUPPORTED for FUSED, whose stages are
+ * phases of a single kernel).
  *   ma_r_step  replaces al_cl_ref (ma/ma_torch.py:10-23) and, with with_v != 0,
  *              al_y_cl_ref (:38-52).  first != 0: take aR = Q, cR = 1 straight
  *              from q (the state before the first step, :88-89) instead of the

@@ -23,6 +23,7 @@ int check_shape(const ma_fwd_params* p) {
     if (p->E < 1 || p->H < 1 || p->N < 1 || p->D < 1 || p->Dv < 1 || p->B < 1 || p->T < 1) return MA_ERR_SHAPE;
     if (!dtype_ok(p->dtype_qk) || !dtype_ok(p->dtype_v)) return MA_ERR_DTYPE;
     if (p->variant < MA_VARIANT_AUTO || p->variant > MA_VARIANT_FUSED) return MA_ERR_VARIANT;
+    if (p->flags & ~MA_FLAG_SYNC_READY) return MA_ERR_SHAPE;
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
     const long long Np = M * p->B;
     // every launch grid and every in-kernel int index must stay inside int32
@@ -48,14 +49,16 @@ int layout_of(const ma_fwd_params* p, ma_ws_layout* L) {
     const uint64_t M = (static_cast<uint64_t>(p->N) + p->B - 1) / p->B;
     const uint64_t rows = static_cast<uint64_t>(p->E) * p->H * M * p->B;  // E*H*Np
     const uint64_t sq = elt_size(p->dtype_qk), sv = elt_size(p->dtype_v);
+    // the sync area comes first so that it stays put (and stays zero) when one
+    // workspace serves calls of different shapes
     uint64_t off = 0;
+    L->sync = off; off = align_up(off + kSyncAreaBytes);
     L->aR = off; off = align_up(off + rows * p->D * sq);
     L->cR = off; off = align_up(off + rows * 4);
     L->aL = off; off = align_up(off + rows * p->D * sq);
     L->cL = off; off = align_up(off + rows * 4);
     L->Y = off; off = align_up(off + rows * p->Dv * sv);
     L->stats = off; off = align_up(off + rows * 8);
-    L->sync = off; off = align_up(off + 4096);
     L->total = off;
     return MA_OK;
 }
@@ -119,22 +122,35 @@ bool mfma_supported(const ma_fwd_params* p) {
     return true;
 }
 
-// The variant a problem resolves to (the fused variant is not part of this
-// build of the library).
+// The variant a problem resolves to.
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
     switch (p->variant) {
         case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
         case MA_VARIANT_STAGED: return fast ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
-        case MA_VARIANT_FUSED: return MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_FUSED: return fast ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
         default: return fast ? MA_VARIANT_STAGED : MA_VARIANT_GENERIC;
     }
+}
+
+__global__ void zero_sync_kernel(unsigned* sync, int words) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x) sync[i] = 0u;
 }
 
 struct Prepared {
     Problem P;
     int variant;
 };
+
+int run_fused(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
+    const bool ready = (p->flags & MA_FLAG_SYNC_READY) != 0;
+    const bool h = p->dtype_qk == MA_F16;
+    const int D = p->D;
+    if (D <= 32) return h ? launch_fused_f16_d2(pr.P, ready, s) : launch_fused_bf16_d2(pr.P, ready, s);
+    if (D <= 64) return h ? launch_fused_f16_d4(pr.P, ready, s) : launch_fused_bf16_d4(pr.P, ready, s);
+    if (D <= 80) return h ? launch_fused_f16_d5(pr.P, ready, s) : launch_fused_bf16_d5(pr.P, ready, s);
+    return h ? launch_fused_f16_d8(pr.P, ready, s) : launch_fused_bf16_d8(pr.P, ready, s);
+}
 
 int run_r(const Prepared& pr, const ma_fwd_params* p, bool first, bool with_v, hipStream_t s) {
     if (pr.variant == MA_VARIANT_GENERIC) return launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, first, with_v, s);
@@ -163,6 +179,13 @@ int prepare(const ma_fwd_params* p, Prepared* out) {
 }
 
 }  // namespace
+
+int launch_zero_sync(unsigned* sync, hipStream_t s) {
+    const int words = static_cast<int>(kSyncAreaBytes / 4);
+    hipLaunchKernelGGL(zero_sync_kernel, dim3(8), dim3(256), 0, s, sync, words);
+    return static_cast<int>(hipGetLastError());
+}
+
 }  // namespace ma
 
 using namespace ma;
@@ -198,6 +221,14 @@ uint64_t ma_fwd_workspace_bytes(const ma_fwd_params* p) {
     return layout_of(p, &L) == MA_OK ? L.total : 0;
 }
 
+int ma_workspace_init(const ma_fwd_params* p, void* stream) {
+    ma_ws_layout L;
+    const int st = layout_of(p, &L);
+    if (st != MA_OK) return st;
+    if (!p->workspace || reinterpret_cast<uintptr_t>(p->workspace) % kAlign || p->workspace_bytes < L.total) return MA_ERR_WORKSPACE;
+    return launch_zero_sync(reinterpret_cast<unsigned*>(static_cast<char*>(p->workspace) + L.sync), static_cast<hipStream_t>(stream));
+}
+
 int ma_fwd_select_variant(const ma_fwd_params* p) {
     const int st = check_shape(p);
     if (st != MA_OK) return st;
@@ -208,6 +239,7 @@ int ma_r_step(const ma_fwd_params* p, int first, int with_v, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
+    if (pr.variant == MA_VARIANT_FUSED) return MA_ERR_UNSUPPORTED;
     return run_r(pr, p, first != 0, with_v != 0, static_cast<hipStream_t>(stream));
 }
 
@@ -215,6 +247,7 @@ int ma_l_step(const ma_fwd_params* p, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
+    if (pr.variant == MA_VARIANT_FUSED) return MA_ERR_UNSUPPORTED;
     return run_l(pr, p, static_cast<hipStream_t>(stream));
 }
 
@@ -222,6 +255,7 @@ int ma_z_step(const ma_fwd_params* p, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
+    if (pr.variant == MA_VARIANT_FUSED) return MA_ERR_UNSUPPORTED;
     return run_z(pr, p, static_cast<hipStream_t>(stream));
 }
 
@@ -230,6 +264,7 @@ int ma_fwd(const ma_fwd_params* p, void* stream) {
     int st = prepare(p, &pr);
     if (st != MA_OK) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pr.variant == MA_VARIANT_FUSED) return run_fused(pr, p, s);
     for (int t = 0; t < p->T - 1; ++t) {
         st = run_r(pr, p, t == 0, false, s);
         if (st) return st;

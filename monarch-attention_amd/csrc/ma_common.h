@@ -60,4 +60,19 @@ int launch_mfma_r_bf16(const Problem& P, bool first, bool with_v, hipStream_t s)
 int launch_mfma_l_bf16(const Problem& P, hipStream_t s);
 int launch_mfma_z_bf16(const Problem& P, hipStream_t s);
 
+// Fused forward (one launch), by dtype and head-dim class (D <= 32/64/80/128).
+// sync_ready: the workspace's sync area is known to be zero.
+int launch_fused_f16_d2(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_fused_f16_d4(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_fused_f16_d5(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_fused_f16_d8(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_fused_bf16_d2(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_fused_bf16_d4(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_fused_bf16_d5(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_fused_bf16_d8(const Problem& P, bool sync_ready, hipStream_t s);
+
+constexpr uint64_t kSyncAreaBytes = 4 * (16 + (16 + 2 * 64) * 1024);  // header + one sector per multi-workgroup team
+// Zero-fills the sync area of a workspace (a small fill kernel, graph-capture safe).
+int launch_zero_sync(unsigned* sync, hipStream_t s);
+
 }  // namespace ma

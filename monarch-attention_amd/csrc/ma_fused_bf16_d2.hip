@@ -1,0 +1,6 @@
+// Fused forward kernels, bf16 operands, head-dim class 2 (D <= 32).
+#include "ma_fused_launch.h"
+
+namespace ma {
+int launch_fused_bf16_d2(const Problem& P, bool sync_ready, hipStream_t s) { return mfma::launch_fused<bf16, 2>(P, sync_ready, s); }
+}  // namespace ma

@@ -1,0 +1,6 @@
+// Fused forward kernels, f16 operands, head-dim class 8 (D <= 128).
+#include "ma_fused_launch.h"
+
+namespace ma {
+int launch_fused_f16_d8(const Problem& P, bool sync_ready, hipStream_t s) { return mfma::launch_fused<f16, 8>(P, sync_ready, s); }
+}  // namespace ma

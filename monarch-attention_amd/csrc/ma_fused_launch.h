@@ -1,0 +1,90 @@
+// Host-side planning and dispatch of the fused forward kernel.  Included by one
+// .hip file per (dtype, head-dim class) so the instantiations compile in parallel.
+#pragma once
+
+#include <cstdlib>
+#include <type_traits>
+
+#include "ma_fused.h"
+#include "ma_mfma_launch.h"
+
+namespace ma {
+namespace mfma {
+
+// Team size and team count for `heads` heads when `capacity` workgroups are
+// co-resident: as many workgroups per head as there are tasks in the widest
+// phase, but never more than fit at once; tasks are dealt evenly.
+inline FusedPlan plan_teams(long long heads, int tasks_r, int tasks_l, int capacity) {
+    FusedPlan pl;
+    const int widest = tasks_r > tasks_l ? tasks_r : tasks_l;
+    long long limit = capacity / heads;
+    if (limit < 1) limit = 1;
+    if (limit > widest) limit = widest;
+    if (limit > kMaxTeamSize) limit = kMaxTeamSize;
+    const int per_wg = static_cast<int>((widest + limit - 1) / limit);
+    pl.G = (widest + per_wg - 1) / per_wg;
+    long long nteams = capacity / pl.G;
+    if (nteams > heads) nteams = heads;
+    if (nteams > 8) nteams -= nteams % 8;  // whole teams per XCD
+    pl.nteams = static_cast<int>(nteams);
+    pl.xcd_map = (pl.nteams % 8 == 0) ? 1 : 0;
+    pl.spin_limit = 1u << 22;
+    const char* dbg = getenv("MA_FUSED_DEBUG");
+    pl.debug = dbg ? atoi(dbg) : 0;
+    return pl;
+}
+
+template <class T, int DT, int NTB, int NTM>
+int launch_fused_one(const Problem& P, bool sync_ready, hipStream_t s) {
+    using FL = FusedLds<T, DT, NTB, NTM>;
+    auto kernel = fused_fwd_mfma<T, DT, NTB, NTM>;
+    struct Caps {
+        int err = 0, capacity = 0;
+    };
+    static const Caps caps = [&] {
+        Caps c;
+        c.err = set_lds_limit(kernel, FL::bytes);
+        int dev = 0, cus = 0, per_cu = 0;
+        if (!c.err) c.err = static_cast<int>(hipGetDevice(&dev));
+        if (!c.err) c.err = static_cast<int>(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        if (!c.err)
+            c.err = static_cast<int>(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), kThreads, FL::bytes));
+        c.capacity = cus * per_cu;
+        return c;
+    }();
+    if (caps.err) return caps.err;
+    if (caps.capacity < 1) return MA_ERR_UNSUPPORTED;
+    const long long heads = static_cast<long long>(P.E) * P.H;
+    const int tasks_r = (P.M + Split<NTB>::PPW - 1) / Split<NTB>::PPW;
+    const int tasks_l = (P.B + Split<NTM>::PPW - 1) / Split<NTM>::PPW;
+    const FusedPlan pl = plan_teams(heads, tasks_r, tasks_l, caps.capacity);
+    if (pl.G > 1 && pl.nteams > kMaxTeams) return MA_ERR_UNSUPPORTED;
+    if (!sync_ready) {
+        const int err = launch_zero_sync(P.sync, s);
+        if (err) return err;
+    }
+    hipLaunchKernelGGL((fused_fwd_mfma<T, DT, NTB, NTM>), dim3(pl.nteams * pl.G), dim3(kThreads), FL::bytes, s, P, pl);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <class T, int DT>
+int launch_fused(const Problem& P, bool sync_ready, hipStream_t s) {
+    const int ntb = nt_class(P.B), ntm = nt_class(P.M);
+#define MA_NTM(NB)                                                              \
+    switch (ntm) {                                                              \
+        case 1: return launch_fused_one<T, DT, NB, 1>(P, sync_ready, s);        \
+        case 2: return launch_fused_one<T, DT, NB, 2>(P, sync_ready, s);        \
+        case 4: return launch_fused_one<T, DT, NB, 4>(P, sync_ready, s);        \
+        default: return launch_fused_one<T, DT, NB, 8>(P, sync_ready, s);       \
+    }
+    switch (ntb) {
+        case 1: MA_NTM(1)
+        case 2: MA_NTM(2)
+        case 4: MA_NTM(4)
+        default: MA_NTM(8)
+    }
+#undef MA_NTM
+}
+
+}  // namespace mfma
+}  // namespace ma

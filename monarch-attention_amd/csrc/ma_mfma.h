@@ -110,7 +110,21 @@ struct Geom {
 // Cooperative global -> LDS copy of `rows` rows (zero rows where rowptr gives
 // nullptr, zero columns beyond D).  tix / nth: this thread's index and the
 // number of threads that share the copy.
-template <class T, int DT, class RowPtr>
+// 16-byte global load.  SHARED = true is for state another workgroup wrote during
+// this launch: a streaming ("nt") load, which is served by L2 and never by a
+// line this CU's L1 kept from an earlier step.
+template <bool SHARED>
+__device__ __forceinline__ u32x4 ld16(const void* p) {
+    if (SHARED) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return *reinterpret_cast<const u32x4*>(p);
+}
+template <bool SHARED>
+__device__ __forceinline__ float ldf(const float* p) {
+    if (SHARED) return __builtin_nontemporal_load(p);
+    return *p;
+}
+
+template <class T, int DT, bool SHARED, class RowPtr>
 __device__ __forceinline__ void load_tile(T* tile, int rows, int D, RowPtr rowptr, int tix, int nth) {
     constexpr int CH = Geom<DT>::COLS / 8;
     constexpr int LD = Geom<DT>::LD;
@@ -118,19 +132,19 @@ __device__ __forceinline__ void load_tile(T* tile, int rows, int D, RowPtr rowpt
         const int row = c / CH, ch = c % CH;
         u32x4 val = {0u, 0u, 0u, 0u};
         const T* p = rowptr(row);
-        if (p != nullptr && ch * 8 < D) val = *reinterpret_cast<const u32x4*>(p + ch * 8);
+        if (p != nullptr && ch * 8 < D) val = ld16<SHARED>(p + ch * 8);
         *reinterpret_cast<u32x4*>(tile + row * LD + ch * 8) = val;
     }
 }
 
 // B operand of GEMM1 straight from HBM: row `p` (or zeros), k step ks.
-template <class T, int DT>
+template <class T, int DT, bool SHARED>
 __device__ __forceinline__ void load_x(typename Ops<T>::v8 (&x)[Geom<DT>::KS], const T* p, int D, int q) {
 #pragma unroll
     for (int ks = 0; ks < Geom<DT>::KS; ++ks) {
         const int col = 32 * ks + 8 * q;
         u32x4 val = {0u, 0u, 0u, 0u};
-        if (p != nullptr && col < D) val = *reinterpret_cast<const u32x4*>(p + col);
+        if (p != nullptr && col < D) val = ld16<SHARED>(p + col);
         x[ks] = __builtin_bit_cast(typename Ops<T>::v8, val);
     }
 }
@@ -240,8 +254,8 @@ struct Lds {
 // (ma/ma_torch.py:10-23, :38-52).
 // ============================================================================
 template <class T, int DT, int NWT>
-__device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool active, int e, int h, int m, bool first,
-                                          bool with_v, int wig, int lane) {
+__device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int m,
+                                          bool first, bool with_v, int wig, int lane) {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
     constexpr int WPP = Split<NWT>::WPP;
@@ -252,12 +266,12 @@ __device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool act
     const int B = P.B, M = P.M, D = P.D;
     const int r = lane & 15, q = lane >> 4;
     const int tix = wig * 64 + lane, nth = WPP * 64;
-    const long long eh = static_cast<long long>(e) * P.H + h;
+    const long long eh = wh;  // workspace slot: (e,h) itself in the staged kernels, the team's slot in the fused one
 
     if (active) {
-        load_tile<T, DT>(Kt, ROWS, D, [&](int i) { return i < B ? token_row<T>(P.k, P.ks, e, h, m * B + i - P.pad_off, P.N) : nullptr; }, tix, nth);
+        load_tile<T, DT, false>(Kt, ROWS, D, [&](int i) { return i < B ? token_row<T>(P.k, P.ks, e, h, m * B + i - P.pad_off, P.N) : nullptr; }, tix, nth);
         if (with_v)
-            load_tile<T, DT>(Vt, ROWS, D, [&](int i) { return i < B ? token_row<T>(P.v, P.vs, e, h, m * B + i - P.pad_off, P.N) : nullptr; }, tix, nth);
+            load_tile<T, DT, false>(Vt, ROWS, D, [&](int i) { return i < B ? token_row<T>(P.v, P.vs, e, h, m * B + i - P.pad_off, P.N) : nullptr; }, tix, nth);
         for (int i = tix; i < ROWS; i += nth) kbias[i] = (i < B && token_ok(P, e, m * B + i - P.pad_off)) ? 0.f : kNegBig;
     }
     __syncthreads();
@@ -269,8 +283,8 @@ __device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool act
             const T* xrow = nullptr;
             if (jv) xrow = first ? token_row<T>(P.q, P.qs, e, h, m * B + j - P.pad_off, P.N) : reinterpret_cast<const T*>(P.aR) + rowid * D;
             V8 xb[G::KS];
-            load_x<T, DT>(xb, xrow, D, q);
-            const float cr = (first || !jv) ? 1.0f : P.cR[rowid];
+            if (first) load_x<T, DT, false>(xb, xrow, D, q); else load_x<T, DT, true>(xb, xrow, D, q);
+            const float cr = (first || !jv) ? 1.0f : ldf<true>(P.cR + rowid);
             const float cj = (P.sm_scale * kLog2e) / (cr + P.eps);  // logits in log2 units
 
             f32x4 C[NWT];
@@ -342,8 +356,8 @@ __device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool act
 // Reference: z_ref (ma/ma_torch.py:55-62) and the final slice (:106-108).
 // ============================================================================
 template <class T, int DT, int NWT>
-__device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool active, int e, int h, int j, int wig,
-                                          int lane) {
+__device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int j,
+                                          int wig, int lane) {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
     constexpr int WPP = Split<NWT>::WPP;
@@ -354,15 +368,15 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
     const int B = P.B, M = P.M, D = P.D;
     const int r = lane & 15, q = lane >> 4;
     const int tix = wig * 64 + lane, nth = WPP * 64;
-    const long long eh = static_cast<long long>(e) * P.H + h;
+    const long long eh = wh;  // workspace slot: (e,h) itself in the staged kernels, the team's slot in the fused one
 
     if (active) {
         const T* aL = reinterpret_cast<const T*>(P.aL) + (eh * B + j) * M * D;
         const T* Y = reinterpret_cast<const T*>(P.Y) + (eh * B + j) * M * D;
-        load_tile<T, DT>(At, ROWS, D, [&](int k) { return k < M ? aL + k * D : nullptr; }, tix, nth);
-        load_tile<T, DT>(Yt, ROWS, D, [&](int k) { return k < M ? Y + k * D : nullptr; }, tix, nth);
+        load_tile<T, DT, true>(At, ROWS, D, [&](int k) { return k < M ? aL + k * D : nullptr; }, tix, nth);
+        load_tile<T, DT, true>(Yt, ROWS, D, [&](int k) { return k < M ? Y + k * D : nullptr; }, tix, nth);
         const float* cL = P.cL + (eh * B + j) * M;
-        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * cL[k] : kNegBig;
+        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * ldf<true>(cL + k) : kNegBig;
     }
     __syncthreads();
     if (active) {
@@ -371,7 +385,7 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
             const int t = l * B + j - P.pad_off;
             const bool lv = l < M && t >= 0 && t < P.N;
             V8 xb[G::KS];
-            load_x<T, DT>(xb, lv ? token_row<T>(P.q, P.qs, e, h, t, P.N) : nullptr, D, q);
+            load_x<T, DT, false>(xb, lv ? token_row<T>(P.q, P.qs, e, h, t, P.N) : nullptr, D, q);
             f32x4 C[NWT];
 #pragma unroll
             for (int wt = 0; wt < NWT; ++wt) {
@@ -420,8 +434,8 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
 // Reference: ar_cr_ref (ma/ma_torch.py:26-35).
 // ============================================================================
 template <class T, int DT, int NWT>
-__device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool active, int e, int h, int j, int wig,
-                                          int lane) {
+__device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int j,
+                                          int wig, int lane) {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
     using LS = Lds<T, DT, NWT>;
@@ -435,14 +449,14 @@ __device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool act
     const int B = P.B, M = P.M, D = P.D;
     const int r = lane & 15, q = lane >> 4;
     const int tix = wig * 64 + lane, nth = WPP * 64;
-    const long long eh = static_cast<long long>(e) * P.H + h;
+    const long long eh = wh;  // workspace slot: (e,h) itself in the staged kernels, the team's slot in the fused one
 
     if (active) {
         const T* aL = reinterpret_cast<const T*>(P.aL) + (eh * B + j) * M * D;
-        load_tile<T, DT>(Qt, ROWS2, D, [&](int l) { return l < M ? token_row<T>(P.q, P.qs, e, h, l * B + j - P.pad_off, P.N) : nullptr; }, tix, nth);
-        load_tile<T, DT>(At, ROWS, D, [&](int k) { return k < M ? aL + k * D : nullptr; }, tix, nth);
+        load_tile<T, DT, false>(Qt, ROWS2, D, [&](int l) { return l < M ? token_row<T>(P.q, P.qs, e, h, l * B + j - P.pad_off, P.N) : nullptr; }, tix, nth);
+        load_tile<T, DT, true>(At, ROWS, D, [&](int k) { return k < M ? aL + k * D : nullptr; }, tix, nth);
         const float* cL = P.cL + (eh * B + j) * M;
-        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * cL[k] : kNegBig;
+        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * ldf<true>(cL + k) : kNegBig;
         if (ROWS2 > ROWS)  // zero the phantom l columns of PT that phase 2 reads
             for (int i = tix; i < ROWS * (ROWS2 - ROWS); i += nth) PT[(i / (ROWS2 - ROWS)) * LDP + ROWS + i % (ROWS2 - ROWS)] = from_f<T>(0.f);
     }
@@ -554,7 +568,8 @@ __global__ __launch_bounds__(kThreads) void r_step_mfma(Problem P, int first, in
     const int m = pid % P.M;
     const int h = (pid / P.M) % P.H;
     const int e = pid / (static_cast<long long>(P.M) * P.H);
-    r_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::R, active, e, h, m, first != 0, with_v != 0, wig, lane);
+    r_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::R, active, e, h, static_cast<long long>(e) * P.H + h, m, first != 0,
+                          with_v != 0, wig, lane);
 }
 
 template <class T, int DT, int NWT>
@@ -570,7 +585,7 @@ __global__ __launch_bounds__(kThreads) void l_step_mfma(Problem P) {
     const int j = pid % P.B;
     const int h = (pid / P.B) % P.H;
     const int e = pid / (static_cast<long long>(P.B) * P.H);
-    l_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::L, active, e, h, j, wig, lane);
+    l_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::L, active, e, h, static_cast<long long>(e) * P.H + h, j, wig, lane);
 }
 
 template <class T, int DT, int NWT>
@@ -586,7 +601,7 @@ __global__ __launch_bounds__(kThreads) void z_step_mfma(Problem P) {
     const int j = pid % P.B;
     const int h = (pid / P.B) % P.H;
     const int e = pid / (static_cast<long long>(P.B) * P.H);
-    z_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::Z, active, e, h, j, wig, lane);
+    z_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::Z, active, e, h, static_cast<long long>(e) * P.H + h, j, wig, lane);
 }
 
 }  // namespace mfma

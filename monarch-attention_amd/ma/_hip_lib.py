@@ -29,7 +29,7 @@ class FwdParams(C.Structure):
         ("out", C.c_void_p), ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
         ("E", C.c_int32), ("H", C.c_int32), ("N", C.c_int32), ("D", C.c_int32), ("Dv", C.c_int32),
         ("B", C.c_int32), ("T", C.c_int32), ("pre_pad", C.c_int32),
-        ("dtype_qk", C.c_int32), ("dtype_v", C.c_int32), ("variant", C.c_int32), ("reserved", C.c_int32),
+        ("dtype_qk", C.c_int32), ("dtype_v", C.c_int32), ("variant", C.c_int32), ("flags", C.c_int32),
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("out_stride", C.c_int64 * 3), ("mask_stride", C.c_int64 * 2),
         ("eps", C.c_float), ("reserved2", C.c_int32),
@@ -41,8 +41,10 @@ class WsLayout(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("aR", "cR", "aL", "cL", "Y", "stats", "sync", "total")]
 
 
+MA_FLAG_SYNC_READY = 1
+
 EXPORTS = ("ma_abi_version", "ma_strerror", "ma_fwd_workspace_layout", "ma_fwd_workspace_bytes",
-           "ma_fwd_select_variant", "ma_fwd", "ma_r_step", "ma_l_step", "ma_z_step")
+           "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_r_step", "ma_l_step", "ma_z_step")
 
 _lock = threading.Lock()
 _lib = None
@@ -77,6 +79,8 @@ def load() -> C.CDLL:
         lib.ma_fwd_workspace_layout.argtypes = [P, C.POINTER(WsLayout)]
         lib.ma_fwd_workspace_bytes.restype = C.c_uint64
         lib.ma_fwd_workspace_bytes.argtypes = [P]
+        lib.ma_workspace_init.restype = C.c_int
+        lib.ma_workspace_init.argtypes = [P, C.c_void_p]
         lib.ma_fwd_select_variant.restype = C.c_int
         lib.ma_fwd_select_variant.argtypes = [P]
         lib.ma_fwd.restype = C.c_int

@@ -29,6 +29,27 @@ _DTYPES = {torch.float32: L.MA_F32, torch.float16: L.MA_F16, torch.bfloat16: L.M
 # per call through the `variant` keyword
 DEFAULT_VARIANT = "auto"
 
+# One workspace per (device, stream), grown on demand and reused call after
+# call: calls on one stream are ordered, so they can share it, and a reused
+# buffer keeps the intermediate state of the fused kernel resident in L2.  It
+# is allocated zero-filled and every forward call leaves its sync area zeroed,
+# which is what MA_FLAG_SYNC_READY promises to the library.
+_WORKSPACES: dict[tuple[int, int], Tensor] = {}
+
+
+def _workspace(device: torch.device, stream_ptr: int, nbytes: int) -> Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = ws
+    return ws
+
+
+def clear_workspace_cache() -> None:
+    """Drop the cached per-stream workspaces (frees their device memory)."""
+    _WORKSPACES.clear()
+
 
 def _check_inputs(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int) -> None:
     for name, t in (("q", q), ("k", k), ("v", v)):
@@ -109,8 +130,9 @@ def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | N
         nbytes = lib.ma_fwd_workspace_bytes(p)
         if nbytes == 0:
             L.check(lib.ma_fwd_workspace_layout(p, L.WsLayout()), "monarch_attention_hip")
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-        p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
         stream = torch.cuda.current_stream(q.device).cuda_stream
+        ws = _workspace(q.device, stream, nbytes)
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+        p.flags = L.MA_FLAG_SYNC_READY
         L.check(lib.ma_fwd(p, stream), "ma_fwd")
     return out

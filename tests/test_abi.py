@@ -67,8 +67,8 @@ def test_workspace_layout_is_ordered_and_aligned():
     p = good_params()
     lay = L.WsLayout()
     assert lib.ma_fwd_workspace_layout(p, lay) == L.MA_OK
-    offs = [lay.aR, lay.cR, lay.aL, lay.cL, lay.Y, lay.stats, lay.sync, lay.total]
-    assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
+    offs = [lay.sync, lay.aR, lay.cR, lay.aL, lay.cL, lay.Y, lay.stats, lay.total]
+    assert lay.sync == 0 and offs == sorted(offs) and all(o % 256 == 0 for o in offs)
     rows = 2 * 3 * 7 * 8                       # E*H*Np with Np = ceil(50/8)*8
     assert lay.cR - lay.aR >= rows * 16 * 2 and lay.aL - lay.cR >= rows * 4
     assert lib.ma_fwd_workspace_bytes(p) == lay.total
