@@ -115,21 +115,33 @@ bool mfma_supported(const ma_fwd_params* p) {
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
     if (p->B > 128 || M > 128) return false;
     for (int i = 0; i < 3; ++i)
-        if (p->q_stride[i] % 8 || p->k_stride[i] % 8 || p->v_stride[i] % 8 || p->out_stride[i] % 4) return false;
+        if (p->q_stride[i] % 8 || p->k_stride[i] % 8 || p->v_stride[i] % 8 || p->out_stride[i] % 8) return false;
     if (reinterpret_cast<uintptr_t>(p->q) % 16 || reinterpret_cast<uintptr_t>(p->k) % 16 ||
-        reinterpret_cast<uintptr_t>(p->v) % 16 || reinterpret_cast<uintptr_t>(p->out) % 8)
+        reinterpret_cast<uintptr_t>(p->v) % 16 || reinterpret_cast<uintptr_t>(p->out) % 16)
+        return false;
+    // one (e, h) slice of every tensor and one head of state must fit a 32-bit byte offset
+    const unsigned long long lim = 0xFFFF0000ull;
+    const unsigned long long n1 = static_cast<unsigned long long>(p->N - 1), db = 2ull * p->D;
+    if (n1 * p->q_stride[2] * 2 + db >= lim || n1 * p->k_stride[2] * 2 + db >= lim || n1 * p->v_stride[2] * 2 + db >= lim ||
+        n1 * p->out_stride[2] * 2 + db >= lim || static_cast<unsigned long long>(M) * p->B * db >= lim)
         return false;
     return true;
 }
 
-// The variant a problem resolves to.
+// The variant a problem resolves to.  AUTO: the MFMA kernels when the problem
+// qualifies; among them the one-launch kernel when there are enough heads to
+// give every team several problems per phase (measured: with E*H >= 32 it beats
+// the per-stage launches, with fewer, larger teams the launch boundaries are
+// cheaper than its in-kernel barriers).
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
     switch (p->variant) {
         case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
         case MA_VARIANT_STAGED: return fast ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_FUSED: return fast ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
-        default: return fast ? MA_VARIANT_STAGED : MA_VARIANT_GENERIC;
+        default:
+            if (!fast) return MA_VARIANT_GENERIC;
+            return static_cast<long long>(p->E) * p->H >= 32 ? MA_VARIANT_FUSED : MA_VARIANT_STAGED;
     }
 }
 

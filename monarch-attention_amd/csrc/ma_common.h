@@ -71,7 +71,7 @@ int launch_fused_bf16_d4(const Problem& P, bool sync_ready, hipStream_t s);
 int launch_fused_bf16_d5(const Problem& P, bool sync_ready, hipStream_t s);
 int launch_fused_bf16_d8(const Problem& P, bool sync_ready, hipStream_t s);
 
-constexpr uint64_t kSyncAreaBytes = 4 * (16 + (16 + 2 * 64) * 1024);  // header + one sector per multi-workgroup team
+constexpr uint64_t kSyncAreaBytes = 4 * (16 + (16 + 3 * 64) * 1024);  // header + one sector per multi-workgroup team
 // Zero-fills the sync area of a workspace (a small fill kernel, graph-capture safe).
 int launch_zero_sync(unsigned* sync, hipStream_t s);
 

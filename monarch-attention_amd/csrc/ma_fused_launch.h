@@ -2,7 +2,6 @@
 // .hip file per (dtype, head-dim class) so the instantiations compile in parallel.
 #pragma once
 
-#include <cstdlib>
 #include <type_traits>
 
 #include "ma_fused.h"
@@ -17,20 +16,19 @@ namespace mfma {
 inline FusedPlan plan_teams(long long heads, int tasks_r, int tasks_l, int capacity) {
     FusedPlan pl;
     const int widest = tasks_r > tasks_l ? tasks_r : tasks_l;
-    long long limit = capacity / heads;
+    const long long pairs = (heads + 1) / 2;  // a team keeps two heads in flight
+    long long limit = capacity / pairs;
     if (limit < 1) limit = 1;
     if (limit > widest) limit = widest;
     if (limit > kMaxTeamSize) limit = kMaxTeamSize;
     const int per_wg = static_cast<int>((widest + limit - 1) / limit);
     pl.G = (widest + per_wg - 1) / per_wg;
     long long nteams = capacity / pl.G;
-    if (nteams > heads) nteams = heads;
+    if (nteams > pairs) nteams = pairs;
     if (nteams > 8) nteams -= nteams % 8;  // whole teams per XCD
     pl.nteams = static_cast<int>(nteams);
     pl.xcd_map = (pl.nteams % 8 == 0) ? 1 : 0;
     pl.spin_limit = 1u << 22;
-    const char* dbg = getenv("MA_FUSED_DEBUG");
-    pl.debug = dbg ? atoi(dbg) : 0;
     return pl;
 }
 

@@ -97,6 +97,29 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
     return x;
 }
 
+// ---- global memory through buffer resources ---------------------------------
+// Every tensor slice a block problem touches is addressed as (uniform base in
+// SGPRs) + (32-bit byte offset per lane).  Rows that do not exist (padding,
+// masked-out tails, tile tails) get the offset kOob, which the hardware bounds
+// check turns into a load of zeros / a dropped store - no branches.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr unsigned kOob = 0xFFFF0000u;  // beyond any slice (extents are validated to stay below it)
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+// SHARED = true is for state another workgroup wrote during this launch: a
+// streaming ("nt") load, which is served by L2 and never by a line this CU's L1
+// kept from an earlier step.
+template <bool SHARED>
+__device__ __forceinline__ u32x4 bload16(rsrc_t r, unsigned off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, SHARED ? 2 : 0);
+}
+template <bool SHARED>
+__device__ __forceinline__ float bloadf(rsrc_t r, unsigned off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, SHARED ? 2 : 0));
+}
+
 // ---- operand tiles ----------------------------------------------------------
 // LDS tile geometry for a head dim that needs DT 16-wide output tiles:
 // KS 32-wide k steps, row pitch LD elements (the +8 staggers rows over banks).
@@ -107,45 +130,37 @@ struct Geom {
     static constexpr int LD = COLS + 8;
 };
 
-// Cooperative global -> LDS copy of `rows` rows (zero rows where rowptr gives
-// nullptr, zero columns beyond D).  tix / nth: this thread's index and the
-// number of threads that share the copy.
-// 16-byte global load.  SHARED = true is for state another workgroup wrote during
-// this launch: a streaming ("nt") load, which is served by L2 and never by a
-// line this CU's L1 kept from an earlier step.
-template <bool SHARED>
-__device__ __forceinline__ u32x4 ld16(const void* p) {
-    if (SHARED) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-    return *reinterpret_cast<const u32x4*>(p);
-}
-template <bool SHARED>
-__device__ __forceinline__ float ldf(const float* p) {
-    if (SHARED) return __builtin_nontemporal_load(p);
-    return *p;
-}
-
-template <class T, int DT, bool SHARED, class RowPtr>
-__device__ __forceinline__ void load_tile(T* tile, int rows, int D, RowPtr rowptr, int tix, int nth) {
+// Cooperative global -> LDS copy of ROWS rows of 16-byte chunks by NTH threads.
+// rowoff(row) gives the row's byte offset in the resource or kOob; columns at or
+// beyond D are zero-filled.  All loads are issued before the first LDS write.
+template <class T, int DT, int ROWS, int NTH, bool SHARED, class RowOff>
+__device__ __forceinline__ void load_tile(T* tile, rsrc_t src, int D, RowOff rowoff, int tix) {
     constexpr int CH = Geom<DT>::COLS / 8;
     constexpr int LD = Geom<DT>::LD;
-    for (int c = tix; c < rows * CH; c += nth) {
+    constexpr int CNT = ROWS * CH / NTH;
+    static_assert(ROWS * CH % NTH == 0, "tile chunks must divide evenly among the threads");
+    u32x4 val[CNT];
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+        const int c = tix + i * NTH;
         const int row = c / CH, ch = c % CH;
-        u32x4 val = {0u, 0u, 0u, 0u};
-        const T* p = rowptr(row);
-        if (p != nullptr && ch * 8 < D) val = ld16<SHARED>(p + ch * 8);
-        *reinterpret_cast<u32x4*>(tile + row * LD + ch * 8) = val;
+        const unsigned ro = rowoff(row);
+        val[i] = bload16<SHARED>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
+    }
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+        const int c = tix + i * NTH;
+        *reinterpret_cast<u32x4*>(tile + (c / CH) * LD + (c % CH) * 8) = val[i];
     }
 }
 
-// B operand of GEMM1 straight from HBM: row `p` (or zeros), k step ks.
+// B operand of GEMM1 straight from memory: the row at byte offset ro (or kOob)
 template <class T, int DT, bool SHARED>
-__device__ __forceinline__ void load_x(typename Ops<T>::v8 (&x)[Geom<DT>::KS], const T* p, int D, int q) {
+__device__ __forceinline__ void load_x(typename Ops<T>::v8 (&x)[Geom<DT>::KS], rsrc_t src, unsigned ro, int D, int q) {
 #pragma unroll
     for (int ks = 0; ks < Geom<DT>::KS; ++ks) {
         const int col = 32 * ks + 8 * q;
-        u32x4 val = {0u, 0u, 0u, 0u};
-        if (p != nullptr && col < D) val = ld16<SHARED>(p + col);
-        x[ks] = __builtin_bit_cast(typename Ops<T>::v8, val);
+        x[ks] = __builtin_bit_cast(typename Ops<T>::v8, bload16<SHARED>(src, col < D ? ro + col * 2 : kOob));
     }
 }
 
@@ -154,36 +169,28 @@ __device__ __forceinline__ typename Ops<T>::v8 lds_row8(const T* tile_elem) {
     return __builtin_bit_cast(typename Ops<T>::v8, *reinterpret_cast<const u32x4*>(tile_elem));
 }
 
-// Transposed A operand for k step g of GEMM2 from a row-major LDS tile:
-// returns tile[32g + 16(s/4) + 4q + s%4][col0 + r] for s = 0..7.
-template <class T, int NWT>
-__device__ __forceinline__ typename Ops<T>::v8 lds_tr8(const T* tile, int ld, int g, int col0, int r, int q) {
+// Transposed A operand of GEMM2 from a row-major LDS tile via ds_read_b64_tr_b16.
+// Output tile dt, lane (r, q) = MFMA row r: the row is mapped to the tile column
+// d = 4*DT*(r/4) + 4*dt + r%4, so that after all DT tiles a lane of the C layout
+// (rows 4q..4q+3) owns the 4*DT CONSECUTIVE columns 4*DT*q .. 4*DT*(q+1)-1 and
+// can store them as one contiguous run.  row0 is the tile row of k slot 0,
+// hi_rows the distance to the row of k slot 4.
+template <class T, int DT>
+__device__ __forceinline__ typename Ops<T>::v8 lds_tr8(const T* tile, int row0, int hi_rows, bool with_hi, int dt, int r) {
     typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
+    constexpr int LD = Geom<DT>::LD;
     const int e = r >> 2, c = r & 3;
-    const T* p0 = tile + (32 * g + 4 * q + e) * ld + col0 + 4 * c;
+    const T* p0 = tile + (row0 + e) * LD + 4 * DT * c + 4 * dt;
     i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
     i16x4 hi = {0, 0, 0, 0};
-    if (2 * g + 1 < NWT) hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 16 * ld));
+    if (with_hi) hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + hi_rows * LD));
     typedef short i16x8 __attribute__((ext_vector_type(8)));
     i16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     return __builtin_bit_cast(typename Ops<T>::v8, v);
 }
 
-// Natural-order transposed A operand (k slot s <-> row 32g + 8q + s), used by
-// the L step whose B operand is read back from LDS in natural order.
-template <class T>
-__device__ __forceinline__ typename Ops<T>::v8 lds_tr8_natural(const T* tile, int ld, int g, int col0, int r, int q) {
-    typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
-    const int e = r >> 2, c = r & 3;
-    const T* p0 = tile + (32 * g + 8 * q + e) * ld + col0 + 4 * c;
-    i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
-    i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 4 * ld));
-    typedef short i16x8 __attribute__((ext_vector_type(8)));
-    i16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    return __builtin_bit_cast(typename Ops<T>::v8, v);
-}
-
-// P (fp32, C layout, NWT tiles) -> B operands of GEMM2, rounded to T.
+// P (fp32, C layout, NWT tiles) -> B operands of GEMM2, rounded to T.  k slot s of
+// step g is row w = 32g + 16(s/4) + 4q + s%4: slots 0-3 from C tile 2g, 4-7 from 2g+1.
 template <class T, int NWT>
 __device__ __forceinline__ void pack_p(typename Ops<T>::v8 (&pb)[(NWT + 1) / 2], const f32x4 (&C)[NWT]) {
 #pragma unroll
@@ -198,32 +205,44 @@ __device__ __forceinline__ void pack_p(typename Ops<T>::v8 (&pb)[(NWT + 1) / 2],
     }
 }
 
-// GEMM2: O[dt][v] = sum_w tile[w][16dt + 4q + v] * P[w][x = lane column]
+// GEMM2: O[dt][v] = sum_w tile[w][4*DT*q + 4*dt + v] * P[w][x = lane column]
 template <class T, int DT, int NWT>
 __device__ __forceinline__ void gemm2(f32x4 (&O)[DT], const T* tile, const typename Ops<T>::v8 (&pb)[(NWT + 1) / 2],
                                       int r, int q) {
-    constexpr int LD = Geom<DT>::LD;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int g = 0; g < (NWT + 1) / 2; ++g) acc = Ops<T>::mma(lds_tr8<T, NWT>(tile, LD, g, 16 * dt, r, q), pb[g], acc);
+        for (int g = 0; g < (NWT + 1) / 2; ++g)
+            acc = Ops<T>::mma(lds_tr8<T, DT>(tile, 32 * g + 4 * q, 16, 2 * g + 1 < NWT, dt, r), pb[g], acc);
         O[dt] = acc;
     }
 }
 
-// 4 consecutive output elements (d = 16dt + 4q .. +3) of one row, 8-byte store
-template <class T>
-__device__ __forceinline__ void store4(T* row, int d0, int D, f32x4 v) {
-    if (row == nullptr || d0 >= D) return;  // D is a multiple of 8, d0 of 4
-    typename Ops<T>::v4 o = {from_f<T>(v[0]), from_f<T>(v[1]), from_f<T>(v[2]), from_f<T>(v[3])};
-    *reinterpret_cast<u32x2*>(row + d0) = __builtin_bit_cast(u32x2, o);
-}
-
-template <class T>
-__device__ __forceinline__ const T* token_row(const char* base, const long long* st, int e, int h, int t, int N) {
-    if (t < 0 || t >= N) return nullptr;
-    return reinterpret_cast<const T*>(base) + e * st[0] + h * st[1] + static_cast<long long>(t) * st[2];
+// Store a lane's 4*DT consecutive output elements (columns 4*DT*q ..) of the row at
+// byte offset ro (kOob drops the store): 16-byte pieces when the head dim fills the
+// tiles exactly, else 8-byte pieces so that a piece never straddles D.
+template <class T, int DT>
+__device__ __forceinline__ void store_row(rsrc_t dst, unsigned ro, int D, const f32x4 (&O)[DT], int q) {
+    typedef typename Ops<T>::v4 V4;
+    const unsigned base = ro + 8 * DT * q;  // bytes
+    if (DT % 2 == 0 && D == 16 * DT) {
+#pragma unroll
+        for (int p = 0; p < DT / 2; ++p) {
+            V4 a = {from_f<T>(O[2 * p][0]), from_f<T>(O[2 * p][1]), from_f<T>(O[2 * p][2]), from_f<T>(O[2 * p][3])};
+            V4 b = {from_f<T>(O[2 * p + 1][0]), from_f<T>(O[2 * p + 1][1]), from_f<T>(O[2 * p + 1][2]), from_f<T>(O[2 * p + 1][3])};
+            const u32x2 lo = __builtin_bit_cast(u32x2, a), hi = __builtin_bit_cast(u32x2, b);
+            const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+            __builtin_amdgcn_raw_buffer_store_b128(v, dst, base + 16 * p, 0, 0);
+        }
+    } else {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            V4 a = {from_f<T>(O[dt][0]), from_f<T>(O[dt][1]), from_f<T>(O[dt][2]), from_f<T>(O[dt][3])};
+            const int d0 = 4 * DT * q + 4 * dt;
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, a), dst, d0 < D ? base + 8 * dt : kOob, 0, 0);
+        }
+    }
 }
 
 // How a workgroup's four waves are shared among block problems with NT strips:
@@ -248,6 +267,39 @@ struct Lds {
     static constexpr size_t L = (TILE2 + TILE + ROWS * LDP) * sizeof(T) + (1 + Split<NWT>::WPP) * ROWS * sizeof(float);
 };
 
+// Uniform (per problem) description of the tensors: resources and row pitches in bytes.
+struct Slices {
+    rsrc_t q, k, v, out, aR, cR, aL, cL, Y;
+    unsigned qst, kst, vst, ost;
+};
+
+template <class T>
+__device__ __forceinline__ Slices make_slices(const Problem& P, int e, int h, long long wh) {
+    Slices S;
+    const unsigned n1 = static_cast<unsigned>(P.N - 1), db = static_cast<unsigned>(P.D) * sizeof(T);
+    S.qst = static_cast<unsigned>(P.qs[2]) * sizeof(T);
+    S.kst = static_cast<unsigned>(P.ks[2]) * sizeof(T);
+    S.vst = static_cast<unsigned>(P.vs[2]) * sizeof(T);
+    S.ost = static_cast<unsigned>(P.os[2]) * sizeof(T);
+    S.q = make_rsrc(P.q + (e * P.qs[0] + h * P.qs[1]) * static_cast<long long>(sizeof(T)), n1 * S.qst + db);
+    S.k = make_rsrc(P.k + (e * P.ks[0] + h * P.ks[1]) * static_cast<long long>(sizeof(T)), n1 * S.kst + db);
+    S.v = make_rsrc(P.v + (e * P.vs[0] + h * P.vs[1]) * static_cast<long long>(sizeof(T)), n1 * S.vst + db);
+    S.out = make_rsrc(P.out + (e * P.os[0] + h * P.os[1]) * static_cast<long long>(sizeof(T)), n1 * S.ost + db);
+    const long long np = static_cast<long long>(P.M) * P.B;
+    const unsigned state = static_cast<unsigned>(np) * db, stat4 = static_cast<unsigned>(np) * 4u;
+    S.aR = make_rsrc(P.aR + wh * np * db, state);
+    S.aL = make_rsrc(P.aL + wh * np * db, state);
+    S.Y = make_rsrc(P.Y + wh * np * db, state);
+    S.cR = make_rsrc(P.cR + wh * np, stat4);
+    S.cL = make_rsrc(P.cL + wh * np, stat4);
+    return S;
+}
+
+// byte offset of real token t's row (pitch st) or kOob for a padding position
+__device__ __forceinline__ unsigned tok_off(int t, int N, unsigned st) {
+    return static_cast<unsigned>(t) < static_cast<unsigned>(N) ? static_cast<unsigned>(t) * st : kOob;
+}
+
 // ============================================================================
 // R step for one block problem (e,h,m), run by WPP waves (wig = wave in group).
 // smem: K tile, V tile, key bias.   Reference: al_cl_ref / al_y_cl_ref
@@ -265,26 +317,31 @@ __device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool act
     float* kbias = reinterpret_cast<float*>(Vt + Lds<T, DT, NWT>::TILE);
     const int B = P.B, M = P.M, D = P.D;
     const int r = lane & 15, q = lane >> 4;
-    const int tix = wig * 64 + lane, nth = WPP * 64;
-    const long long eh = wh;  // workspace slot: (e,h) itself in the staged kernels, the team's slot in the fused one
+    const int tix = wig * 64 + lane;
+    const unsigned db = static_cast<unsigned>(D) * sizeof(T);
+    const Slices S = make_slices<T>(P, e, h, wh);
 
     if (active) {
-        load_tile<T, DT, false>(Kt, ROWS, D, [&](int i) { return i < B ? token_row<T>(P.k, P.ks, e, h, m * B + i - P.pad_off, P.N) : nullptr; }, tix, nth);
+        const int t0 = m * B - P.pad_off;
+        load_tile<T, DT, ROWS, WPP * 64, true>(Kt, S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
         if (with_v)
-            load_tile<T, DT, false>(Vt, ROWS, D, [&](int i) { return i < B ? token_row<T>(P.v, P.vs, e, h, m * B + i - P.pad_off, P.N) : nullptr; }, tix, nth);
-        for (int i = tix; i < ROWS; i += nth) kbias[i] = (i < B && token_ok(P, e, m * B + i - P.pad_off)) ? 0.f : kNegBig;
+            load_tile<T, DT, ROWS, WPP * 64, true>(Vt, S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix);
+        for (int i = tix; i < ROWS; i += WPP * 64) kbias[i] = (i < B && token_ok(P, e, t0 + i)) ? 0.f : kNegBig;
     }
     __syncthreads();
     if (active) {
         for (int strip = wig; strip < NWT; strip += WPP) {
             const int j = 16 * strip + r;
             const bool jv = j < B;
-            const long long rowid = (eh * M + m) * B + j;
-            const T* xrow = nullptr;
-            if (jv) xrow = first ? token_row<T>(P.q, P.qs, e, h, m * B + j - P.pad_off, P.N) : reinterpret_cast<const T*>(P.aR) + rowid * D;
+            const unsigned rowid = static_cast<unsigned>(m * B + j);   // row inside the head's state
             V8 xb[G::KS];
-            if (first) load_x<T, DT, false>(xb, xrow, D, q); else load_x<T, DT, true>(xb, xrow, D, q);
-            const float cr = (first || !jv) ? 1.0f : ldf<true>(P.cR + rowid);
+            float cr = 1.0f;
+            if (first) {
+                load_x<T, DT, false>(xb, S.q, jv ? tok_off(m * B + j - P.pad_off, P.N, S.qst) : kOob, D, q);
+            } else {
+                load_x<T, DT, true>(xb, S.aR, jv ? rowid * db : kOob, D, q);
+                cr = bloadf<true>(S.cR, jv ? rowid * 4u : kOob);   // an out-of-range row reads 0: harmless, never stored
+            }
             const float cj = (P.sm_scale * kLog2e) / (cr + P.eps);  // logits in log2 units
 
             f32x4 C[NWT];
@@ -325,27 +382,26 @@ __device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool act
 #pragma unroll
                 for (int v = 0; v < 4; ++v) C[wt][v] *= inv;
             // cL = sum_i r log r with r = p / den (ma_torch.py:20); rows of tiny r add ~1e-36
-            if (jv && q == 0) P.cL[(eh * B + j) * M + m] = kLn2 * ent * inv - logf(den) * (sum * inv);
+            const unsigned lrow = static_cast<unsigned>(j * M + m);   // row of aL / cL / Y: (j, m)
+            if (q == 0)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, kLn2 * ent * inv - __logf(den) * (sum * inv)),
+                                                      S.cL, jv ? lrow * 4u : kOob, 0, 0);
 
             V8 pb[(NWT + 1) / 2];
             pack_p<T, NWT>(pb, C);
-            T* arow = jv ? reinterpret_cast<T*>(P.aL) + ((eh * B + j) * M + m) * D : nullptr;
             {
                 f32x4 O[DT];
                 gemm2<T, DT, NWT>(O, Kt, pb, r, q);
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
+                for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                     for (int v = 0; v < 4; ++v) O[dt][v] = P.sm_scale * round_to<T>(O[dt][v]);
-                    store4<T>(arow, 16 * dt + 4 * q, D, O[dt]);
-                }
+                store_row<T, DT>(S.aL, jv ? lrow * db : kOob, D, O, q);
             }
             if (with_v) {
-                T* yrow = jv ? reinterpret_cast<T*>(P.Y) + ((eh * B + j) * M + m) * D : nullptr;
                 f32x4 O[DT];
                 gemm2<T, DT, NWT>(O, Vt, pb, r, q);
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) store4<T>(yrow, 16 * dt + 4 * q, D, O[dt]);
+                store_row<T, DT>(S.Y, jv ? lrow * db : kOob, D, O, q);
             }
         }
     }
@@ -367,25 +423,24 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
     float* cb = reinterpret_cast<float*>(Yt + Lds<T, DT, NWT>::TILE);
     const int B = P.B, M = P.M, D = P.D;
     const int r = lane & 15, q = lane >> 4;
-    const int tix = wig * 64 + lane, nth = WPP * 64;
-    const long long eh = wh;  // workspace slot: (e,h) itself in the staged kernels, the team's slot in the fused one
+    const int tix = wig * 64 + lane;
+    const unsigned db = static_cast<unsigned>(D) * sizeof(T);
+    const Slices S = make_slices<T>(P, e, h, wh);
 
     if (active) {
-        const T* aL = reinterpret_cast<const T*>(P.aL) + (eh * B + j) * M * D;
-        const T* Y = reinterpret_cast<const T*>(P.Y) + (eh * B + j) * M * D;
-        load_tile<T, DT, true>(At, ROWS, D, [&](int k) { return k < M ? aL + k * D : nullptr; }, tix, nth);
-        load_tile<T, DT, true>(Yt, ROWS, D, [&](int k) { return k < M ? Y + k * D : nullptr; }, tix, nth);
-        const float* cL = P.cL + (eh * B + j) * M;
-        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * ldf<true>(cL + k) : kNegBig;
+        const unsigned row0 = static_cast<unsigned>(j * M);
+        load_tile<T, DT, ROWS, WPP * 64, true>(At, S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        load_tile<T, DT, ROWS, WPP * 64, true>(Yt, S.Y, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        for (int k = tix; k < ROWS; k += WPP * 64) cb[k] = k < M ? -kLog2e * bloadf<true>(S.cL, (row0 + k) * 4u) : kNegBig;
     }
     __syncthreads();
     if (active) {
         for (int strip = wig; strip < NWT; strip += WPP) {
             const int l = 16 * strip + r;
             const int t = l * B + j - P.pad_off;
-            const bool lv = l < M && t >= 0 && t < P.N;
+            const bool lv = l < M;
             V8 xb[G::KS];
-            load_x<T, DT, false>(xb, lv ? token_row<T>(P.q, P.qs, e, h, t, P.N) : nullptr, D, q);
+            load_x<T, DT, false>(xb, S.q, lv ? tok_off(t, P.N, S.qst) : kOob, D, q);
             f32x4 C[NWT];
 #pragma unroll
             for (int wt = 0; wt < NWT; ++wt) {
@@ -421,9 +476,7 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
             pack_p<T, NWT>(pb, C);
             f32x4 O[DT];
             gemm2<T, DT, NWT>(O, Yt, pb, r, q);
-            T* orow = lv ? reinterpret_cast<T*>(P.out) + e * P.os[0] + h * P.os[1] + static_cast<long long>(t) * P.os[2] : nullptr;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) store4<T>(orow, 16 * dt + 4 * q, D, O[dt]);
+            store_row<T, DT>(S.out, lv ? tok_off(t, P.N, S.ost) : kOob, D, O, q);   // padded query rows are dropped (:108)
         }
     }
 }
@@ -448,15 +501,16 @@ __device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool act
     float* crp = cb + ROWS;  // [WPP][ROWS]
     const int B = P.B, M = P.M, D = P.D;
     const int r = lane & 15, q = lane >> 4;
-    const int tix = wig * 64 + lane, nth = WPP * 64;
-    const long long eh = wh;  // workspace slot: (e,h) itself in the staged kernels, the team's slot in the fused one
+    const int tix = wig * 64 + lane;
+    constexpr int nth = WPP * 64;
+    const unsigned db = static_cast<unsigned>(D) * sizeof(T);
+    const Slices S = make_slices<T>(P, e, h, wh);
 
     if (active) {
-        const T* aL = reinterpret_cast<const T*>(P.aL) + (eh * B + j) * M * D;
-        load_tile<T, DT, false>(Qt, ROWS2, D, [&](int l) { return l < M ? token_row<T>(P.q, P.qs, e, h, l * B + j - P.pad_off, P.N) : nullptr; }, tix, nth);
-        load_tile<T, DT, true>(At, ROWS, D, [&](int k) { return k < M ? aL + k * D : nullptr; }, tix, nth);
-        const float* cL = P.cL + (eh * B + j) * M;
-        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * ldf<true>(cL + k) : kNegBig;
+        const unsigned row0 = static_cast<unsigned>(j * M);
+        load_tile<T, DT, ROWS2, nth, false>(Qt, S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
+        load_tile<T, DT, ROWS, nth, true>(At, S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * bloadf<true>(S.cL, (row0 + k) * 4u) : kNegBig;
         if (ROWS2 > ROWS)  // zero the phantom l columns of PT that phase 2 reads
             for (int i = tix; i < ROWS * (ROWS2 - ROWS); i += nth) PT[(i / (ROWS2 - ROWS)) * LDP + ROWS + i % (ROWS2 - ROWS)] = from_f<T>(0.f);
     }
@@ -536,19 +590,22 @@ __device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool act
             V8 pb[NG];
 #pragma unroll
             for (int g = 0; g < NG; ++g) pb[g] = lds_row8<T>(PT + k * LDP + 32 * g + 8 * q);
-            T* arow = kv ? reinterpret_cast<T*>(P.aR) + ((eh * M + k) * B + j) * D : nullptr;
+            f32x4 O[DT];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int g = 0; g < NG; ++g) acc = Ops<T>::mma(lds_tr8_natural<T>(Qt, G::LD, g, 16 * dt, r, q), pb[g], acc);
-                store4<T>(arow, 16 * dt + 4 * q, D, acc);
+                for (int g = 0; g < NG; ++g)   // natural k-slot order here: slot s <-> row 32g + 8q + s
+                    acc = Ops<T>::mma(lds_tr8<T, DT>(Qt, 32 * g + 8 * q, 4, true, dt, r), pb[g], acc);
+                O[dt] = acc;
             }
-            if (kv && q == 0) {
+            const unsigned arow = static_cast<unsigned>(k * B + j);   // row of aR / cR: (k, j)
+            store_row<T, DT>(S.aR, kv ? arow * db : kOob, D, O, q);
+            if (q == 0) {
                 float s = 0.f;
 #pragma unroll
                 for (int w = 0; w < WPP; ++w) s += crp[w * ROWS + k];
-                P.cR[(eh * M + k) * B + j] = s;
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, s), S.cR, kv ? arow * 4u : kOob, 0, 0);
             }
         }
     }
