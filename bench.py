@@ -43,6 +43,15 @@ CONFIGS = {  # name: (E, H, N, D, B, T, dtype, scale)  - BASELINE.json configs +
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
 
+# HBM-side bytes per launch of the dominant kernels on the metric workload, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for a plain
+# 256 MiB device copy (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); see profiles/traffic_cM_T1.md.
+MEASURED_TRAFFIC_BYTES = {
+    ("cM", 1, "r_step(with V)"): 44_188_000,
+    ("cM", 1, "z_step"): 33_935_000,
+    ("cM", 1, "fused_fwd_mfma"): 72_430_000,
+}
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -161,7 +170,7 @@ def main():
     dom_ms, dom_bytes = kernels[dom]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, T, dom)),
                 "algorithmic_bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_ms * 1e3, 2),
                 "kernels_us": {kname: round(v[0] * 1e3, 2) for kname, v in kernels.items()}}
 

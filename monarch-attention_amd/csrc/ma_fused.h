@@ -45,11 +45,11 @@ constexpr int kMaxTeams = 1024;    // teams of more than one workgroup
 constexpr int kSyncWords = kSyncHeader + kSyncStride * kMaxTeams;
 static_assert(static_cast<uint64_t>(kSyncWords) * 4 == kSyncAreaBytes, "sync area size mismatch");
 
-template <class T, int DT, int NTB, int NTM>
+template <class T, int DT, int NTB, int NTM, int W>
 struct FusedLds {
-    static constexpr size_t r = Split<NTB>::PPW * Lds<T, DT, NTB>::R;
-    static constexpr size_t l = Split<NTM>::PPW * Lds<T, DT, NTM>::L;
-    static constexpr size_t z = Split<NTM>::PPW * Lds<T, DT, NTM>::Z;
+    static constexpr size_t r = Split<NTB, W>::PPW * Lds<T, DT, NTB>::R;
+    static constexpr size_t l = Split<NTM, W>::PPW * Lds<T, DT, NTM>::L;
+    static constexpr size_t z = Split<NTM, W>::PPW * Lds<T, DT, NTM>::Z;
     static constexpr size_t bytes = r > l ? (r > z ? r : z) : (l > z ? l : z);
 };
 
@@ -157,13 +157,13 @@ __device__ __forceinline__ void team_wait(TeamSync& ts, int slot) {
 
 // One phase of one head: p even = R step (p = 0 reads Q, the last one forms Y),
 // p odd = L step, p = 2T-1 = Z step.
-template <class T, int DT, int NTB, int NTM>
+template <class T, int DT, int NTB, int NTM, int W>
 __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, long long head, long long slot_ws, int member,
                                           int G, int wave, int lane) {
     const int e = head / P.H, h = head % P.H;
     const int nph = 2 * P.T;
     if (p == nph - 1) {
-        constexpr int WPP = Split<NTM>::WPP, PPW = Split<NTM>::PPW;
+        constexpr int WPP = Split<NTM, W>::WPP, PPW = Split<NTM, W>::PPW;
         const int slot = wave / WPP, wig = wave % WPP;
         const int tasks = (P.B + PPW - 1) / PPW;
         for (int task = member; task < tasks; task += G) {
@@ -173,7 +173,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, l
             __syncthreads();  // the LDS tiles are reused by the next task
         }
     } else if (p & 1) {
-        constexpr int WPP = Split<NTM>::WPP, PPW = Split<NTM>::PPW;
+        constexpr int WPP = Split<NTM, W>::WPP, PPW = Split<NTM, W>::PPW;
         const int slot = wave / WPP, wig = wave % WPP;
         const int tasks = (P.B + PPW - 1) / PPW;
         for (int task = member; task < tasks; task += G) {
@@ -183,7 +183,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, l
             __syncthreads();
         }
     } else {
-        constexpr int WPP = Split<NTB>::WPP, PPW = Split<NTB>::PPW;
+        constexpr int WPP = Split<NTB, W>::WPP, PPW = Split<NTB, W>::PPW;
         const int slot = wave / WPP, wig = wave % WPP;
         const int tasks = (P.M + PPW - 1) / PPW;
         for (int task = member; task < tasks; task += G) {
@@ -196,8 +196,8 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, l
     }
 }
 
-template <class T, int DT, int NTB, int NTM>
-__global__ __launch_bounds__(kThreads) void fused_fwd_mfma(Problem P, FusedPlan plan) {
+template <class T, int DT, int NTB, int NTM, int W>
+__global__ __launch_bounds__(64 * W) void fused_fwd_mfma(Problem P, FusedPlan plan) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int G = plan.G;
@@ -231,21 +231,24 @@ __global__ __launch_bounds__(kThreads) void fused_fwd_mfma(Problem P, FusedPlan 
     const long long heads = static_cast<long long>(P.E) * P.H;
     const int nph = 2 * P.T;
 
-    // heads of this team: team, team + nteams, ...; consecutive ones are paired on slots 0 / 1
-    for (long long hA = team; hA < heads; hA += 2ll * plan.nteams) {
+    // heads of this team: team, team + nteams, ...; a multi-workgroup team pairs consecutive
+    // ones on slots 0 / 1, a single workgroup (nothing to wait for) takes them one by one
+    const long long stride = (G > 1 ? 2ll : 1ll) * plan.nteams;
+    const long long ws_a = G > 1 ? 2ll * team : team, ws_b = ws_a + 1;  // state slots in the workspace
+    for (long long hA = team; hA < heads; hA += stride) {
         const long long hB = hA + plan.nteams;
-        const bool has_b = hB < heads;
+        const bool has_b = G > 1 && hB < heads;
         const bool first_pair = hA == team;
-        const bool more_a = hA + 2ll * plan.nteams < heads, more_b = hB + 2ll * plan.nteams < heads;
+        const bool more_a = hA + stride < heads, more_b = hB + stride < heads;
         for (int p = 0; p < nph; ++p) {
             // a phase may start once every member has finished the previous phase on the same slot
             // (it reads what they wrote, or overwrites what they were reading)
             if (!(first_pair && p == 0)) team_wait(ts, 0);
-            run_phase<T, DT, NTB, NTM>(P, smem, p, hA, 2ll * team, member, G, wave, lane);
+            run_phase<T, DT, NTB, NTM, W>(P, smem, p, hA, ws_a, member, G, wave, lane);
             if (p < nph - 1 || more_a) team_arrive(ts, 0);
             if (has_b) {
                 if (!(first_pair && p == 0)) team_wait(ts, 1);
-                run_phase<T, DT, NTB, NTM>(P, smem, p, hB, 2ll * team + 1, member, G, wave, lane);
+                run_phase<T, DT, NTB, NTM, W>(P, smem, p, hB, ws_b, member, G, wave, lane);
                 if (p < nph - 1 || more_b) team_arrive(ts, 1);
             }
         }

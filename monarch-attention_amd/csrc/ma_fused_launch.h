@@ -2,6 +2,7 @@
 // .hip file per (dtype, head-dim class) so the instantiations compile in parallel.
 #pragma once
 
+#include <cstdlib>
 #include <type_traits>
 
 #include "ma_fused.h"
@@ -24,7 +25,8 @@ inline FusedPlan plan_teams(long long heads, int tasks_r, int tasks_l, int capac
     const int per_wg = static_cast<int>((widest + limit - 1) / limit);
     pl.G = (widest + per_wg - 1) / per_wg;
     long long nteams = capacity / pl.G;
-    if (nteams > pairs) nteams = pairs;
+    const long long most = pl.G > 1 ? pairs : heads;  // one-workgroup teams take their heads one at a time
+    if (nteams > most) nteams = most;
     if (nteams > 8) nteams -= nteams % 8;  // whole teams per XCD
     pl.nteams = static_cast<int>(nteams);
     pl.xcd_map = (pl.nteams % 8 == 0) ? 1 : 0;
@@ -32,10 +34,11 @@ inline FusedPlan plan_teams(long long heads, int tasks_r, int tasks_l, int capac
     return pl;
 }
 
-template <class T, int DT, int NTB, int NTM>
-int launch_fused_one(const Problem& P, bool sync_ready, hipStream_t s) {
-    using FL = FusedLds<T, DT, NTB, NTM>;
-    auto kernel = fused_fwd_mfma<T, DT, NTB, NTM>;
+template <class T, int DT, int NTB, int NTM, int W>
+int launch_fused_w(const Problem& P, bool sync_ready, hipStream_t s) {
+    using FL = FusedLds<T, DT, NTB, NTM, W>;
+    if (FL::bytes > 160 * 1024) return MA_ERR_UNSUPPORTED;
+    auto kernel = fused_fwd_mfma<T, DT, NTB, NTM, W>;
     struct Caps {
         int err = 0, capacity = 0;
     };
@@ -46,23 +49,38 @@ int launch_fused_one(const Problem& P, bool sync_ready, hipStream_t s) {
         if (!c.err) c.err = static_cast<int>(hipGetDevice(&dev));
         if (!c.err) c.err = static_cast<int>(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
         if (!c.err)
-            c.err = static_cast<int>(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), kThreads, FL::bytes));
+            c.err = static_cast<int>(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), 64 * W, FL::bytes));
         c.capacity = cus * per_cu;
         return c;
     }();
     if (caps.err) return caps.err;
     if (caps.capacity < 1) return MA_ERR_UNSUPPORTED;
     const long long heads = static_cast<long long>(P.E) * P.H;
-    const int tasks_r = (P.M + Split<NTB>::PPW - 1) / Split<NTB>::PPW;
-    const int tasks_l = (P.B + Split<NTM>::PPW - 1) / Split<NTM>::PPW;
+    const int tasks_r = (P.M + Split<NTB, W>::PPW - 1) / Split<NTB, W>::PPW;
+    const int tasks_l = (P.B + Split<NTM, W>::PPW - 1) / Split<NTM, W>::PPW;
     const FusedPlan pl = plan_teams(heads, tasks_r, tasks_l, caps.capacity);
+    {   // the workspace holds one state slot per head: the slots the grid will touch must exist
+        const long long last = pl.nteams - 1;
+        const long long max_slot = pl.G > 1 ? 2 * last + ((last + pl.nteams < heads) ? 1 : 0) : last;
+        if (pl.nteams < 1 || pl.G < 1 || pl.G > kMaxTeamSize || max_slot >= heads) return MA_ERR_UNSUPPORTED;
+        if (pl.xcd_map && (pl.nteams % 8 != 0)) return MA_ERR_UNSUPPORTED;
+    }
     if (pl.G > 1 && pl.nteams > kMaxTeams) return MA_ERR_UNSUPPORTED;
     if (!sync_ready) {
         const int err = launch_zero_sync(P.sync, s);
         if (err) return err;
     }
-    hipLaunchKernelGGL((fused_fwd_mfma<T, DT, NTB, NTM>), dim3(pl.nteams * pl.G), dim3(kThreads), FL::bytes, s, P, pl);
+    hipLaunchKernelGGL((fused_fwd_mfma<T, DT, NTB, NTM, W>), dim3(pl.nteams * pl.G), dim3(64 * W), FL::bytes, s, P, pl);
     return static_cast<int>(hipGetLastError());
+}
+
+template <class T, int DT, int NTB, int NTM>
+int launch_fused_one(const Problem& P, bool sync_ready, hipStream_t s) {
+    int w = 4;
+    if (const char* e = getenv("MA_FUSED_WAVES")) w = atoi(e);
+    if (w == 16) return launch_fused_w<T, DT, NTB, NTM, 16>(P, sync_ready, s);
+    if (w == 8) return launch_fused_w<T, DT, NTB, NTM, 8>(P, sync_ready, s);
+    return launch_fused_w<T, DT, NTB, NTM, 4>(P, sync_ready, s);
 }
 
 template <class T, int DT>

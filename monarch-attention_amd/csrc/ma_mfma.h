@@ -130,29 +130,37 @@ struct Geom {
     static constexpr int LD = COLS + 8;
 };
 
-// Cooperative global -> LDS copy of ROWS rows of 16-byte chunks by NTH threads.
-// rowoff(row) gives the row's byte offset in the resource or kOob; columns at or
-// beyond D are zero-filled.  All loads are issued before the first LDS write.
-template <class T, int DT, int ROWS, int NTH, bool SHARED, class RowOff>
-__device__ __forceinline__ void load_tile(T* tile, rsrc_t src, int D, RowOff rowoff, int tix) {
-    constexpr int CH = Geom<DT>::COLS / 8;
-    constexpr int LD = Geom<DT>::LD;
-    constexpr int CNT = ROWS * CH / NTH;
+// Cooperative global -> LDS copy of ROWS rows of 16-byte chunks by NTH threads, in
+// two halves so that a problem can put ALL its loads in flight before it waits
+// for any of them: tile_issue starts the loads into registers, tile_commit
+// writes them to LDS.  rowoff(row) gives the row's byte offset in the resource
+// or kOob; columns at or beyond D are zero-filled.
+template <class T, int DT, int ROWS, int NTH>
+struct TileCopy {
+    static constexpr int CH = Geom<DT>::COLS / 8;
+    static constexpr int LD = Geom<DT>::LD;
+    static constexpr int CNT = ROWS * CH / NTH;
     static_assert(ROWS * CH % NTH == 0, "tile chunks must divide evenly among the threads");
     u32x4 val[CNT];
+
+    template <bool SHARED, class RowOff>
+    __device__ __forceinline__ void issue(rsrc_t src, int D, RowOff rowoff, int tix) {
 #pragma unroll
-    for (int i = 0; i < CNT; ++i) {
-        const int c = tix + i * NTH;
-        const int row = c / CH, ch = c % CH;
-        const unsigned ro = rowoff(row);
-        val[i] = bload16<SHARED>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
+        for (int i = 0; i < CNT; ++i) {
+            const int c = tix + i * NTH;
+            const int row = c / CH, ch = c % CH;
+            const unsigned ro = rowoff(row);
+            val[i] = bload16<SHARED>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
+        }
     }
+    __device__ __forceinline__ void commit(T* tile, int tix) const {
 #pragma unroll
-    for (int i = 0; i < CNT; ++i) {
-        const int c = tix + i * NTH;
-        *reinterpret_cast<u32x4*>(tile + (c / CH) * LD + (c % CH) * 8) = val[i];
+        for (int i = 0; i < CNT; ++i) {
+            const int c = tix + i * NTH;
+            *reinterpret_cast<u32x4*>(tile + (c / CH) * LD + (c % CH) * 8) = val[i];
+        }
     }
-}
+};
 
 // B operand of GEMM1 straight from memory: the row at byte offset ro (or kOob)
 template <class T, int DT, bool SHARED>
@@ -245,13 +253,13 @@ __device__ __forceinline__ void store_row(rsrc_t dst, unsigned ro, int D, const 
     }
 }
 
-// How a workgroup's four waves are shared among block problems with NT strips:
-// WPP waves per problem, PPW problems per workgroup.
-template <int NT>
+// How a workgroup's W waves are shared among block problems with NT strips:
+// WPP waves per problem (at most four), PPW problems per workgroup.
+template <int NT, int W = kWaves>
 struct Split {
     static_assert(NT == 1 || NT == 2 || NT == 4 || NT == 8, "strip counts are rounded up to a power of two");
     static constexpr int WPP = NT < kWaves ? NT : kWaves;
-    static constexpr int PPW = kWaves / WPP;
+    static constexpr int PPW = W / WPP;
 };
 
 // LDS bytes of one problem slot of each stage
@@ -321,26 +329,45 @@ __device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool act
     const unsigned db = static_cast<unsigned>(D) * sizeof(T);
     const Slices S = make_slices<T>(P, e, h, wh);
 
+    // the R problem's first strip of queries (one strip per wave unless the block has more than 64 rows)
+    auto load_strip = [&](int strip, typename Ops<T>::v8 (&xb)[G::KS], float& cr) {
+        const int j = 16 * strip + r;
+        const bool jv = j < B;
+        const unsigned rowid = static_cast<unsigned>(m * B + j);   // row inside the head's state
+        cr = 1.0f;
+        if (first) {
+            load_x<T, DT, true>(xb, S.q, jv ? tok_off(m * B + j - P.pad_off, P.N, S.qst) : kOob, D, q);
+        } else {
+            load_x<T, DT, true>(xb, S.aR, jv ? rowid * db : kOob, D, q);
+            cr = bloadf<true>(S.cR, jv ? rowid * 4u : kOob);   // an out-of-range row reads 0: harmless, never stored
+        }
+    };
+    V8 xb0[G::KS];
+    float cr0 = 1.0f;
     if (active) {
+        // every load of the problem goes out before the first wait
         const int t0 = m * B - P.pad_off;
-        load_tile<T, DT, ROWS, WPP * 64, true>(Kt, S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
-        if (with_v)
-            load_tile<T, DT, ROWS, WPP * 64, true>(Vt, S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix);
+        TileCopy<T, DT, ROWS, WPP * 64> kc, vc;
+        kc.template issue<true>(S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
+        if (with_v) vc.template issue<true>(S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix);
+        load_strip(wig, xb0, cr0);
         for (int i = tix; i < ROWS; i += WPP * 64) kbias[i] = (i < B && token_ok(P, e, t0 + i)) ? 0.f : kNegBig;
+        kc.commit(Kt, tix);
+        if (with_v) vc.commit(Vt, tix);
     }
     __syncthreads();
     if (active) {
         for (int strip = wig; strip < NWT; strip += WPP) {
             const int j = 16 * strip + r;
             const bool jv = j < B;
-            const unsigned rowid = static_cast<unsigned>(m * B + j);   // row inside the head's state
             V8 xb[G::KS];
-            float cr = 1.0f;
-            if (first) {
-                load_x<T, DT, false>(xb, S.q, jv ? tok_off(m * B + j - P.pad_off, P.N, S.qst) : kOob, D, q);
+            float cr;
+            if (strip == wig) {
+#pragma unroll
+                for (int ks = 0; ks < G::KS; ++ks) xb[ks] = xb0[ks];
+                cr = cr0;
             } else {
-                load_x<T, DT, true>(xb, S.aR, jv ? rowid * db : kOob, D, q);
-                cr = bloadf<true>(S.cR, jv ? rowid * 4u : kOob);   // an out-of-range row reads 0: harmless, never stored
+                load_strip(strip, xb, cr);
             }
             const float cj = (P.sm_scale * kLog2e) / (cr + P.eps);  // logits in log2 units
 
@@ -427,11 +454,21 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
     const unsigned db = static_cast<unsigned>(D) * sizeof(T);
     const Slices S = make_slices<T>(P, e, h, wh);
 
+    auto load_strip = [&](int strip, typename Ops<T>::v8 (&xb)[G::KS]) {
+        const int l = 16 * strip + r;
+        load_x<T, DT, true>(xb, S.q, l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob, D, q);
+    };
+    V8 xb0[G::KS];
     if (active) {
+        // every load of the problem goes out before the first wait
         const unsigned row0 = static_cast<unsigned>(j * M);
-        load_tile<T, DT, ROWS, WPP * 64, true>(At, S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
-        load_tile<T, DT, ROWS, WPP * 64, true>(Yt, S.Y, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        TileCopy<T, DT, ROWS, WPP * 64> ac, yc;
+        ac.template issue<true>(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        yc.template issue<true>(S.Y, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        load_strip(wig, xb0);
         for (int k = tix; k < ROWS; k += WPP * 64) cb[k] = k < M ? -kLog2e * bloadf<true>(S.cL, (row0 + k) * 4u) : kNegBig;
+        ac.commit(At, tix);
+        yc.commit(Yt, tix);
     }
     __syncthreads();
     if (active) {
@@ -440,7 +477,12 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
             const int t = l * B + j - P.pad_off;
             const bool lv = l < M;
             V8 xb[G::KS];
-            load_x<T, DT, false>(xb, S.q, lv ? tok_off(t, P.N, S.qst) : kOob, D, q);
+            if (strip == wig) {
+#pragma unroll
+                for (int ks = 0; ks < G::KS; ++ks) xb[ks] = xb0[ks];
+            } else {
+                load_strip(strip, xb);
+            }
             f32x4 C[NWT];
 #pragma unroll
             for (int wt = 0; wt < NWT; ++wt) {
@@ -508,9 +550,13 @@ __device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool act
 
     if (active) {
         const unsigned row0 = static_cast<unsigned>(j * M);
-        load_tile<T, DT, ROWS2, nth, false>(Qt, S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
-        load_tile<T, DT, ROWS, nth, true>(At, S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        TileCopy<T, DT, ROWS2, nth> qc;
+        TileCopy<T, DT, ROWS, nth> ac;
+        qc.template issue<true>(S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
+        ac.template issue<true>(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
         for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * bloadf<true>(S.cL, (row0 + k) * 4u) : kNegBig;
+        qc.commit(Qt, tix);
+        ac.commit(At, tix);
         if (ROWS2 > ROWS)  // zero the phantom l columns of PT that phase 2 reads
             for (int i = tix; i < ROWS * (ROWS2 - ROWS); i += nth) PT[(i / (ROWS2 - ROWS)) * LDP + ROWS + i % (ROWS2 - ROWS)] = from_f<T>(0.f);
     }

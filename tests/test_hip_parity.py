@@ -113,6 +113,8 @@ CONFIGS = [  # name, E, H, N, D, B, T, pre, dt, scale
     ("gps", 1, 2, 7600, 48, 128, 2, False, "f32", 1.0),
     ("vit_b14", 2, 12, 197, 64, 14, 2, True, "f16", 0.125),
     ("roberta_b24", 2, 12, 384, 64, 24, 1, False, "f16", 1.0),
+    ("many_heads", 40, 64, 64, 32, 16, 2, False, "f16", 1.0),      # more heads than co-resident workgroups
+    ("many_heads_odd", 3, 7, 80, 32, 16, 3, True, "bf16", 1.0),    # odd head count, ragged N
 ]
 
 
