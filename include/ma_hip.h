@@ -42,7 +42,10 @@ typedef enum ma_variant {
     MA_VARIANT_AUTO = 0,    /* fastest variant that supports the problem            */
     MA_VARIANT_GENERIC = 1, /* FMA kernels, 2T(+T-1) launches: any dtype/shape/stride */
     MA_VARIANT_STAGED = 2,  /* MFMA kernels, one launch per half step (2T launches)  */
-    MA_VARIANT_FUSED = 3    /* MFMA, all T steps in ONE launch                       */
+    MA_VARIANT_FUSED = 3,   /* MFMA, all T steps in ONE launch, teams of workgroups  */
+                            /* per head, state exchanged through the workspace       */
+    MA_VARIANT_RESIDENT = 4 /* MFMA, ONE launch, one workgroup per head with the     */
+                            /* whole per-head state resident in LDS (small heads)    */
 } ma_variant;
 
 typedef enum ma_status {
@@ -127,8 +130,8 @@ int ma_fwd_select_variant(const ma_fwd_params* p);
 int ma_fwd(const ma_fwd_params* p, void* stream);
 
 /* One stage on the state held in the workspace (stage-level parity tests;
- * variants GENERIC and STAGED; MA_ERR_UNSUPPORTED for FUSED, whose stages are
- * phases of a single kernel).
+ * variants GENERIC and STAGED; MA_ERR_UNSUPPORTED for FUSED and RESIDENT, whose
+ * stages are phases of a single kernel).
  *   ma_r_step  replaces al_cl_ref (ma/ma_torch.py:10-23) and, with with_v != 0,
  *              al_y_cl_ref (:38-52).  first != 0: take aR = Q, cR = 1 straight
  *              from q (the state before the first step, :88-89) instead of the

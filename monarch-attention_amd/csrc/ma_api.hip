@@ -22,7 +22,7 @@ int check_shape(const ma_fwd_params* p) {
     if (p == nullptr) return MA_ERR_NULL;
     if (p->E < 1 || p->H < 1 || p->N < 1 || p->D < 1 || p->Dv < 1 || p->B < 1 || p->T < 1) return MA_ERR_SHAPE;
     if (!dtype_ok(p->dtype_qk) || !dtype_ok(p->dtype_v)) return MA_ERR_DTYPE;
-    if (p->variant < MA_VARIANT_AUTO || p->variant > MA_VARIANT_FUSED) return MA_ERR_VARIANT;
+    if (p->variant < MA_VARIANT_AUTO || p->variant > MA_VARIANT_RESIDENT) return MA_ERR_VARIANT;
     if (p->flags & ~MA_FLAG_SYNC_READY) return MA_ERR_SHAPE;
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
     const long long Np = M * p->B;
@@ -128,20 +128,45 @@ bool mfma_supported(const ma_fwd_params* p) {
     return true;
 }
 
+int run_resident(const Problem& P, int dtype_qk, bool dry_run, hipStream_t s) {
+    const bool h = dtype_qk == MA_F16;
+    const int D = P.D;
+    if (D <= 32) return h ? launch_resident_f16_d2(P, dry_run, s) : launch_resident_bf16_d2(P, dry_run, s);
+    if (D <= 64) return h ? launch_resident_f16_d4(P, dry_run, s) : launch_resident_bf16_d4(P, dry_run, s);
+    if (D <= 80) return h ? launch_resident_f16_d5(P, dry_run, s) : launch_resident_bf16_d5(P, dry_run, s);
+    return h ? launch_resident_f16_d8(P, dry_run, s) : launch_resident_bf16_d8(P, dry_run, s);
+}
+
+// Does a head's state fit in LDS (the resident kernel's condition)?
+bool resident_fits(const ma_fwd_params* p) {
+    Problem P;
+    std::memset(&P, 0, sizeof(P));
+    P.E = p->E; P.H = p->H; P.N = p->N; P.D = p->D; P.Dv = p->Dv; P.B = p->B; P.T = p->T;
+    P.M = (p->N + p->B - 1) / p->B;
+    return run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
+}
+
 // The variant a problem resolves to.  AUTO: the MFMA kernels when the problem
-// qualifies; among them the one-launch kernel when there are enough heads to
-// give every team several problems per phase (measured: with E*H >= 32 it beats
-// the per-stage launches, with fewer, larger teams the launch boundaries are
-// cheaper than its in-kernel barriers).
+// qualifies; among them
+//  * the resident kernel when a head's state fits in LDS and there are enough
+//    heads to occupy the device with one workgroup per head,
+//  * else the team kernel (one launch) when there are enough heads to give every
+//    team several problems per phase (measured: with E*H >= 32 it beats the
+//    per-stage launches; with fewer, larger teams the launch boundaries are
+//    cheaper than its in-kernel barriers),
+//  * else one launch per half step.
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
+    const long long heads = static_cast<long long>(p->E) * p->H;
     switch (p->variant) {
         case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
         case MA_VARIANT_STAGED: return fast ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_FUSED: return fast ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_RESIDENT: return fast && resident_fits(p) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
         default:
             if (!fast) return MA_VARIANT_GENERIC;
-            return static_cast<long long>(p->E) * p->H >= 32 ? MA_VARIANT_FUSED : MA_VARIANT_STAGED;
+            if (heads >= 128 && resident_fits(p)) return MA_VARIANT_RESIDENT;
+            return heads >= 32 ? MA_VARIANT_FUSED : MA_VARIANT_STAGED;
     }
 }
 
@@ -251,7 +276,7 @@ int ma_r_step(const ma_fwd_params* p, int first, int with_v, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    if (pr.variant == MA_VARIANT_FUSED) return MA_ERR_UNSUPPORTED;
+    if (pr.variant == MA_VARIANT_FUSED || pr.variant == MA_VARIANT_RESIDENT) return MA_ERR_UNSUPPORTED;
     return run_r(pr, p, first != 0, with_v != 0, static_cast<hipStream_t>(stream));
 }
 
@@ -259,7 +284,7 @@ int ma_l_step(const ma_fwd_params* p, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    if (pr.variant == MA_VARIANT_FUSED) return MA_ERR_UNSUPPORTED;
+    if (pr.variant == MA_VARIANT_FUSED || pr.variant == MA_VARIANT_RESIDENT) return MA_ERR_UNSUPPORTED;
     return run_l(pr, p, static_cast<hipStream_t>(stream));
 }
 
@@ -267,7 +292,7 @@ int ma_z_step(const ma_fwd_params* p, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    if (pr.variant == MA_VARIANT_FUSED) return MA_ERR_UNSUPPORTED;
+    if (pr.variant == MA_VARIANT_FUSED || pr.variant == MA_VARIANT_RESIDENT) return MA_ERR_UNSUPPORTED;
     return run_z(pr, p, static_cast<hipStream_t>(stream));
 }
 
@@ -277,6 +302,7 @@ int ma_fwd(const ma_fwd_params* p, void* stream) {
     if (st != MA_OK) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (pr.variant == MA_VARIANT_FUSED) return run_fused(pr, p, s);
+    if (pr.variant == MA_VARIANT_RESIDENT) return run_resident(pr.P, p->dtype_qk, false, s);
     for (int t = 0; t < p->T - 1; ++t) {
         st = run_r(pr, p, t == 0, false, s);
         if (st) return st;

@@ -71,6 +71,17 @@ int launch_fused_bf16_d4(const Problem& P, bool sync_ready, hipStream_t s);
 int launch_fused_bf16_d5(const Problem& P, bool sync_ready, hipStream_t s);
 int launch_fused_bf16_d8(const Problem& P, bool sync_ready, hipStream_t s);
 
+// Resident forward (one launch, per-head state kept in LDS).  dry_run: only report
+// whether the problem fits (MA_OK / MA_ERR_UNSUPPORTED), launch nothing.
+int launch_resident_f16_d2(const Problem& P, bool dry_run, hipStream_t s);
+int launch_resident_f16_d4(const Problem& P, bool dry_run, hipStream_t s);
+int launch_resident_f16_d5(const Problem& P, bool dry_run, hipStream_t s);
+int launch_resident_f16_d8(const Problem& P, bool dry_run, hipStream_t s);
+int launch_resident_bf16_d2(const Problem& P, bool dry_run, hipStream_t s);
+int launch_resident_bf16_d4(const Problem& P, bool dry_run, hipStream_t s);
+int launch_resident_bf16_d5(const Problem& P, bool dry_run, hipStream_t s);
+int launch_resident_bf16_d8(const Problem& P, bool dry_run, hipStream_t s);
+
 constexpr uint64_t kSyncAreaBytes = 4 * (16 + (16 + 3 * 64) * 1024);  // header + one sector per multi-workgroup team
 // Zero-fills the sync area of a workspace (a small fill kernel, graph-capture safe).
 int launch_zero_sync(unsigned* sync, hipStream_t s);

@@ -2,7 +2,6 @@
 // .hip file per (dtype, head-dim class) so the instantiations compile in parallel.
 #pragma once
 
-#include <cstdlib>
 #include <type_traits>
 
 #include "ma_fused.h"
@@ -76,11 +75,7 @@ int launch_fused_w(const Problem& P, bool sync_ready, hipStream_t s) {
 
 template <class T, int DT, int NTB, int NTM>
 int launch_fused_one(const Problem& P, bool sync_ready, hipStream_t s) {
-    int w = 4;
-    if (const char* e = getenv("MA_FUSED_WAVES")) w = atoi(e);
-    if (w == 16) return launch_fused_w<T, DT, NTB, NTM, 16>(P, sync_ready, s);
-    if (w == 8) return launch_fused_w<T, DT, NTB, NTM, 8>(P, sync_ready, s);
-    return launch_fused_w<T, DT, NTB, NTM, 4>(P, sync_ready, s);
+    return launch_fused_w<T, DT, NTB, NTM, kWaves>(P, sync_ready, s);
 }
 
 template <class T, int DT>

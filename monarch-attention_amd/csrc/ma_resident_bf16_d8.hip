@@ -1,0 +1,6 @@
+// Resident forward kernels, bf16 operands, head-dim class 8 (D <= 128).
+#include "ma_resident_launch.h"
+
+namespace ma {
+int launch_resident_bf16_d8(const Problem& P, bool dry_run, hipStream_t s) { return mfma::launch_resident<bf16, 8>(P, dry_run, s); }
+}  // namespace ma

@@ -1,0 +1,67 @@
+// Host-side dispatch of the resident (state-in-LDS) forward kernel.  Included by
+// one .hip file per (dtype, head-dim class).
+#pragma once
+
+#include <type_traits>
+
+#include "ma_mfma_launch.h"
+#include "ma_resident.h"
+
+namespace ma {
+namespace mfma {
+
+constexpr size_t kLdsPerCu = 160 * 1024;
+constexpr int kResidentWaves = 8;
+
+template <class T, int DT, int NTB, int NTM>
+int launch_resident_one(const Problem& P, bool dry_run, hipStream_t s) {
+    constexpr int W = kResidentWaves;
+    using RS = Resident<T, DT, NTB, NTM, W>;
+    const int Np = P.M * P.B;
+    const size_t lds = RS::lds_bytes(Np);
+    if (lds > kLdsPerCu) return MA_ERR_UNSUPPORTED;   // the head's state does not fit in LDS
+    if (dry_run) return MA_OK;
+    auto kernel = resident_fwd_mfma<T, DT, NTB, NTM, W>;
+    struct Caps {
+        int err = 0, cus = 0;
+    };
+    static const Caps caps = [&] {
+        Caps c;
+        c.err = set_lds_limit(kernel, kLdsPerCu);
+        int dev = 0;
+        if (!c.err) c.err = static_cast<int>(hipGetDevice(&dev));
+        if (!c.err) c.err = static_cast<int>(hipDeviceGetAttribute(&c.cus, hipDeviceAttributeMultiprocessorCount, dev));
+        return c;
+    }();
+    if (caps.err) return caps.err;
+    if (caps.cus < 1) return MA_ERR_DEVICE;
+    // one workgroup per CU at a time when the state takes more than half the LDS, else two;
+    // the workgroups are independent (no waiting on each other), so any grid size is safe
+    const long long heads = static_cast<long long>(P.E) * P.H;
+    const long long per_cu = lds * 2 <= kLdsPerCu ? 2 : 1;
+    long long grid = caps.cus * per_cu;
+    if (grid > heads) grid = heads;
+    hipLaunchKernelGGL((resident_fwd_mfma<T, DT, NTB, NTM, W>), dim3(grid), dim3(64 * W), lds, s, P);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <class T, int DT>
+int launch_resident(const Problem& P, bool dry_run, hipStream_t s) {
+    if (P.B > 64 || P.M > 64) return MA_ERR_UNSUPPORTED;
+    const int ntb = nt_class(P.B), ntm = nt_class(P.M);
+#define MA_NTM(NB)                                                            \
+    switch (ntm) {                                                            \
+        case 1: return launch_resident_one<T, DT, NB, 1>(P, dry_run, s);      \
+        case 2: return launch_resident_one<T, DT, NB, 2>(P, dry_run, s);      \
+        default: return launch_resident_one<T, DT, NB, 4>(P, dry_run, s);     \
+    }
+    switch (ntb) {
+        case 1: MA_NTM(1)
+        case 2: MA_NTM(2)
+        default: MA_NTM(4)
+    }
+#undef MA_NTM
+}
+
+}  // namespace mfma
+}  // namespace ma

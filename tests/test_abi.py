@@ -77,7 +77,7 @@ def test_workspace_layout_is_ordered_and_aligned():
 @pytest.mark.parametrize("field,value,status", [
     ("E", 0, L.MA_ERR_SHAPE), ("N", -3, L.MA_ERR_SHAPE), ("B", 0, L.MA_ERR_SHAPE), ("T", 0, L.MA_ERR_SHAPE),
     ("Dv", 0, L.MA_ERR_SHAPE), ("dtype_qk", 7, L.MA_ERR_DTYPE), ("dtype_v", -1, L.MA_ERR_DTYPE),
-    ("variant", 9, L.MA_ERR_VARIANT),
+    ("variant", 9, L.MA_ERR_VARIANT), ("variant", -1, L.MA_ERR_VARIANT),
 ])
 def test_invalid_problem_is_rejected(field, value, status):
     lib = L.load()
@@ -122,7 +122,7 @@ def test_pointer_and_workspace_checks_precede_any_launch():
 def test_select_variant_reports_a_known_variant():
     lib = L.load()
     v = lib.ma_fwd_select_variant(good_params())
-    assert v in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["fused"])
+    assert v in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["fused"], L.VARIANTS["resident"])
     p32 = good_params(dtype_qk=L.MA_F32, dtype_v=L.MA_F32)
     assert lib.ma_fwd_select_variant(p32) == L.VARIANTS["generic"]
 

@@ -18,7 +18,7 @@ from oracle.ma_oracle import OracleTrace, monarch_attention_oracle, monarch_matr
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-VARIANTS = ["generic", "staged", "fused", "auto"]
+VARIANTS = ["generic", "staged", "fused", "resident", "auto"]
 
 
 def run_hip(q, k, v, mask, T, B, pre, variant):
@@ -297,7 +297,7 @@ FULL = [  # E, H, N, D, B, T, dt
 ]
 
 
-@pytest.mark.parametrize("variant", ["staged", "fused", "auto"])
+@pytest.mark.parametrize("variant", ["staged", "fused", "resident", "auto"])
 @pytest.mark.parametrize("E,H,N,D,B,T,dt", FULL)
 def test_full_size_properties(E, H, N, D, B, T, dt, variant):
     """At the full benchmark sizes: finite output, bit-reproducible, a single
