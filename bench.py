@@ -2,7 +2,7 @@
 """Benchmark of the MonarchAttention forward pass on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cM] [--T 1]
-                    [--variant auto|generic|staged|fused] [--no-cpu] [--no-sdpa]
+                    [--variant auto|generic|staged|fused|resident] [--no-cpu] [--no-sdpa] [--no-sweep]
 
 A step is ONE forward call of the hot path (monarch_attention, all T steps)
 through the C ABI on synthetic inputs that are already resident in HBM.  The
@@ -60,7 +60,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--config", default="cM", choices=sorted(CONFIGS))
     ap.add_argument("--T", type=int, default=None, help="override the number of alternating steps")
-    ap.add_argument("--variant", default="auto", choices=["auto", "generic", "staged", "fused"])
+    ap.add_argument("--variant", default="auto", choices=["auto", "generic", "staged", "fused", "resident"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sdpa", action="store_true", help="skip the dense SDPA comparison")
     ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep")
@@ -152,20 +152,25 @@ def main():
     M = -(-N // B)
     Np = M * B
     kernels = {}
-    if resolved == "fused":
-        kernels["fused_fwd_mfma"] = (event_avg(lambda i: lib.ma_fwd(ps[i % nbuf], sp), min(args.steps, 200)), cbytes)
+    def checked(status):
+        if status:
+            L.check(status, "stage launch")
+
+    if resolved in ("fused", "resident"):   # the whole forward is one kernel
+        kname = "fused_fwd_mfma" if resolved == "fused" else "resident_fwd_mfma"
+        kernels[kname] = (event_avg(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), min(args.steps, 200)), cbytes)
     else:
         # per-stage kernels on the state a full forward left in the workspace
         n = min(args.steps, 200)
         rv_bytes = E * H * ((2 * N * D + N * D) * elt + 2 * Np * D * elt + 4 * Np)          # Q,K,V -> aL,Y,cL
-        kernels["r_step(with V)"] = (event_avg(lambda i: lib.ma_r_step(ps[i % nbuf], int(T == 1), 1, sp), n), rv_bytes)
+        kernels["r_step(with V)"] = (event_avg(lambda i: checked(lib.ma_r_step(ps[i % nbuf], int(T == 1), 1, sp)), n), rv_bytes)
         z_bytes = E * H * (N * D * elt + 2 * Np * D * elt + 4 * Np + N * D * elt)            # Q,aL,Y,cL -> out
-        kernels["z_step"] = (event_avg(lambda i: lib.ma_z_step(ps[i % nbuf], sp), n), z_bytes)
+        kernels["z_step"] = (event_avg(lambda i: checked(lib.ma_z_step(ps[i % nbuf], sp)), n), z_bytes)
         if T > 1:
             l_bytes = E * H * (N * D * elt + Np * D * elt + 4 * Np + Np * D * elt + 4 * Np)  # Q,aL,cL -> aR,cR
-            kernels["l_step"] = (event_avg(lambda i: lib.ma_l_step(ps[i % nbuf], sp), n), l_bytes)
+            kernels["l_step"] = (event_avg(lambda i: checked(lib.ma_l_step(ps[i % nbuf], sp)), n), l_bytes)
             r_bytes = E * H * (2 * N * D * elt + Np * D * elt + 4 * Np + 4 * Np)              # aR,cR,K -> aL,cL
-            kernels["r_step"] = (event_avg(lambda i: lib.ma_r_step(ps[i % nbuf], 0, 0, sp), n), r_bytes)
+            kernels["r_step"] = (event_avg(lambda i: checked(lib.ma_r_step(ps[i % nbuf], 0, 0, sp)), n), r_bytes)
     dom = max(kernels, key=lambda kname: kernels[kname][0])
     dom_ms, dom_bytes = kernels[dom]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
@@ -204,7 +209,7 @@ def main():
     if not args.no_sweep:
         sweep = {}
         for T_ in (1, 2, 3):
-            for variant in ("staged", "fused"):
+            for variant in ("staged", "fused", "resident"):
                 try:
                     _, ems, _, _ = time_forward(T_, variant, max(50, args.steps // 4), 10)
                 except (NotImplementedError, ValueError):

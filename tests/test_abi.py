@@ -135,3 +135,30 @@ def test_check_maps_status_to_python_exceptions():
     with pytest.raises(RuntimeError):
         L.check(L.MA_ERR_WORKSPACE, "x")
     L.check(L.MA_OK, "x")
+
+
+def test_auto_variant_policy():
+    """AUTO: generic when the MFMA kernels do not apply; resident when a head's
+    state fits in LDS and there are many heads; the team kernel from 32 heads;
+    per-stage launches for a few large heads."""
+    lib = L.load()
+
+    def auto(E, H, N, D, B, dt=L.MA_F16, Dv=None):
+        p = L.FwdParams()
+        p.E, p.H, p.N, p.D, p.Dv, p.B, p.T = E, H, N, D, Dv or D, B, 2
+        p.dtype_qk = p.dtype_v = dt
+        for name, w in (("q_stride", D), ("k_stride", D), ("v_stride", p.Dv), ("out_stride", p.Dv)):
+            setattr(p, name, (C.c_int64 * 3)(H * N * w, N * w, w))
+        p.eps = 1e-12
+        return L.VARIANT_NAMES[lib.ma_fwd_select_variant(p)]
+
+    assert auto(1, 16, 4096, 64, 64) == "staged"
+    assert auto(1, 16, 16384, 64, 128) == "staged"
+    assert auto(64, 12, 197, 64, 16) == "resident"
+    assert auto(16, 12, 512, 64, 32) == "fused"        # state of a 512-token head does not fit in LDS
+    assert auto(8, 16, 1024, 72, 32) == "fused"
+    assert auto(2, 2, 197, 64, 16) == "staged"          # few heads
+    assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "generic"
+    assert auto(1, 16, 4096, 64, 64, Dv=128) == "generic"
+    assert auto(1, 16, 4096, 60, 64) == "generic"       # D % 8 != 0
+    assert auto(1, 16, 4096, 64, 256) == "generic"      # B > 128

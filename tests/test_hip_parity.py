@@ -113,6 +113,10 @@ CONFIGS = [  # name, E, H, N, D, B, T, pre, dt, scale
     ("gps", 1, 2, 7600, 48, 128, 2, False, "f32", 1.0),
     ("vit_b14", 2, 12, 197, 64, 14, 2, True, "f16", 0.125),
     ("roberta_b24", 2, 12, 384, 64, 24, 1, False, "f16", 1.0),
+    ("big_block", 1, 2, 600, 64, 200, 2, False, "f16", 1.0),       # B > 128: beyond the MFMA tiles, AUTO -> generic
+    ("many_blocks", 1, 2, 4096, 32, 16, 2, False, "bf16", 1.0),    # M = 256 > 128: AUTO -> generic
+    ("one_block", 2, 2, 100, 64, 128, 3, True, "f16", 1.0),        # M = 1: dense softmax attention
+    ("unit_blocks", 1, 2, 96, 32, 1, 1, False, "f16", 1.0),        # B = 1, M = N
     ("many_heads", 40, 64, 64, 32, 16, 2, False, "f16", 1.0),      # more heads than co-resident workgroups
     ("many_heads_odd", 3, 7, 80, 32, 16, 3, True, "bf16", 1.0),    # odd head count, ragged N
 ]
@@ -225,6 +229,34 @@ def test_stages_against_oracle_trace(E, H, N, D, Dv, B, T, pre, dt, vdt, with_ma
     st["Y"].copy_(tr.steps[-1]["Y"].to(DEV))
     _call(lib.ma_z_step, p, None)
     assert_parity(out.cpu(), ref, dt if dt == vdt else dt, "Z")
+
+
+def test_empty_and_invalid_inputs_raise():
+    q = torch.empty(1, 2, 0, 64, dtype=torch.float16, device=DEV)
+    with pytest.raises(ValueError):
+        monarch_attention_hip(q, q, q, None, 1, 16, False)
+    q, k, v = to_dev(*seeded_qkv(1, 2, 32, 64, torch.float16))
+    with pytest.raises(ValueError):
+        monarch_attention_hip(q, k, v, None, 1, 16, False, variant="nope")
+    with pytest.raises(NotImplementedError):                 # fp32 cannot run on the MFMA kernels: no silent fallback
+        monarch_attention_hip(q.float(), k.float(), v.float(), None, 1, 16, False, variant="staged")
+    with pytest.raises(NotImplementedError):
+        with torch.enable_grad():
+            monarch_attention_hip(q.requires_grad_(), k, v, None, 1, 16, False)
+
+
+def test_workspace_is_shared_across_shapes_and_calls():
+    """One cached workspace serves calls of different shapes back to back (the
+    fused kernels' barrier epochs continue across launches)."""
+    outs = []
+    shapes = [(1, 16, 1024, 64, 64, 2), (2, 40, 128, 64, 16, 3), (1, 2, 2048, 64, 32, 1), (1, 16, 1024, 64, 64, 2)]
+    for rep in range(3):
+        for (E, H, N, D, B, T) in shapes:
+            q, k, v = seeded_qkv(E, H, N, D, torch.float16)
+            ref = monarch_attention_oracle(q, k, v, None, T, B, False, upcast=True)
+            for variant in ("fused", "staged"):
+                out = run_hip(*to_dev(q, k, v), None, T, B, False, variant)
+                assert_parity(out.cpu(), ref, "f16", f"rep{rep}/{variant}/{(E, H, N, B, T)}")
 
 
 # ---------------------------------------------------------------- caller-side layouts and masks
