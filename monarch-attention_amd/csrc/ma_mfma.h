@@ -309,65 +309,97 @@ __device__ __forceinline__ unsigned tok_off(int t, int N, unsigned st) {
 }
 
 // ============================================================================
+// The three block problems.  Each is split in three parts so that a caller can
+// overlap memory latency with other work:
+//   issue()  starts the loads that depend only on the INPUTS (K / V / Q tiles and
+//            rows, mask bytes) into registers (Pre) - they may be issued long
+//            before the problem runs, e.g. while the previous problem computes;
+//   state()  starts the loads of the STATE another phase produced (aR rows, aL /
+//            Y tiles, cL, cR) into registers (St) - only legal once that phase
+//            is known to be complete;
+//   run()    commits the tiles to LDS and does the arithmetic; it contains no
+//            global load of its own for problems of up to 64 rows.
+// `active` is uniform per wave; inactive waves only take part in the barriers.
+// ============================================================================
+
 // R step for one block problem (e,h,m), run by WPP waves (wig = wave in group).
 // smem: K tile, V tile, key bias.   Reference: al_cl_ref / al_y_cl_ref
 // (ma/ma_torch.py:10-23, :38-52).
-// ============================================================================
 template <class T, int DT, int NWT>
-__device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int m,
-                                          bool first, bool with_v, int wig, int lane) {
+struct RProb {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
-    constexpr int WPP = Split<NWT>::WPP;
-    constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
-    T* Kt = reinterpret_cast<T*>(smem);
-    T* Vt = Kt + Lds<T, DT, NWT>::TILE;
-    float* kbias = reinterpret_cast<float*>(Vt + Lds<T, DT, NWT>::TILE);
-    const int B = P.B, M = P.M, D = P.D;
-    const int r = lane & 15, q = lane >> 4;
-    const int tix = wig * 64 + lane;
-    const unsigned db = static_cast<unsigned>(D) * sizeof(T);
-    const Slices S = make_slices<T>(P, e, h, wh);
-
-    // the R problem's first strip of queries (one strip per wave unless the block has more than 64 rows)
-    auto load_strip = [&](int strip, typename Ops<T>::v8 (&xb)[G::KS], float& cr) {
-        const int j = 16 * strip + r;
-        const bool jv = j < B;
-        const unsigned rowid = static_cast<unsigned>(m * B + j);   // row inside the head's state
-        cr = 1.0f;
-        if (first) {
-            load_x<T, DT, true>(xb, S.q, jv ? tok_off(m * B + j - P.pad_off, P.N, S.qst) : kOob, D, q);
-        } else {
-            load_x<T, DT, true>(xb, S.aR, jv ? rowid * db : kOob, D, q);
-            cr = bloadf<true>(S.cR, jv ? rowid * 4u : kOob);   // an out-of-range row reads 0: harmless, never stored
-        }
-    };
-    V8 xb0[G::KS];
-    float cr0 = 1.0f;
-    if (active) {
-        // every load of the problem goes out before the first wait
-        const int t0 = m * B - P.pad_off;
+    static constexpr int WPP = Split<NWT>::WPP;
+    static constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
+    struct Pre {
         TileCopy<T, DT, ROWS, WPP * 64> kc, vc;
-        kc.template issue<true>(S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
-        if (with_v) vc.template issue<true>(S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix);
-        load_strip(wig, xb0, cr0);
-        for (int i = tix; i < ROWS; i += WPP * 64) kbias[i] = (i < B && token_ok(P, e, t0 + i)) ? 0.f : kNegBig;
-        kc.commit(Kt, tix);
-        if (with_v) vc.commit(Vt, tix);
+        V8 xq[G::KS];   // first step: the first strip's Q rows
+        float kb;       // key bias of tile row `tix`
+    };
+    struct St {
+        V8 xa[G::KS];   // later steps: the first strip's aR rows
+        float cr;
+    };
+
+    static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int e, int m, bool first,
+                                                 bool with_v, int wig, int lane) {
+        if (!active) return;
+        const int B = P.B, D = P.D;
+        const int tix = wig * 64 + lane;
+        const int t0 = m * B - P.pad_off;
+        pre.kc.template issue<true>(S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
+        if (with_v) pre.vc.template issue<true>(S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix);
+        if (first) {
+            const int j = 16 * wig + (lane & 15);
+            load_x<T, DT, true>(pre.xq, S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, lane >> 4);
+        }
+        pre.kb = (tix < B && token_ok(P, e, t0 + tix)) ? 0.f : kNegBig;
     }
-    __syncthreads();
-    if (active) {
+
+    static __device__ __forceinline__ void load_state_strip(const Problem& P, const Slices& S, V8 (&xa)[G::KS], float& cr, int m,
+                                                            int strip, int lane) {
+        const int j = 16 * strip + (lane & 15);
+        const unsigned rowid = static_cast<unsigned>(m * P.B + j);   // row inside the head's state
+        const unsigned db = static_cast<unsigned>(P.D) * sizeof(T);
+        load_x<T, DT, true>(xa, S.aR, j < P.B ? rowid * db : kOob, P.D, lane >> 4);
+        cr = bloadf<true>(S.cR, j < P.B ? rowid * 4u : kOob);   // an out-of-range row reads 0: harmless, never stored
+    }
+
+    static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int m, bool first, int wig,
+                                                 int lane) {
+        st.cr = 1.0f;
+        if (active && !first) load_state_strip(P, S, st.xa, st.cr, m, wig, lane);
+    }
+
+    static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
+                                               int m, bool first, bool with_v, int wig, int lane) {
+        T* Kt = reinterpret_cast<T*>(smem);
+        T* Vt = Kt + Lds<T, DT, NWT>::TILE;
+        float* kbias = reinterpret_cast<float*>(Vt + Lds<T, DT, NWT>::TILE);
+        const int B = P.B, M = P.M, D = P.D;
+        const int r = lane & 15, q = lane >> 4;
+        const int tix = wig * 64 + lane;
+        const unsigned db = static_cast<unsigned>(D) * sizeof(T);
+        if (active) {
+            pre.kc.commit(Kt, tix);
+            if (with_v) pre.vc.commit(Vt, tix);
+            if (tix < ROWS) kbias[tix] = pre.kb;
+        }
+        __syncthreads();
+        if (!active) return;
         for (int strip = wig; strip < NWT; strip += WPP) {
             const int j = 16 * strip + r;
             const bool jv = j < B;
             V8 xb[G::KS];
-            float cr;
+            float cr = 1.0f;
             if (strip == wig) {
 #pragma unroll
-                for (int ks = 0; ks < G::KS; ++ks) xb[ks] = xb0[ks];
-                cr = cr0;
+                for (int ks = 0; ks < G::KS; ++ks) xb[ks] = first ? pre.xq[ks] : st.xa[ks];
+                cr = st.cr;
+            } else if (first) {   // blocks of more than 64 rows: a second strip per wave
+                load_x<T, DT, true>(xb, S.q, jv ? tok_off(m * B + j - P.pad_off, P.N, S.qst) : kOob, D, q);
             } else {
-                load_strip(strip, xb, cr);
+                load_state_strip(P, S, xb, cr, m, strip, lane);
             }
             const float cj = (P.sm_scale * kLog2e) / (cr + P.eps);  // logits in log2 units
 
@@ -432,46 +464,56 @@ __device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool act
             }
         }
     }
-}
+};
 
-// ============================================================================
 // Z step for one column problem (e,h,j).  smem: aL tile, Y tile, cL bias.
 // Reference: z_ref (ma/ma_torch.py:55-62) and the final slice (:106-108).
-// ============================================================================
 template <class T, int DT, int NWT>
-__device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int j,
-                                          int wig, int lane) {
+struct ZProb {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
-    constexpr int WPP = Split<NWT>::WPP;
-    constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
-    T* At = reinterpret_cast<T*>(smem);
-    T* Yt = At + Lds<T, DT, NWT>::TILE;
-    float* cb = reinterpret_cast<float*>(Yt + Lds<T, DT, NWT>::TILE);
-    const int B = P.B, M = P.M, D = P.D;
-    const int r = lane & 15, q = lane >> 4;
-    const int tix = wig * 64 + lane;
-    const unsigned db = static_cast<unsigned>(D) * sizeof(T);
-    const Slices S = make_slices<T>(P, e, h, wh);
-
-    auto load_strip = [&](int strip, typename Ops<T>::v8 (&xb)[G::KS]) {
-        const int l = 16 * strip + r;
-        load_x<T, DT, true>(xb, S.q, l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob, D, q);
+    static constexpr int WPP = Split<NWT>::WPP;
+    static constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
+    struct Pre {
+        V8 xq[G::KS];   // the first strip's Q rows
     };
-    V8 xb0[G::KS];
-    if (active) {
-        // every load of the problem goes out before the first wait
-        const unsigned row0 = static_cast<unsigned>(j * M);
+    struct St {
         TileCopy<T, DT, ROWS, WPP * 64> ac, yc;
-        ac.template issue<true>(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
-        yc.template issue<true>(S.Y, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
-        load_strip(wig, xb0);
-        for (int k = tix; k < ROWS; k += WPP * 64) cb[k] = k < M ? -kLog2e * bloadf<true>(S.cL, (row0 + k) * 4u) : kNegBig;
-        ac.commit(At, tix);
-        yc.commit(Yt, tix);
+        float cbv;      // softmax bias of tile row `tix`
+    };
+
+    static __device__ __forceinline__ void load_strip(const Problem& P, const Slices& S, V8 (&xb)[G::KS], int j, int strip, int lane) {
+        const int l = 16 * strip + (lane & 15);
+        load_x<T, DT, true>(xb, S.q, l < P.M ? tok_off(l * P.B + j - P.pad_off, P.N, S.qst) : kOob, P.D, lane >> 4);
     }
-    __syncthreads();
-    if (active) {
+    static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int j, int wig, int lane) {
+        if (active) load_strip(P, S, pre.xq, j, wig, lane);
+    }
+    static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
+        if (!active) return;
+        const int M = P.M, D = P.D;
+        const int tix = wig * 64 + lane;
+        const unsigned db = static_cast<unsigned>(D) * sizeof(T);
+        const unsigned row0 = static_cast<unsigned>(j * M);
+        st.ac.template issue<true>(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        st.yc.template issue<true>(S.Y, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        st.cbv = tix < M ? -kLog2e * bloadf<true>(S.cL, (row0 + tix) * 4u) : kNegBig;
+    }
+    static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
+                                               int j, int wig, int lane) {
+        T* At = reinterpret_cast<T*>(smem);
+        T* Yt = At + Lds<T, DT, NWT>::TILE;
+        float* cb = reinterpret_cast<float*>(Yt + Lds<T, DT, NWT>::TILE);
+        const int B = P.B, M = P.M, D = P.D;
+        const int r = lane & 15, q = lane >> 4;
+        const int tix = wig * 64 + lane;
+        if (active) {
+            st.ac.commit(At, tix);
+            st.yc.commit(Yt, tix);
+            if (tix < ROWS) cb[tix] = st.cbv;
+        }
+        __syncthreads();
+        if (!active) return;
         for (int strip = wig; strip < NWT; strip += WPP) {
             const int l = 16 * strip + r;
             const int t = l * B + j - P.pad_off;
@@ -479,9 +521,9 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
             V8 xb[G::KS];
             if (strip == wig) {
 #pragma unroll
-                for (int ks = 0; ks < G::KS; ++ks) xb[ks] = xb0[ks];
+                for (int ks = 0; ks < G::KS; ++ks) xb[ks] = pre.xq[ks];
             } else {
-                load_strip(strip, xb);
+                load_strip(P, S, xb, j, strip, lane);
             }
             f32x4 C[NWT];
 #pragma unroll
@@ -521,140 +563,203 @@ __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool act
             store_row<T, DT>(S.out, lv ? tok_off(t, P.N, S.ost) : kOob, D, O, q);   // padded query rows are dropped (:108)
         }
     }
-}
+};
 
-// ============================================================================
 // L step for one column problem (e,h,j).  smem: Qt tile (ROWS2 rows), aL tile,
 // transposed L tile PT[k][l], cL bias, per-wave partial cR.
 // Reference: ar_cr_ref (ma/ma_torch.py:26-35).
-// ============================================================================
 template <class T, int DT, int NWT>
-__device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int j,
-                                          int wig, int lane) {
+struct LProb {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
     using LS = Lds<T, DT, NWT>;
-    constexpr int WPP = Split<NWT>::WPP;
-    constexpr int ROWS = LS::ROWS, ROWS2 = LS::ROWS2, LDP = LS::LDP, NG = (NWT + 1) / 2;
-    T* Qt = reinterpret_cast<T*>(smem);
-    T* At = Qt + LS::TILE2;
-    T* PT = At + LS::TILE;
-    float* cb = reinterpret_cast<float*>(PT + ROWS * LDP);
-    float* crp = cb + ROWS;  // [WPP][ROWS]
-    const int B = P.B, M = P.M, D = P.D;
-    const int r = lane & 15, q = lane >> 4;
-    const int tix = wig * 64 + lane;
-    constexpr int nth = WPP * 64;
-    const unsigned db = static_cast<unsigned>(D) * sizeof(T);
-    const Slices S = make_slices<T>(P, e, h, wh);
+    static constexpr int WPP = Split<NWT>::WPP;
+    static constexpr int ROWS = LS::ROWS, ROWS2 = LS::ROWS2, LDP = LS::LDP, NG = (NWT + 1) / 2;
+    static constexpr int nth = WPP * 64;
+    static constexpr int SPW = NWT / WPP;   // strips per wave (2 for blocks counts above 64)
+    struct Pre {
+        TileCopy<T, DT, ROWS2, nth> qc;   // Q^T tile
+        unsigned qok;                     // bit 4*i + v: query block 16*(wig + i*WPP) + 4q + v is real and unmasked
+    };
+    struct St {
+        TileCopy<T, DT, ROWS, nth> ac;    // aL tile
+        float cbv;
+    };
 
-    if (active) {
-        const unsigned row0 = static_cast<unsigned>(j * M);
-        TileCopy<T, DT, ROWS2, nth> qc;
-        TileCopy<T, DT, ROWS, nth> ac;
-        qc.template issue<true>(S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
-        ac.template issue<true>(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
-        for (int k = tix; k < ROWS; k += nth) cb[k] = k < M ? -kLog2e * bloadf<true>(S.cL, (row0 + k) * 4u) : kNegBig;
-        qc.commit(Qt, tix);
-        ac.commit(At, tix);
-        if (ROWS2 > ROWS)  // zero the phantom l columns of PT that phase 2 reads
-            for (int i = tix; i < ROWS * (ROWS2 - ROWS); i += nth) PT[(i / (ROWS2 - ROWS)) * LDP + ROWS + i % (ROWS2 - ROWS)] = from_f<T>(0.f);
-    }
-    __syncthreads();
-    if (active) {
-        // phase 1: L[l, k] for 16-row strips of l; lane holds column k = 16kt + r, rows l0 + 4q + v
-        float crsum[NWT];
+    static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int e, int j, int wig,
+                                                 int lane) {
+        if (!active) return;
+        const int B = P.B, M = P.M;
+        const int tix = wig * 64 + lane;
+        pre.qc.template issue<true>(S.q, P.D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
+        unsigned ok = 0;
 #pragma unroll
-        for (int kt = 0; kt < NWT; ++kt) crsum[kt] = 0.f;
-        for (int strip = wig; strip < NWT; strip += WPP) {
-            const int l0 = 16 * strip;
-            V8 xa[G::KS];
-#pragma unroll
-            for (int ks = 0; ks < G::KS; ++ks) xa[ks] = lds_row8<T>(Qt + (l0 + r) * G::LD + 32 * ks + 8 * q);
-            f32x4 C[NWT];
-#pragma unroll
-            for (int kt = 0; kt < NWT; ++kt) {
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(xa[ks], lds_row8<T>(At + (16 * kt + r) * G::LD + 32 * ks + 8 * q), acc);
-                const float b = cb[16 * kt + r];
-#pragma unroll
-                for (int v = 0; v < 4; ++v) acc[v] = fmaf(round_to<T>(acc[v]), kLog2e, b);
-                C[kt] = acc;
-            }
-            f32x4 mx = C[0];
-#pragma unroll
-            for (int kt = 1; kt < NWT; ++kt)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) mx[v] = fmaxf(mx[v], C[kt][v]);
-#pragma unroll
-            for (int v = 0; v < 4; ++v) mx[v] = row16_max(mx[v]);
-            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int kt = 0; kt < NWT; ++kt)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float p = __builtin_amdgcn_exp2f(C[kt][v] - mx[v]);
-                    sum[v] += p;
-                    C[kt][v] = p;
-                }
-            f32x4 inv;
+        for (int i = 0; i < SPW; ++i)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const int l = l0 + 4 * q + v;
+                const int l = 16 * (wig + i * WPP) + 4 * (lane >> 4) + v;
                 // padded / masked query tokens are zeroed after the softmax (ma_torch.py:30)
-                const bool ok = l < M && token_ok(P, e, l * B + j - P.pad_off);
-                const float s = row16_sum(sum[v]);
-                inv[v] = ok ? 1.0f / s : 0.f;
+                if (l < M && token_ok(P, e, l * B + j - P.pad_off)) ok |= 1u << (4 * i + v);
+            }
+        pre.qok = ok;
+    }
+    static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
+        if (!active) return;
+        const int M = P.M, D = P.D;
+        const int tix = wig * 64 + lane;
+        const unsigned db = static_cast<unsigned>(D) * sizeof(T);
+        const unsigned row0 = static_cast<unsigned>(j * M);
+        st.ac.template issue<true>(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        st.cbv = tix < M ? -kLog2e * bloadf<true>(S.cL, (row0 + tix) * 4u) : kNegBig;
+    }
+    static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
+                                               int j, int wig, int lane) {
+        T* Qt = reinterpret_cast<T*>(smem);
+        T* At = Qt + LS::TILE2;
+        T* PT = At + LS::TILE;
+        float* cb = reinterpret_cast<float*>(PT + ROWS * LDP);
+        float* crp = cb + ROWS;  // [WPP][ROWS]
+        const int B = P.B, M = P.M, D = P.D;
+        const int r = lane & 15, q = lane >> 4;
+        const int tix = wig * 64 + lane;
+        const unsigned db = static_cast<unsigned>(D) * sizeof(T);
+        if (active) {
+            pre.qc.commit(Qt, tix);
+            st.ac.commit(At, tix);
+            if (tix < ROWS) cb[tix] = st.cbv;
+            constexpr int PH = ROWS2 > ROWS ? ROWS2 - ROWS : 1;   // phantom l columns of PT that phase 2 reads
+            if (ROWS2 > ROWS)
+                for (int i = tix; i < ROWS * PH; i += nth) PT[(i / PH) * LDP + ROWS + i % PH] = from_f<T>(0.f);
+        }
+        __syncthreads();
+        if (active) {
+            // phase 1: L[l, k] for 16-row strips of l; lane holds column k = 16kt + r, rows l0 + 4q + v
+            float crsum[NWT];
+#pragma unroll
+            for (int kt = 0; kt < NWT; ++kt) crsum[kt] = 0.f;
+#pragma unroll
+            for (int si = 0; si < SPW; ++si) {
+                const int l0 = 16 * (wig + si * WPP);
+                V8 xa[G::KS];
+#pragma unroll
+                for (int ks = 0; ks < G::KS; ++ks) xa[ks] = lds_row8<T>(Qt + (l0 + r) * G::LD + 32 * ks + 8 * q);
+                f32x4 C[NWT];
+#pragma unroll
+                for (int kt = 0; kt < NWT; ++kt) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(xa[ks], lds_row8<T>(At + (16 * kt + r) * G::LD + 32 * ks + 8 * q), acc);
+                    const float b = cb[16 * kt + r];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[v] = fmaf(round_to<T>(acc[v]), kLog2e, b);
+                    C[kt] = acc;
+                }
+                f32x4 mx = C[0];
+#pragma unroll
+                for (int kt = 1; kt < NWT; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) mx[v] = fmaxf(mx[v], C[kt][v]);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) mx[v] = row16_max(mx[v]);
+                f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kt = 0; kt < NWT; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float p = __builtin_amdgcn_exp2f(C[kt][v] - mx[v]);
+                        sum[v] += p;
+                        C[kt][v] = p;
+                    }
+                f32x4 inv;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float sv = row16_sum(sum[v]);
+                    inv[v] = ((pre.qok >> (4 * si + v)) & 1u) ? 1.0f / sv : 0.f;
+                }
+#pragma unroll
+                for (int kt = 0; kt < NWT; ++kt) {
+                    typename Ops<T>::v4 o;
+                    float part = 0.f;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float lv = C[kt][v] * inv[v];
+                        part += lv;
+                        o[v] = from_f<T>(lv);
+                    }
+                    crsum[kt] += part;
+                    *reinterpret_cast<u32x2*>(PT + (16 * kt + r) * LDP + l0 + 4 * q) = __builtin_bit_cast(u32x2, o);
+                }
             }
 #pragma unroll
             for (int kt = 0; kt < NWT; ++kt) {
-                typename Ops<T>::v4 o;
-                float part = 0.f;
+                const float sv = quad_rows_sum(crsum[kt]);
+                if (q == 0) crp[wig * ROWS + 16 * kt + r] = sv;
+            }
+        }
+        __syncthreads();
+        if (active) {
+            // phase 2: aR[k, :] = sum_l round(L[l,k]) Qt[l, :] for 16-wide tiles of k
+            for (int kt = wig; kt < NWT; kt += WPP) {
+                const int k = 16 * kt + r;
+                const bool kv = k < M;
+                V8 pb[NG];
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float lv = C[kt][v] * inv[v];
-                    part += lv;
-                    o[v] = from_f<T>(lv);
+                for (int g = 0; g < NG; ++g) pb[g] = lds_row8<T>(PT + k * LDP + 32 * g + 8 * q);
+                f32x4 O[DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int g = 0; g < NG; ++g)   // natural k-slot order here: slot s <-> row 32g + 8q + s
+                        acc = Ops<T>::mma(lds_tr8<T, DT>(Qt, 32 * g + 8 * q, 4, true, dt, r), pb[g], acc);
+                    O[dt] = acc;
                 }
-                crsum[kt] += part;
-                *reinterpret_cast<u32x2*>(PT + (16 * kt + r) * LDP + l0 + 4 * q) = __builtin_bit_cast(u32x2, o);
-            }
-        }
+                const unsigned arow = static_cast<unsigned>(k * B + j);   // row of aR / cR: (k, j)
+                store_row<T, DT>(S.aR, kv ? arow * db : kOob, D, O, q);
+                if (q == 0) {
+                    float sv = 0.f;
 #pragma unroll
-        for (int kt = 0; kt < NWT; ++kt) {
-            const float s = quad_rows_sum(crsum[kt]);
-            if (q == 0) crp[wig * ROWS + 16 * kt + r] = s;
-        }
-    }
-    __syncthreads();
-    if (active) {
-        // phase 2: aR[k, :] = sum_l round(L[l,k]) Qt[l, :] for 16-wide tiles of k
-        for (int kt = wig; kt < NWT; kt += WPP) {
-            const int k = 16 * kt + r;
-            const bool kv = k < M;
-            V8 pb[NG];
-#pragma unroll
-            for (int g = 0; g < NG; ++g) pb[g] = lds_row8<T>(PT + k * LDP + 32 * g + 8 * q);
-            f32x4 O[DT];
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int g = 0; g < NG; ++g)   // natural k-slot order here: slot s <-> row 32g + 8q + s
-                    acc = Ops<T>::mma(lds_tr8<T, DT>(Qt, 32 * g + 8 * q, 4, true, dt, r), pb[g], acc);
-                O[dt] = acc;
-            }
-            const unsigned arow = static_cast<unsigned>(k * B + j);   // row of aR / cR: (k, j)
-            store_row<T, DT>(S.aR, kv ? arow * db : kOob, D, O, q);
-            if (q == 0) {
-                float s = 0.f;
-#pragma unroll
-                for (int w = 0; w < WPP; ++w) s += crp[w * ROWS + k];
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, s), S.cR, kv ? arow * 4u : kOob, 0, 0);
+                    for (int w = 0; w < WPP; ++w) sv += crp[w * ROWS + k];
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, sv), S.cR, kv ? arow * 4u : kOob, 0, 0);
+                }
             }
         }
     }
+};
+
+// the three parts back to back (one launch per half step has nothing to overlap them with)
+template <class T, int DT, int NWT>
+__device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int m,
+                                          bool first, bool with_v, int wig, int lane) {
+    using RP = RProb<T, DT, NWT>;
+    const Slices S = make_slices<T>(P, e, h, wh);
+    typename RP::Pre pre;
+    typename RP::St st;
+    RP::issue(P, S, pre, active, e, m, first, with_v, wig, lane);
+    RP::state(P, S, st, active, m, first, wig, lane);
+    RP::run(P, S, smem, pre, st, active, m, first, with_v, wig, lane);
+}
+template <class T, int DT, int NWT>
+__device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int j,
+                                          int wig, int lane) {
+    using ZP = ZProb<T, DT, NWT>;
+    const Slices S = make_slices<T>(P, e, h, wh);
+    typename ZP::Pre pre;
+    typename ZP::St st;
+    ZP::state(P, S, st, active, j, wig, lane);
+    ZP::issue(P, S, pre, active, j, wig, lane);
+    ZP::run(P, S, smem, pre, st, active, j, wig, lane);
+}
+template <class T, int DT, int NWT>
+__device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int j,
+                                          int wig, int lane) {
+    using LP = LProb<T, DT, NWT>;
+    const Slices S = make_slices<T>(P, e, h, wh);
+    typename LP::Pre pre;
+    typename LP::St st;
+    LP::state(P, S, st, active, j, wig, lane);
+    LP::issue(P, S, pre, active, e, j, wig, lane);
+    LP::run(P, S, smem, pre, st, active, j, wig, lane);
 }
 
 // ---- staged kernels: one launch per half step ---------------------------------
