@@ -199,7 +199,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, l
 template <class T, int DT, int NTB, int NTM, int W>
 __global__ __launch_bounds__(64 * W) void fused_fwd_mfma(Problem P, FusedPlan plan) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = wave_id(), lane = threadIdx.x & 63;
     const int G = plan.G;
     int team, member;
     if (plan.xcd_map) {

@@ -34,6 +34,13 @@
 namespace ma {
 namespace mfma {
 
+// Index of the wave inside its workgroup, as a value the compiler knows to be
+// uniform: everything derived from it (problem index, tensor slices, buffer
+// resources) then lives in scalar registers, and buffer instructions take their
+// resource operand directly instead of through a per-lane "waterfall" loop.
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x)) >> 6; }
+
+
 constexpr int kWaves = 4;
 constexpr int kThreads = 64 * kWaves;
 constexpr float kLog2e = 1.4426950408889634f;
@@ -767,7 +774,7 @@ template <class T, int DT, int NWT>
 __global__ __launch_bounds__(kThreads) void r_step_mfma(Problem P, int first, int with_v) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
     const long long total = static_cast<long long>(P.E) * P.H * P.M;
     long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;
@@ -784,7 +791,7 @@ template <class T, int DT, int NWT>
 __global__ __launch_bounds__(kThreads) void l_step_mfma(Problem P) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
     const long long total = static_cast<long long>(P.E) * P.H * P.B;
     long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;
@@ -800,7 +807,7 @@ template <class T, int DT, int NWT>
 __global__ __launch_bounds__(kThreads) void z_step_mfma(Problem P) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
     const long long total = static_cast<long long>(P.E) * P.H * P.B;
     long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;

@@ -444,7 +444,7 @@ __global__ __launch_bounds__(64 * W) void resident_fwd_mfma(Problem P) {
     c.cLs = reinterpret_cast<float*>(c.ZR + RS::LD);
     c.cRs = c.cLs + (Np + 3) / 4 * 4;
     c.stage = smem + RS::state_bytes(Np);
-    c.wave = threadIdx.x >> 6;
+    c.wave = wave_id();
     c.lane = threadIdx.x & 63;
     c.r = c.lane & 15;
     c.q = c.lane >> 4;
