@@ -45,13 +45,16 @@ struct Resident {
     static constexpr size_t kStageR = 2 * ROWSB * LD * sizeof(T) + ROWSB * sizeof(float);
     static constexpr size_t kStageL = (ROWSM * LD + ROWSM * LDP) * sizeof(T) + (1 + WPM) * ROWSM * sizeof(float);
     static constexpr size_t kSlotR = (kStageR + 15) / 16 * 16, kSlotL = (kStageL + 15) / 16 * 16;
-    static constexpr size_t kStage = (PPB * kSlotR > PPM * kSlotL) ? PPB * kSlotR : PPM * kSlotL;
 
     static __host__ __device__ size_t state_bytes(int Np) {   // SA, SX, SY, ZR, cLs, cRs
         const size_t np4 = (static_cast<size_t>(Np) + 3) / 4 * 4;
         return (3 * static_cast<size_t>(Np) + 1) * LD * sizeof(T) + 2 * np4 * sizeof(float);
     }
-    static __host__ __device__ size_t lds_bytes(int Np) { return state_bytes(Np) + kStage; }
+    // staging is only needed for the problems a round can actually hold
+    static __host__ __device__ size_t lds_bytes(int Np, int M, int B) {
+        const size_t sr = static_cast<size_t>(M < PPB ? M : PPB) * kSlotR, sl = static_cast<size_t>(B < PPM ? B : PPM) * kSlotL;
+        return state_bytes(Np) + (sr > sl ? sr : sl);
+    }
 
     // registers that carry one round's global loads from issue to execute
     struct Pre {
@@ -449,6 +452,13 @@ __global__ __launch_bounds__(64 * W) void resident_fwd_mfma(Problem P) {
     c.r = c.lane & 15;
     c.q = c.lane >> 4;
     for (int i = threadIdx.x; i < RS::LD; i += 64 * W) c.ZR[i] = from_f<T>(0.f);
+    // The state rows are written 16*DT columns wide but read as GEMM operands over all 32*KS
+    // columns: where the two differ (head dims of 65..80) the columns in between are never
+    // written and must not hold leftovers (0 * NaN) of whatever used the LDS before.
+    if constexpr (16 * DT < 32 * RS::KS) {
+        constexpr int kTail = 32 * RS::KS - 16 * DT;
+        for (int i = threadIdx.x; i < 3 * Np * kTail; i += 64 * W) c.SA[(i / kTail) * RS::LD + 16 * DT + i % kTail] = from_f<T>(0.f);
+    }
     __syncthreads();
 
     const int heads = P.E * P.H;

@@ -11,14 +11,14 @@ namespace ma {
 namespace mfma {
 
 constexpr size_t kLdsPerCu = 160 * 1024;
-constexpr int kResidentWaves = 8;
+constexpr int kResidentWaves = 8;       // workgroup size in waves ...
+constexpr int kResidentWavesWide = 16;  // ... and for blocks of up to 32 rows when the staging of 16 waves still fits
 
-template <class T, int DT, int NTB, int NTM>
-int launch_resident_one(const Problem& P, bool dry_run, hipStream_t s) {
-    constexpr int W = kResidentWaves;
+template <class T, int DT, int NTB, int NTM, int W>
+int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
     using RS = Resident<T, DT, NTB, NTM, W>;
     const int Np = P.M * P.B;
-    const size_t lds = RS::lds_bytes(Np);
+    const size_t lds = RS::lds_bytes(Np, P.M, P.B);
     if (lds > kLdsPerCu) return MA_ERR_UNSUPPORTED;   // the head's state does not fit in LDS
     if (dry_run) return MA_OK;
     auto kernel = resident_fwd_mfma<T, DT, NTB, NTM, W>;
@@ -43,6 +43,17 @@ int launch_resident_one(const Problem& P, bool dry_run, hipStream_t s) {
     if (grid > heads) grid = heads;
     hipLaunchKernelGGL((resident_fwd_mfma<T, DT, NTB, NTM, W>), dim3(grid), dim3(64 * W), lds, s, P);
     return static_cast<int>(hipGetLastError());
+}
+
+// The problems of a head are small and latency-bound: more waves per workgroup run more of
+// them at once, so the wide workgroup is preferred wherever its staging fits beside the state.
+template <class T, int DT, int NTB, int NTM>
+int launch_resident_one(const Problem& P, bool dry_run, hipStream_t s) {
+    if constexpr (NTB <= 2 && NTM <= 2) {
+        const int err = launch_resident_w<T, DT, NTB, NTM, kResidentWavesWide>(P, dry_run, s);
+        if (err != MA_ERR_UNSUPPORTED) return err;
+    }
+    return launch_resident_w<T, DT, NTB, NTM, kResidentWaves>(P, dry_run, s);
 }
 
 template <class T, int DT>
