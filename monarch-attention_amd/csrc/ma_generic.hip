@@ -47,7 +47,8 @@ __device__ __forceinline__ float dot_rows(const T* a, const T* b, int D) {
     if (D % 4 == 0 && (reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % sizeof(Quad) == 0) {
         const Quad* qa = reinterpret_cast<const Quad*>(a);
         const Quad* qb = reinterpret_cast<const Quad*>(b);
-        for (int d = 0; d < D / 4; ++d) {
+#pragma unroll 4
+        for (int d = 0; d < D / 4; ++d) {   // unrolled: the loads of several steps are in flight together
             const Quad x = qa[d], y = qb[d];
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc = fmaf(to_f(x.v[i]), to_f(y.v[i]), acc);
@@ -55,6 +56,25 @@ __device__ __forceinline__ float dot_rows(const T* a, const T* b, int D) {
         return acc;
     }
     for (int d = 0; d < D; ++d) acc = fmaf(to_f(a[d]), to_f(b[d]), acc);
+    return acc;
+}
+
+// sum_i round(w[i * ws]) * X[t0 + i * ts][d] over `rows` tokens of q / k / v; pad rows
+// (t outside [0, N)) count as zero.  The row index is clamped and the weight
+// zeroed instead of branching, so that the unrolled loop keeps several
+// (independent) loads in flight.
+template <class T>
+__device__ __forceinline__ float weighted_column(const float* w, int ws, const char* base, const long long* st, int e, int h, int t0,
+                                                 int ts, int rows, int N, int d) {
+    const T* x = reinterpret_cast<const T*>(base) + e * st[0] + h * st[1] + d;
+    float acc = 0.f;
+#pragma unroll 4
+    for (int i = 0; i < rows; ++i) {
+        const int t = t0 + i * ts;
+        const bool ok = t >= 0 && t < N;
+        const float xv = to_f(x[static_cast<long long>(ok ? t : 0) * st[2]]);
+        acc = fmaf(ok ? round_to<T>(w[i * ws]) : 0.f, xv, acc);
+    }
     return acc;
 }
 
@@ -120,11 +140,7 @@ __global__ __launch_bounds__(kThreads) void r_step_kernel(Problem P, int TJ, int
     for (int idx = threadIdx.x; idx < rows * D; idx += kThreads) {
         const int jj = idx / D, d = idx % D;
         const float* S = lds + jj * B;
-        float acc = 0.f;
-        for (int i = 0; i < B; ++i) {
-            const TQ* kr = tok_row<TQ>(P.k, P.ks, e, h, m * B + i - P.pad_off, P.N);
-            if (kr) acc = fmaf(round_to<TQ>(S[i]), to_f(kr[d]), acc);
-        }
+        const float acc = weighted_column<TQ>(S, 1, P.k, P.ks, e, h, m * B - P.pad_off, 1, B, P.N, d);
         aL[((eh * B + (j0 + jj)) * M + m) * D + d] = from_f<TQ>(P.sm_scale * round_to<TQ>(acc));
     }
     if (with_v) {
@@ -132,11 +148,7 @@ __global__ __launch_bounds__(kThreads) void r_step_kernel(Problem P, int TJ, int
         for (int idx = threadIdx.x; idx < rows * Dv; idx += kThreads) {
             const int jj = idx / Dv, d = idx % Dv;
             const float* S = lds + jj * B;
-            float acc = 0.f;
-            for (int i = 0; i < B; ++i) {
-                const TV* vr = tok_row<TV>(P.v, P.vs, e, h, m * B + i - P.pad_off, P.N);
-                if (vr) acc = fmaf(round_to<TV>(S[i]), to_f(vr[d]), acc);
-            }
+            const float acc = weighted_column<TV>(S, 1, P.v, P.vs, e, h, m * B - P.pad_off, 1, B, P.N, d);
             Y[((eh * B + (j0 + jj)) * M + m) * static_cast<long long>(Dv) + d] = from_f<TV>(acc);
         }
     }
@@ -224,10 +236,7 @@ __global__ __launch_bounds__(kThreads) void l_accum_kernel(Problem P, int TK) {
             for (int l = 0; l < M; ++l) acc += lds[l * TK + kk];
             P.cR[(eh * M + (k0 + kk)) * B + j] = acc;
         } else {
-            for (int l = 0; l < M; ++l) {
-                const TQ* qr = tok_row<TQ>(P.q, P.qs, e, h, l * B + j - P.pad_off, P.N);
-                if (qr) acc = fmaf(round_to<TQ>(lds[l * TK + kk]), to_f(qr[d]), acc);
-            }
+            acc = weighted_column<TQ>(lds + kk, TK, P.q, P.qs, e, h, j - P.pad_off, B, M, P.N, d);
             aR[((eh * M + (k0 + kk)) * B + j) * D + d] = from_f<TQ>(acc);
         }
     }
@@ -268,6 +277,7 @@ __global__ __launch_bounds__(kThreads) void z_step_kernel(Problem P, int TL) {
         if (t < 0 || t >= P.N) continue;  // padded query rows are dropped (:108)
         const float* U = lds + ll * M;
         float acc = 0.f;
+#pragma unroll 4
         for (int k = 0; k < M; ++k) acc = fmaf(round_to<TV>(U[k]), to_f(Y[k * static_cast<long long>(Dv) + d]), acc);
         out[static_cast<long long>(t) * P.os[2] + d] = from_f<TV>(acc);
     }
