@@ -92,17 +92,37 @@ __device__ __forceinline__ float row16_sum(float x) {
     x += dpp<0x140>(x);
     return x;
 }
-// all-reduce over the four lanes {r, r+16, r+32, r+48}
+// all-reduce over the four lanes {r, r+16, r+32, r+48}: two lane-swap steps on the
+// VALU (v_permlane16_swap exchanges the odd 16-lane rows of its first operand with
+// the even rows of its second, v_permlane32_swap the upper half of the first with
+// the lower half of the second; with both operands holding x the two results are
+// x of the lane's own row pair / half and x of the other one) - no trip through
+// the LDS crossbar as a shuffle would take.  The s_nop covers the wait states the
+// swap needs after a VALU write of its operands.
+__device__ __forceinline__ void swap_rows16(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_halves32(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
 __device__ __forceinline__ float quad_rows_max(float x) {
-    x = fmaxf(x, __shfl_xor(x, 16));
-    x = fmaxf(x, __shfl_xor(x, 32));
-    return x;
+    float a = x, b = x;
+    swap_rows16(a, b);
+    x = fmaxf(a, b);
+    a = x, b = x;
+    swap_halves32(a, b);
+    return fmaxf(a, b);
 }
 __device__ __forceinline__ float quad_rows_sum(float x) {
-    x += __shfl_xor(x, 16);
-    x += __shfl_xor(x, 32);
-    return x;
+    float a = x, b = x;
+    swap_rows16(a, b);
+    x = a + b;
+    a = x, b = x;
+    swap_halves32(a, b);
+    return a + b;
 }
+// 1 / x to 1 ulp (v_rcp_f32) instead of the ten-instruction IEEE division
+__device__ __forceinline__ float rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
 // ---- global memory through buffer resources ---------------------------------
 // Every tensor slice a block problem touches is addressed as (uniform base in
@@ -408,7 +428,7 @@ struct RProb {
             } else {
                 load_state_strip(P, S, xb, cr, m, strip, lane);
             }
-            const float cj = (P.sm_scale * kLog2e) / (cr + P.eps);  // logits in log2 units
+            const float cj = (P.sm_scale * kLog2e) * rcp(cr + P.eps);  // logits in log2 units
 
             f32x4 C[NWT];
 #pragma unroll
@@ -442,7 +462,7 @@ struct RProb {
             sum = quad_rows_sum(sum);
             ent = quad_rows_sum(ent);
             const float den = sum + P.eps;
-            const float inv = 1.0f / den;
+            const float inv = rcp(den);
 #pragma unroll
             for (int wt = 0; wt < NWT; ++wt)
 #pragma unroll
@@ -558,7 +578,7 @@ struct ZProb {
                     sum += p;
                     C[wt][v] = p;
                 }
-            const float inv = 1.0f / quad_rows_sum(sum);
+            const float inv = rcp(quad_rows_sum(sum));
 #pragma unroll
             for (int wt = 0; wt < NWT; ++wt)
 #pragma unroll
@@ -681,7 +701,7 @@ struct LProb {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const float sv = row16_sum(sum[v]);
-                    inv[v] = ((pre.qok >> (4 * si + v)) & 1u) ? 1.0f / sv : 0.f;
+                    inv[v] = ((pre.qok >> (4 * si + v)) & 1u) ? rcp(sv) : 0.f;
                 }
 #pragma unroll
                 for (int kt = 0; kt < NWT; ++kt) {

@@ -191,7 +191,7 @@ struct Resident {
                 for (int ks = 0; ks < KS; ++ks) xb[ks] = lds_row8<T>(xrow + 32 * ks + 8 * q);
                 if (jv) cr = c.cRs[m * B + j];
             }
-            const float cj = (P.sm_scale * kLog2e) / (cr + P.eps);
+            const float cj = (P.sm_scale * kLog2e) * rcp(cr + P.eps);
             f32x4 C[NTB];
 #pragma unroll
             for (int wt = 0; wt < NTB; ++wt) {
@@ -222,7 +222,7 @@ struct Resident {
                 }
             sum = quad_rows_sum(sum);
             ent = quad_rows_sum(ent);
-            const float den = sum + P.eps, inv = 1.0f / den;
+            const float den = sum + P.eps, inv = rcp(den);
 #pragma unroll
             for (int wt = 0; wt < NTB; ++wt)
 #pragma unroll
@@ -307,7 +307,7 @@ struct Resident {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const float s = row16_sum(sum[v]);
-                inv[v] = ((pre.qok >> v) & 1u) ? 1.0f / s : 0.f;   // padded / masked queries are zeroed (ma_torch.py:30)
+                inv[v] = ((pre.qok >> v) & 1u) ? rcp(s) : 0.f;   // padded / masked queries are zeroed (ma_torch.py:30)
             }
 #pragma unroll
             for (int kt = 0; kt < NTM; ++kt) {
@@ -401,7 +401,7 @@ struct Resident {
                     sum += p;
                     C[wt][v] = p;
                 }
-            const float inv = 1.0f / quad_rows_sum(sum);
+            const float inv = rcp(quad_rows_sum(sum));
 #pragma unroll
             for (int wt = 0; wt < NTM; ++wt)
 #pragma unroll

@@ -301,6 +301,25 @@ def test_dead_key_block_gives_no_nan(variant):
     assert_parity(out.cpu(), ref, "f16")
 
 
+@pytest.mark.parametrize("D", [40, 72, 80])
+def test_state_in_lds_ignores_what_earlier_kernels_left_there(D):
+    """Head dims that do not fill their 32-column MFMA tiles (D = 40, 72, 80):
+    the columns between the written width of a state row and the tile width must
+    read as zero whatever used the LDS before - fp32 kernels leave bit patterns
+    there that are NaN as fp16.  Alternates the fp32 kernels with the
+    state-in-LDS kernel on many heads so that every CU has run both."""
+    E, H, N, B, T = 8, 64, 128, 32, 3
+    q, k, v = seeded_qkv(E, H, N, D, torch.float16)
+    ref = monarch_attention_oracle(q[:1, :4], k[:1, :4], v[:1, :4], None, T, B, False, upcast=True)
+    dq, dk, dv = to_dev(q, k, v)
+    big = [t.float() * 3e4 for t in (dq, dk, dv)]   # fp32 run whose LDS contents are large / non-fp16 patterns
+    for _ in range(3):
+        monarch_attention_hip(*big, None, 1, B, False, variant="generic")
+        out = run_hip(dq, dk, dv, None, T, B, False, "resident")
+        assert torch.isfinite(out.float()).all()
+        assert_parity(out[:1, :4].cpu(), ref, "f16")
+
+
 @pytest.mark.parametrize("dt", ["f16", "f32"])
 def test_get_matrix_through_the_module(dt):
     E, H, N, D, B, T = 1, 2, 96, 32, 16, 2
