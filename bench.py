@@ -2,7 +2,7 @@
 """Benchmark of the MonarchAttention forward pass on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cM] [--T 1]
-                    [--variant auto|generic|staged|fused|resident] [--no-cpu] [--no-sdpa] [--no-sweep]
+                    [--variant auto|generic|staged|fused|resident|chained] [--no-cpu] [--no-sdpa] [--no-sweep]
 
 A step is ONE forward call of the hot path (monarch_attention, all T steps)
 through the C ABI on synthetic inputs that are already resident in HBM.  The
@@ -60,7 +60,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--config", default="cM", choices=sorted(CONFIGS))
     ap.add_argument("--T", type=int, default=None, help="override the number of alternating steps")
-    ap.add_argument("--variant", default="auto", choices=["auto", "generic", "staged", "fused", "resident"])
+    ap.add_argument("--variant", default="auto", choices=["auto", "generic", "staged", "fused", "resident", "chained"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sdpa", action="store_true", help="skip the dense SDPA comparison")
     ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep")
@@ -156,8 +156,8 @@ def main():
         if status:
             L.check(status, "stage launch")
 
-    if resolved in ("fused", "resident"):   # the whole forward is one kernel
-        kname = "fused_fwd_mfma" if resolved == "fused" else "resident_fwd_mfma"
+    if resolved in ("fused", "resident", "chained"):   # the whole forward is one kernel
+        kname = {"fused": "fused_fwd_mfma", "resident": "resident_fwd_mfma", "chained": "chain_fwd_mfma"}[resolved]
         kernels[kname] = (event_avg(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), min(args.steps, 200)), cbytes)
     else:
         # per-stage kernels on the state a full forward left in the workspace
@@ -209,7 +209,7 @@ def main():
     if not args.no_sweep:
         sweep = {}
         for T_ in (1, 2, 3):
-            for variant in ("staged", "fused", "resident"):
+            for variant in ("staged", "fused", "chained", "resident"):
                 try:
                     _, ems, _, _ = time_forward(T_, variant, max(50, args.steps // 4), 10)
                 except (NotImplementedError, ValueError):

@@ -44,8 +44,11 @@ typedef enum ma_variant {
     MA_VARIANT_STAGED = 2,  /* MFMA kernels, one launch per half step (2T launches)  */
     MA_VARIANT_FUSED = 3,   /* MFMA, all T steps in ONE launch, teams of workgroups  */
                             /* per head, state exchanged through the workspace       */
-    MA_VARIANT_RESIDENT = 4 /* MFMA, ONE launch, one workgroup per head with the     */
+    MA_VARIANT_RESIDENT = 4,/* MFMA, ONE launch, one workgroup per head with the     */
                             /* whole per-head state resident in LDS (small heads)    */
+    MA_VARIANT_CHAINED = 5  /* MFMA, ONE launch, one workgroup per block problem of  */
+                            /* every phase; a problem starts when its head's         */
+                            /* previous phase has raised its flags in the workspace  */
 } ma_variant;
 
 typedef enum ma_status {
@@ -62,8 +65,8 @@ typedef enum ma_status {
 
 /* ma_fwd_params.flags.  MA_FLAG_SYNC_READY: the caller guarantees that the sync
  * area of the workspace is zero - true after ma_workspace_init() and after every
- * completed ma_fwd() on that workspace (the fused kernel leaves it zeroed).
- * Without the flag the fused variant clears the area with one extra small
+ * completed ma_fwd() on that workspace (the one-launch kernels leave it usable).
+ * Without the flag the FUSED and CHAINED variants clear the area with one extra small
  * launch in front of the forward kernel. */
 #define MA_FLAG_SYNC_READY 1
 
@@ -99,7 +102,7 @@ typedef struct ma_fwd_params {
  * (ma/ma_torch.py:88-104), so a stage can be checked on its own:
  *   aR (E,H,M,B,D) dtype_qk   cR (E,H,M,B) f32   [inputs of the R step]
  *   aL (E,H,B,M,D) dtype_qk   cL (E,H,B,M) f32   Y (E,H,B,M,Dv) dtype_v
- *   stats: scratch of the generic L step; sync: counters of the fused kernel,
+ *   stats: scratch of the generic L step; sync: flags of the one-launch kernels,
  *   always at offset 0 so that it does not move when one workspace serves
  *   calls of different shapes */
 typedef struct ma_ws_layout {
@@ -130,8 +133,8 @@ int ma_fwd_select_variant(const ma_fwd_params* p);
 int ma_fwd(const ma_fwd_params* p, void* stream);
 
 /* One stage on the state held in the workspace (stage-level parity tests;
- * variants GENERIC and STAGED; MA_ERR_UNSUPPORTED for FUSED and RESIDENT, whose
- * stages are phases of a single kernel).
+ * variants GENERIC and STAGED; MA_ERR_UNSUPPORTED for FUSED, RESIDENT and
+ * CHAINED, whose stages are phases of a single kernel).
  *   ma_r_step  replaces al_cl_ref (ma/ma_torch.py:10-23) and, with with_v != 0,
  *              al_y_cl_ref (:38-52).  first != 0: take aR = Q, cR = 1 straight
  *              from q (the state before the first step, :88-89) instead of the

@@ -22,6 +22,9 @@ OBJ_DIR = os.path.join(HERE, "build")
 # fp32 VALU forms are not used by these kernels.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # MFMA results straight into VGPRs: the kernels consume every accumulator on the VALU right
+         # away (softmax, rounding), so AGPR accumulators only add a v_accvgpr_read per value
+         "-mllvm", "-amdgpu-mfma-vgpr-form",
          "-I", os.path.join(ROOT, "include"), "-I", CSRC]
 
 

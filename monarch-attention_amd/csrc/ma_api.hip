@@ -22,7 +22,7 @@ int check_shape(const ma_fwd_params* p) {
     if (p == nullptr) return MA_ERR_NULL;
     if (p->E < 1 || p->H < 1 || p->N < 1 || p->D < 1 || p->Dv < 1 || p->B < 1 || p->T < 1) return MA_ERR_SHAPE;
     if (!dtype_ok(p->dtype_qk) || !dtype_ok(p->dtype_v)) return MA_ERR_DTYPE;
-    if (p->variant < MA_VARIANT_AUTO || p->variant > MA_VARIANT_RESIDENT) return MA_ERR_VARIANT;
+    if (p->variant < MA_VARIANT_AUTO || p->variant > MA_VARIANT_CHAINED) return MA_ERR_VARIANT;
     if (p->flags & ~MA_FLAG_SYNC_READY) return MA_ERR_SHAPE;
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
     const long long Np = M * p->B;
@@ -147,14 +147,17 @@ bool resident_fits(const ma_fwd_params* p) {
 }
 
 // The variant a problem resolves to.  AUTO: the MFMA kernels when the problem
-// qualifies; among them
+// qualifies; among them (measured on MI355X)
 //  * the resident kernel when a head's state fits in LDS and there are enough
 //    heads to occupy the device with one workgroup per head,
-//  * else the team kernel (one launch) when there are enough heads to give every
-//    team several problems per phase (measured: with E*H >= 32 it beats the
-//    per-stage launches; with fewer, larger teams the launch boundaries are
-//    cheaper than its in-kernel barriers),
-//  * else one launch per half step.
+//  * else the chained kernel (one launch) from 32 heads on for blocks and block
+//    counts of at most 64: with many heads the wait of one head's phase is
+//    covered by other heads' problems; with few heads nothing covers it, and with
+//    128-row problems the one kernel is held to the register / LDS needs of its
+//    largest phase, so there
+//  * one launch per half step is the fastest.
+// The team kernel (FUSED) is never chosen automatically: the per-stage launches
+// beat it for few heads and the chained kernel for many.
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
     const long long heads = static_cast<long long>(p->E) * p->H;
@@ -162,11 +165,13 @@ int select_variant(const ma_fwd_params* p) {
         case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
         case MA_VARIANT_STAGED: return fast ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_FUSED: return fast ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_CHAINED: return fast ? MA_VARIANT_CHAINED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_RESIDENT: return fast && resident_fits(p) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
         default:
             if (!fast) return MA_VARIANT_GENERIC;
             if (heads >= 128 && resident_fits(p)) return MA_VARIANT_RESIDENT;
-            return heads >= 32 ? MA_VARIANT_FUSED : MA_VARIANT_STAGED;
+            if (heads >= 32 && p->B <= 64 && (static_cast<long long>(p->N) + p->B - 1) / p->B <= 64) return MA_VARIANT_CHAINED;
+            return MA_VARIANT_STAGED;
     }
 }
 
@@ -187,6 +192,16 @@ int run_fused(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
     if (D <= 64) return h ? launch_fused_f16_d4(pr.P, ready, s) : launch_fused_bf16_d4(pr.P, ready, s);
     if (D <= 80) return h ? launch_fused_f16_d5(pr.P, ready, s) : launch_fused_bf16_d5(pr.P, ready, s);
     return h ? launch_fused_f16_d8(pr.P, ready, s) : launch_fused_bf16_d8(pr.P, ready, s);
+}
+
+int run_chain(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
+    const bool ready = (p->flags & MA_FLAG_SYNC_READY) != 0;
+    const bool h = p->dtype_qk == MA_F16;
+    const int D = p->D;
+    if (D <= 32) return h ? launch_chain_f16_d2(pr.P, ready, s) : launch_chain_bf16_d2(pr.P, ready, s);
+    if (D <= 64) return h ? launch_chain_f16_d4(pr.P, ready, s) : launch_chain_bf16_d4(pr.P, ready, s);
+    if (D <= 80) return h ? launch_chain_f16_d5(pr.P, ready, s) : launch_chain_bf16_d5(pr.P, ready, s);
+    return h ? launch_chain_f16_d8(pr.P, ready, s) : launch_chain_bf16_d8(pr.P, ready, s);
 }
 
 int run_r(const Prepared& pr, const ma_fwd_params* p, bool first, bool with_v, hipStream_t s) {
@@ -276,7 +291,7 @@ int ma_r_step(const ma_fwd_params* p, int first, int with_v, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    if (pr.variant == MA_VARIANT_FUSED || pr.variant == MA_VARIANT_RESIDENT) return MA_ERR_UNSUPPORTED;
+    if (pr.variant != MA_VARIANT_GENERIC && pr.variant != MA_VARIANT_STAGED) return MA_ERR_UNSUPPORTED;
     return run_r(pr, p, first != 0, with_v != 0, static_cast<hipStream_t>(stream));
 }
 
@@ -284,7 +299,7 @@ int ma_l_step(const ma_fwd_params* p, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    if (pr.variant == MA_VARIANT_FUSED || pr.variant == MA_VARIANT_RESIDENT) return MA_ERR_UNSUPPORTED;
+    if (pr.variant != MA_VARIANT_GENERIC && pr.variant != MA_VARIANT_STAGED) return MA_ERR_UNSUPPORTED;
     return run_l(pr, p, static_cast<hipStream_t>(stream));
 }
 
@@ -292,7 +307,7 @@ int ma_z_step(const ma_fwd_params* p, void* stream) {
     Prepared pr;
     const int st = prepare(p, &pr);
     if (st != MA_OK) return st;
-    if (pr.variant == MA_VARIANT_FUSED || pr.variant == MA_VARIANT_RESIDENT) return MA_ERR_UNSUPPORTED;
+    if (pr.variant != MA_VARIANT_GENERIC && pr.variant != MA_VARIANT_STAGED) return MA_ERR_UNSUPPORTED;
     return run_z(pr, p, static_cast<hipStream_t>(stream));
 }
 
@@ -302,6 +317,7 @@ int ma_fwd(const ma_fwd_params* p, void* stream) {
     if (st != MA_OK) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (pr.variant == MA_VARIANT_FUSED) return run_fused(pr, p, s);
+    if (pr.variant == MA_VARIANT_CHAINED) return run_chain(pr, p, s);
     if (pr.variant == MA_VARIANT_RESIDENT) return run_resident(pr.P, p->dtype_qk, false, s);
     for (int t = 0; t < p->T - 1; ++t) {
         st = run_r(pr, p, t == 0, false, s);

@@ -1,0 +1,6 @@
+// Chained forward kernels, f16 operands, head-dim class 2 (D <= 32).
+#include "ma_chain_launch.h"
+
+namespace ma {
+int launch_chain_f16_d2(const Problem& P, bool sync_ready, hipStream_t s) { return mfma::launch_chain<f16, 2>(P, sync_ready, s); }
+}  // namespace ma

@@ -1,0 +1,62 @@
+// Host-side planning and dispatch of the chained forward kernel.  Included by one
+// .hip file per (dtype, head-dim class) so the instantiations compile in parallel.
+#pragma once
+
+#include <type_traits>
+
+#include "ma_chain.h"
+#include "ma_mfma_launch.h"
+
+namespace ma {
+namespace mfma {
+
+template <class T, int DT, int NTB, int NTM>
+int launch_chain_one(const Problem& P, bool sync_ready, hipStream_t s) {
+    constexpr int W = kWaves;
+    using FL = FusedLds<T, DT, NTB, NTM, W>;   // the three kinds of block problems share one LDS allocation
+    if (FL::bytes > 160 * 1024) return MA_ERR_UNSUPPORTED;
+    auto kernel = chain_fwd_mfma<T, DT, NTB, NTM, W>;
+    static const int lds_err = set_lds_limit(kernel, FL::bytes);
+    if (lds_err) return lds_err;
+    const long long heads = static_cast<long long>(P.E) * P.H;
+    ChainPlan pl;
+    pl.hx = static_cast<int>((heads + 7) / 8);
+    pl.tR = (P.M + Split<NTB, W>::PPW - 1) / Split<NTB, W>::PPW;
+    pl.tL = (P.B + Split<NTM, W>::PPW - 1) / Split<NTM, W>::PPW;
+    pl.stride = P.T * (pl.tR + pl.tL) + 1;
+    pl.spin_limit = 1u << 18;   // a legitimate wait lasts one phase of one head (well under a millisecond)
+    // one poll covers 128 flags; the heads' flag words must fit their part of the sync area;
+    // the grid must stay a 31-bit count
+    if (pl.tR > 128 || pl.tL > 128) return MA_ERR_UNSUPPORTED;
+    if (heads * pl.stride > kChainWords) return MA_ERR_UNSUPPORTED;
+    const long long grid = 8ll * pl.hx * P.T * (pl.tR + pl.tL);
+    if (grid > 0x7fffffffll) return MA_ERR_UNSUPPORTED;
+    if (!sync_ready) {
+        const int err = launch_zero_sync(P.sync, s);
+        if (err) return err;
+    }
+    hipLaunchKernelGGL((chain_fwd_mfma<T, DT, NTB, NTM, W>), dim3(static_cast<unsigned>(grid)), dim3(64 * W), FL::bytes, s, P, pl);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <class T, int DT>
+int launch_chain(const Problem& P, bool sync_ready, hipStream_t s) {
+    const int ntb = nt_class(P.B), ntm = nt_class(P.M);
+#define MA_NTM(NB)                                                              \
+    switch (ntm) {                                                              \
+        case 1: return launch_chain_one<T, DT, NB, 1>(P, sync_ready, s);        \
+        case 2: return launch_chain_one<T, DT, NB, 2>(P, sync_ready, s);        \
+        case 4: return launch_chain_one<T, DT, NB, 4>(P, sync_ready, s);        \
+        default: return launch_chain_one<T, DT, NB, 8>(P, sync_ready, s);       \
+    }
+    switch (ntb) {
+        case 1: MA_NTM(1)
+        case 2: MA_NTM(2)
+        case 4: MA_NTM(4)
+        default: MA_NTM(8)
+    }
+#undef MA_NTM
+}
+
+}  // namespace mfma
+}  // namespace ma

@@ -82,7 +82,19 @@ int launch_resident_bf16_d4(const Problem& P, bool dry_run, hipStream_t s);
 int launch_resident_bf16_d5(const Problem& P, bool dry_run, hipStream_t s);
 int launch_resident_bf16_d8(const Problem& P, bool dry_run, hipStream_t s);
 
-constexpr uint64_t kSyncAreaBytes = 4 * (16 + (16 + 3 * 64) * 1024);  // header + one sector per multi-workgroup team
+// Chained forward (one launch, one workgroup per block problem, flags between phases).
+int launch_chain_f16_d2(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_chain_f16_d4(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_chain_f16_d5(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_chain_f16_d8(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_chain_bf16_d2(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_chain_bf16_d4(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_chain_bf16_d5(const Problem& P, bool sync_ready, hipStream_t s);
+int launch_chain_bf16_d8(const Problem& P, bool sync_ready, hipStream_t s);
+
+constexpr uint64_t kTeamSyncBytes = 4 * (16 + (16 + 3 * 64) * 1024);  // header + one sector per multi-workgroup team
+constexpr uint64_t kChainSyncBytes = 4 * 256 * 1024;                  // flag words of the chained kernel
+constexpr uint64_t kSyncAreaBytes = kTeamSyncBytes + kChainSyncBytes;
 // Zero-fills the sync area of a workspace (a small fill kernel, graph-capture safe).
 int launch_zero_sync(unsigned* sync, hipStream_t s);
 

@@ -43,7 +43,7 @@ constexpr int kSyncFlags = 16;     // offset of the flag words inside a team sec
 constexpr int kSyncStride = kSyncFlags + 3 * kMaxTeamSize;  // words per team: base epochs, flags of slot 0 / 1, XCC ids
 constexpr int kMaxTeams = 1024;    // teams of more than one workgroup
 constexpr int kSyncWords = kSyncHeader + kSyncStride * kMaxTeams;
-static_assert(static_cast<uint64_t>(kSyncWords) * 4 == kSyncAreaBytes, "sync area size mismatch");
+static_assert(static_cast<uint64_t>(kSyncWords) * 4 == kTeamSyncBytes, "sync area size mismatch");
 
 template <class T, int DT, int NTB, int NTM, int W>
 struct FusedLds {

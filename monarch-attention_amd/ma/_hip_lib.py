@@ -14,7 +14,7 @@ import threading
 ABI_VERSION = 1
 
 MA_F32, MA_F16, MA_BF16 = 0, 1, 2
-VARIANTS = {"auto": 0, "generic": 1, "staged": 2, "fused": 3, "resident": 4}
+VARIANTS = {"auto": 0, "generic": 1, "staged": 2, "fused": 3, "resident": 4, "chained": 5}
 VARIANT_NAMES = {v: k for k, v in VARIANTS.items()}
 
 MA_OK = 0

@@ -122,7 +122,7 @@ def test_pointer_and_workspace_checks_precede_any_launch():
 def test_select_variant_reports_a_known_variant():
     lib = L.load()
     v = lib.ma_fwd_select_variant(good_params())
-    assert v in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["fused"], L.VARIANTS["resident"])
+    assert v in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["chained"], L.VARIANTS["resident"])
     p32 = good_params(dtype_qk=L.MA_F32, dtype_v=L.MA_F32)
     assert lib.ma_fwd_select_variant(p32) == L.VARIANTS["generic"]
 
@@ -139,8 +139,8 @@ def test_check_maps_status_to_python_exceptions():
 
 def test_auto_variant_policy():
     """AUTO: generic when the MFMA kernels do not apply; resident when a head's
-    state fits in LDS and there are many heads; the team kernel from 32 heads;
-    per-stage launches for a few large heads."""
+    state fits in LDS and there are many heads; the chained kernel from 32 heads
+    for problems of up to 64 rows; per-stage launches otherwise."""
     lib = L.load()
 
     def auto(E, H, N, D, B, dt=L.MA_F16, Dv=None):
@@ -155,8 +155,9 @@ def test_auto_variant_policy():
     assert auto(1, 16, 4096, 64, 64) == "staged"
     assert auto(1, 16, 16384, 64, 128) == "staged"
     assert auto(64, 12, 197, 64, 16) == "resident"
-    assert auto(16, 12, 512, 64, 32) == "fused"        # state of a 512-token head does not fit in LDS
-    assert auto(8, 16, 1024, 72, 32) == "fused"
+    assert auto(16, 12, 512, 64, 32) == "chained"      # state of a 512-token head does not fit in LDS
+    assert auto(8, 16, 1024, 72, 32) == "chained"
+    assert auto(4, 16, 16384, 64, 128) == "staged"      # many heads, but 128-row problems
     assert auto(2, 2, 197, 64, 16) == "staged"          # few heads
     assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "generic"
     assert auto(1, 16, 4096, 64, 64, Dv=128) == "generic"

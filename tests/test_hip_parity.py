@@ -18,7 +18,7 @@ from oracle.ma_oracle import OracleTrace, monarch_attention_oracle, monarch_matr
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-VARIANTS = ["generic", "staged", "fused", "resident", "auto"]
+VARIANTS = ["generic", "staged", "fused", "resident", "chained", "auto"]
 
 
 def run_hip(q, k, v, mask, T, B, pre, variant):
@@ -254,9 +254,39 @@ def test_workspace_is_shared_across_shapes_and_calls():
         for (E, H, N, D, B, T) in shapes:
             q, k, v = seeded_qkv(E, H, N, D, torch.float16)
             ref = monarch_attention_oracle(q, k, v, None, T, B, False, upcast=True)
-            for variant in ("fused", "staged"):
+            for variant in ("fused", "chained", "staged"):
                 out = run_hip(*to_dev(q, k, v), None, T, B, False, variant)
                 assert_parity(out.cpu(), ref, "f16", f"rep{rep}/{variant}/{(E, H, N, B, T)}")
+
+
+@pytest.mark.parametrize("E,H,N,D,B,T", [(1, 16, 1024, 64, 64, 2), (3, 7, 197, 64, 16, 3), (2, 40, 128, 32, 16, 1)])
+def test_chained_kernel_leaves_its_flags_cleared(E, H, N, D, B, T):
+    """Through the C ABI on a caller-owned workspace: after a chained forward
+    every flag word and per-head counter of the kernel is zero again (what
+    MA_FLAG_SYNC_READY promises for the next call), the error word is zero (no
+    wait timed out, every producer ran on its consumers' XCD), and a second call
+    on the same workspace gives the same bits."""
+    lib = L.load()
+    q, k, v = to_dev(*seeded_qkv(E, H, N, D, torch.float16))
+    out = torch.zeros(E, H, N, D, dtype=torch.float16, device=DEV)
+    p = make_params(q, k, v, None, out, T, B, False, "chained")
+    lay = L.WsLayout()
+    L.check(lib.ma_fwd_workspace_layout(p, lay), "layout")
+    ws = torch.zeros(lay.total, dtype=torch.uint8, device=DEV)
+    p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), lay.total, L.MA_FLAG_SYNC_READY
+    sync_bytes = lay.aR - lay.sync                      # the sync area ends where the first state array starts
+    chain_bytes = 4 * 256 * 1024                        # the chained kernel's flag words are its last megabyte
+    outs = []
+    for _ in range(2):
+        L.check(lib.ma_fwd(p, None), "ma_fwd")
+        torch.cuda.synchronize()
+        words = ws[lay.sync:lay.sync + sync_bytes].view(torch.int32)
+        assert int(words[1]) == 0, "sync error word raised"
+        assert not words[-chain_bytes // 4 - 64:].any(), "chained kernel left flags behind"
+        outs.append(out.clone())
+    assert torch.equal(outs[0], outs[1])
+    ref = monarch_attention_oracle(q.cpu(), k.cpu(), v.cpu(), None, T, B, False, upcast=True)
+    assert_parity(outs[0].cpu(), ref, "f16")
 
 
 # ---------------------------------------------------------------- caller-side layouts and masks
@@ -348,7 +378,7 @@ FULL = [  # E, H, N, D, B, T, dt
 ]
 
 
-@pytest.mark.parametrize("variant", ["staged", "fused", "resident", "auto"])
+@pytest.mark.parametrize("variant", ["staged", "fused", "resident", "chained", "auto"])
 @pytest.mark.parametrize("E,H,N,D,B,T,dt", FULL)
 def test_full_size_properties(E, H, N, D, B, T, dt, variant):
     """At the full benchmark sizes: finite output, bit-reproducible, a single
