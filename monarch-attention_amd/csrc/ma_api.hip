@@ -123,7 +123,8 @@ bool mfma_supported(const ma_fwd_params* p) {
     const unsigned long long lim = 0xFFFF0000ull;
     const unsigned long long n1 = static_cast<unsigned long long>(p->N - 1), db = 2ull * p->D;
     if (n1 * p->q_stride[2] * 2 + db >= lim || n1 * p->k_stride[2] * 2 + db >= lim || n1 * p->v_stride[2] * 2 + db >= lim ||
-        n1 * p->out_stride[2] * 2 + db >= lim || static_cast<unsigned long long>(M) * p->B * db >= lim)
+        n1 * p->out_stride[2] * 2 + db >= lim || static_cast<unsigned long long>(M) * p->B * db >= lim ||
+        n1 * static_cast<unsigned long long>(p->mask_stride[1]) >= lim)
         return false;
     return true;
 }

@@ -304,8 +304,8 @@ struct Lds {
 
 // Uniform (per problem) description of the tensors: resources and row pitches in bytes.
 struct Slices {
-    rsrc_t q, k, v, out, aR, cR, aL, cL, Y;
-    unsigned qst, kst, vst, ost;
+    rsrc_t q, k, v, out, aR, cR, aL, cL, Y, mask;
+    unsigned qst, kst, vst, ost, mst;   // mst: byte pitch of the mask row, 0 = no mask
 };
 
 template <class T>
@@ -320,6 +320,8 @@ __device__ __forceinline__ Slices make_slices(const Problem& P, int e, int h, lo
     S.k = make_rsrc(P.k + (e * P.ks[0] + h * P.ks[1]) * static_cast<long long>(sizeof(T)), n1 * S.kst + db);
     S.v = make_rsrc(P.v + (e * P.vs[0] + h * P.vs[1]) * static_cast<long long>(sizeof(T)), n1 * S.vst + db);
     S.out = make_rsrc(P.out + (e * P.os[0] + h * P.os[1]) * static_cast<long long>(sizeof(T)), n1 * S.ost + db);
+    S.mst = P.mask ? static_cast<unsigned>(P.ms[1]) : 0u;
+    S.mask = make_rsrc(P.mask ? P.mask + e * P.ms[0] : nullptr, P.mask ? n1 * S.mst + 1u : 0u);
     const long long np = static_cast<long long>(P.M) * P.B;
     const unsigned state = static_cast<unsigned>(np) * db, stat4 = static_cast<unsigned>(np) * 4u;
     S.aR = make_rsrc(P.aR + wh * np * db, state);
@@ -333,6 +335,19 @@ __device__ __forceinline__ Slices make_slices(const Problem& P, int e, int h, lo
 // byte offset of real token t's row (pitch st) or kOob for a padding position
 __device__ __forceinline__ unsigned tok_off(int t, int N, unsigned st) {
     return static_cast<unsigned>(t) < static_cast<unsigned>(N) ? static_cast<unsigned>(t) * st : kOob;
+}
+
+// Mask byte of token t, started as a load and NOT looked at here (a test would wait for it and
+// for every load issued before it): padding positions and "no mask" read 0 through the bounds
+// check.  token_kept() decodes it once the problem runs.
+__device__ __forceinline__ unsigned mask_load(const Slices& S, const Problem& P, int t, bool want) {
+    if (P.mask == nullptr) return 1u;   // uniform: without a mask nothing is loaded
+    const bool in = want && static_cast<unsigned>(t) < static_cast<unsigned>(P.N);
+    return __builtin_amdgcn_raw_buffer_load_b8(S.mask, in ? static_cast<unsigned>(t) * S.mst : kOob, 0, 0);
+}
+// real (in range) and not masked out
+__device__ __forceinline__ bool token_kept(const Problem& P, int t, unsigned mask_byte) {
+    return static_cast<unsigned>(t) < static_cast<unsigned>(P.N) && (P.mask == nullptr || mask_byte != 0u);
 }
 
 // ============================================================================
@@ -361,7 +376,7 @@ struct RProb {
     struct Pre {
         TileCopy<T, DT, ROWS, WPP * 64> kc, vc;
         V8 xq[G::KS];   // first step: the first strip's Q rows
-        float kb;       // key bias of tile row `tix`
+        unsigned km;    // mask byte of the key token of tile row `tix`
     };
     struct St {
         V8 xa[G::KS];   // later steps: the first strip's aR rows
@@ -380,7 +395,7 @@ struct RProb {
             const int j = 16 * wig + (lane & 15);
             load_x<T, DT, true>(pre.xq, S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, lane >> 4);
         }
-        pre.kb = (tix < B && token_ok(P, e, t0 + tix)) ? 0.f : kNegBig;
+        pre.km = mask_load(S, P, t0 + tix, tix < B);
     }
 
     static __device__ __forceinline__ void load_state_strip(const Problem& P, const Slices& S, V8 (&xa)[G::KS], float& cr, int m,
@@ -410,7 +425,7 @@ struct RProb {
         if (active) {
             pre.kc.commit(Kt, tix);
             if (with_v) pre.vc.commit(Vt, tix);
-            if (tix < ROWS) kbias[tix] = pre.kb;
+            if (tix < ROWS) kbias[tix] = (tix < P.B && token_kept(P, m * P.B - P.pad_off + tix, pre.km)) ? 0.f : kNegBig;
         }
         __syncthreads();
         if (!active) return;
@@ -606,7 +621,7 @@ struct LProb {
     static constexpr int SPW = NWT / WPP;   // strips per wave (2 for blocks counts above 64)
     struct Pre {
         TileCopy<T, DT, ROWS2, nth> qc;   // Q^T tile
-        unsigned qok;                     // bit 4*i + v: query block 16*(wig + i*WPP) + 4q + v is real and unmasked
+        unsigned qm[4 * SPW];             // [4*i + v]: mask byte of the query token of block 16*(wig + i*WPP) + 4q + v
     };
     struct St {
         TileCopy<T, DT, ROWS, nth> ac;    // aL tile
@@ -619,16 +634,13 @@ struct LProb {
         const int B = P.B, M = P.M;
         const int tix = wig * 64 + lane;
         pre.qc.template issue<true>(S.q, P.D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
-        unsigned ok = 0;
 #pragma unroll
         for (int i = 0; i < SPW; ++i)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int l = 16 * (wig + i * WPP) + 4 * (lane >> 4) + v;
-                // padded / masked query tokens are zeroed after the softmax (ma_torch.py:30)
-                if (l < M && token_ok(P, e, l * B + j - P.pad_off)) ok |= 1u << (4 * i + v);
+                pre.qm[4 * i + v] = mask_load(S, P, l * B + j - P.pad_off, l < M);
             }
-        pre.qok = ok;
     }
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
         if (!active) return;
@@ -701,7 +713,9 @@ struct LProb {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const float sv = row16_sum(sum[v]);
-                    inv[v] = ((pre.qok >> (4 * si + v)) & 1u) ? rcp(sv) : 0.f;
+                    // padded / masked query tokens are zeroed after the softmax (ma_torch.py:30)
+                    const int l = l0 + 4 * q + v;
+                    inv[v] = (l < M && token_kept(P, l * B + j - P.pad_off, pre.qm[4 * si + v])) ? rcp(sv) : 0.f;
                 }
 #pragma unroll
                 for (int kt = 0; kt < NWT; ++kt) {

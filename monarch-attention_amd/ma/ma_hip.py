@@ -121,8 +121,13 @@ def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | N
     q, k, v = _inner_contiguous(q), _inner_contiguous(k), _inner_contiguous(v)
     mask_u8 = None
     if attn_mask is not None:
-        # truthiness, as torch.logical_and sees it (ma/ma_torch.py:98)
-        mask_u8 = (attn_mask != 0).to(torch.uint8)
+        # truthiness, as torch.logical_and sees it (ma/ma_torch.py:98).  bool / uint8 / int8 masks
+        # are already one byte per token with "non-zero = keep": the kernels read them in place
+        # (any strides); other dtypes are reduced to bytes by one small elementwise kernel.
+        if attn_mask.dtype in (torch.bool, torch.uint8, torch.int8):
+            mask_u8 = attn_mask.view(torch.uint8)
+        else:
+            mask_u8 = (attn_mask != 0).to(torch.uint8)
     E, H, N, _ = q.shape
     with torch.cuda.device(q.device):
         out = torch.empty((E, H, N, v.shape[-1]), dtype=v.dtype, device=q.device)
