@@ -104,7 +104,10 @@ typedef struct ma_fwd_params {
  *   aL (E,H,B,M,D) dtype_qk   cL (E,H,B,M) f32   Y (E,H,B,M,Dv) dtype_v
  *   stats: scratch of the generic L step; sync: flags of the one-launch kernels,
  *   always at offset 0 so that it does not move when one workspace serves
- *   calls of different shapes */
+ *   calls of different shapes.  Its 32-bit word 1 (byte offset sync + 4) is a
+ *   sticky error word a caller may read after synchronising: 0 = ok, 1 = a
+ *   bounded wait between workgroups ran out (that call's output is invalid),
+ *   2 = the CHAINED kernel met a producer on another XCD than its consumer. */
 typedef struct ma_ws_layout {
     uint64_t aR, cR, aL, cL, Y, stats, sync, total;
 } ma_ws_layout;

@@ -46,6 +46,19 @@ def _workspace(device: torch.device, stream_ptr: int, nbytes: int) -> Tensor:
     return ws
 
 
+def sync_status() -> int:
+    """The sticky error word of the one-launch kernels, over all cached
+    workspaces (synchronises the device): 0 = every wait between workgroups was
+    satisfied; 1 = a bounded wait ran out (results of that call are invalid);
+    2 = a producer ran on another XCD than its consumer (the device does not
+    deal workgroup ids to XCDs the way the chained kernel is built on)."""
+    worst = 0
+    for ws in _WORKSPACES.values():
+        torch.cuda.synchronize(ws.device)
+        worst = max(worst, int(ws[4:8].view(torch.int32).item()))
+    return worst
+
+
 def clear_workspace_cache() -> None:
     """Drop the cached per-stream workspaces (frees their device memory)."""
     _WORKSPACES.clear()

@@ -12,7 +12,7 @@ import torch
 
 from helpers import (DT, assert_parity, block_safe_mask, err_metrics, golden_names, load_golden, seeded_qkv)
 from ma import _hip_lib as L
-from ma.ma_hip import make_params, monarch_attention_hip
+from ma.ma_hip import make_params, monarch_attention_hip, sync_status
 from ma.monarch_attention import MonarchAttention, PadType
 from oracle.ma_oracle import OracleTrace, monarch_attention_oracle, monarch_matrix_oracle
 
@@ -257,6 +257,7 @@ def test_workspace_is_shared_across_shapes_and_calls():
             for variant in ("fused", "chained", "staged"):
                 out = run_hip(*to_dev(q, k, v), None, T, B, False, variant)
                 assert_parity(out.cpu(), ref, "f16", f"rep{rep}/{variant}/{(E, H, N, B, T)}")
+    assert sync_status() == 0   # no wait between workgroups ever ran out
 
 
 @pytest.mark.parametrize("E,H,N,D,B,T", [(1, 16, 1024, 64, 64, 2), (3, 7, 197, 64, 16, 3), (2, 40, 128, 32, 16, 1)])
@@ -401,3 +402,4 @@ def test_full_size_properties(E, H, N, D, B, T, dt, variant):
     sub = slice(0, min(E, 2))
     gen = run_hip(q[sub], k[sub], v[sub], None, T, B, False, "generic")
     assert_parity(out[sub].cpu(), gen.cpu(), dt, "vs generic")
+    assert sync_status() == 0
