@@ -49,7 +49,10 @@ MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
 MEASURED_TRAFFIC_BYTES = {
     ("cM", 1, "r_step(with V)"): 44_188_000,
     ("cM", 1, "z_step"): 33_935_000,
-    ("cM", 1, "fused_fwd_mfma"): 72_430_000,
+    ("cM", 1, "fused_fwd_mfma"): 71_980_000,
+    ("cM", 1, "chain_fwd_mfma"): 70_300_000,
+    ("c3", 2, "chain_fwd_mfma"): 175_100_000,
+    ("c2", 2, "resident_fwd_mfma"): 111_960_000,
 }
 
 
