@@ -30,10 +30,10 @@ _DTYPES = {torch.float32: L.MA_F32, torch.float16: L.MA_F16, torch.bfloat16: L.M
 DEFAULT_VARIANT = "auto"
 
 # One workspace per (device, stream), grown on demand and reused call after
-# call: calls on one stream are ordered, so they can share it, and a reused
-# buffer keeps the intermediate state of the fused kernel resident in L2.  It
-# is allocated zero-filled and every forward call leaves its sync area zeroed,
-# which is what MA_FLAG_SYNC_READY promises to the library.
+# call: calls on one stream are ordered, so they can share it.  It is allocated
+# zero-filled, and every forward call leaves its sync area in the state the next
+# call needs (flags cleared, barrier epochs continuing), which is what
+# MA_FLAG_SYNC_READY promises to the library.
 _WORKSPACES: dict[tuple[int, int], Tensor] = {}
 
 
