@@ -103,6 +103,18 @@ def _inner_contiguous(t: Tensor) -> Tensor:
     return t if t.stride(-1) == 1 or t.shape[-1] == 1 else t.contiguous()
 
 
+def _empty_like_layout(v: Tensor, shape) -> Tensor:
+    """Output buffer in v's memory layout: models pass (E,H,N,D) views of
+    (E,N,H,D) projections (experiments/vit/model.py:73-79) and turn the result
+    back with ``permute(0, 2, 1, 3).contiguous()`` (:99) - with the output backed
+    by an (E,N,H,Dv) buffer that copy is a no-op.  Anything else gets a
+    contiguous (E,H,N,Dv) tensor."""
+    E, H, N, Dv = shape
+    if H > 1 and N > 1 and v.permute(0, 2, 1, 3).is_contiguous() and not v.is_contiguous():
+        return torch.empty((E, N, H, Dv), dtype=v.dtype, device=v.device).permute(0, 2, 1, 3)
+    return torch.empty(shape, dtype=v.dtype, device=v.device)
+
+
 def make_params(q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B: int, pre_pad: bool,
                 variant: str = "auto", eps: float = 1e-12) -> L.FwdParams:
     """Fill a ``ma_fwd_params`` (workspace fields left empty)."""
@@ -128,7 +140,8 @@ def make_params(q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B
 def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, T: int, B: int,
                           pre_pad: bool, *, variant: str | None = None) -> Tensor:
     """MonarchAttention forward on the current HIP stream; returns a new
-    contiguous ``(E, H, N, Dv)`` tensor of ``v.dtype``."""
+    ``(E, H, N, Dv)`` tensor of ``v.dtype`` in v's memory layout (contiguous for
+    contiguous v; backed by ``(E, N, H, Dv)`` when v is such a permuted view)."""
     _check_inputs(q, k, v, attn_mask, T, B)
     lib = L.load()
     q, k, v = _inner_contiguous(q), _inner_contiguous(k), _inner_contiguous(v)
@@ -143,7 +156,7 @@ def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | N
             mask_u8 = (attn_mask != 0).to(torch.uint8)
     E, H, N, _ = q.shape
     with torch.cuda.device(q.device):
-        out = torch.empty((E, H, N, v.shape[-1]), dtype=v.dtype, device=q.device)
+        out = _empty_like_layout(v, (E, H, N, v.shape[-1]))
         p = make_params(q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
         nbytes = lib.ma_fwd_workspace_bytes(p)
         if nbytes == 0:

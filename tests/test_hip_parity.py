@@ -306,6 +306,9 @@ def test_permuted_views_as_models_pass_them(dt, variant):
     out = run_hip(qd, kd, vd, None, T, B, True, variant)
     assert_parity(out.cpu(), ref, dt)
     assert torch.equal(qd.cpu(), q)       # inputs are not modified
+    # the output follows v's layout, so the model's permute(0, 2, 1, 3).contiguous() copies nothing
+    back = out.permute(0, 2, 1, 3)
+    assert back.is_contiguous() and back.contiguous().data_ptr() == out.data_ptr()
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
