@@ -469,7 +469,7 @@ __global__ __launch_bounds__(64 * W) void resident_fwd_mfma(Problem P) {
     for (;;) {
         typename RS::Round nxt = cur;
         const bool more = RS::advance(P, nxt, heads, gridDim.x);
-        typename RS::Pre pn;
+        typename RS::Pre pn = {};   // fully defined before the conditional loads: no merge of an old and a new set
         if (more) RS::issue(P, nxt, pn, c);   // next round's loads fly while this round computes
         RS::execute(P, cur, pc, c);
         if (!more) break;
