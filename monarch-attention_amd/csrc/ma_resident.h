@@ -57,13 +57,37 @@ struct Resident {
     }
 
     // registers that carry one round's global loads from issue to execute
+    // All tile copies are CNT 16-byte chunks per thread, whatever the tile's row count (the
+    // threads of a problem grow with its rows), so the K tile of an R round and the Q^T tile of an
+    // L round share one register array.
+    static constexpr int CH = G::COLS / 8, CNT = CH / 4;
+    static_assert(CH % 4 == 0, "tile rows are whole groups of four 16-byte chunks");
     struct Pre {
-        TileCopy<T, DT, ROWSB, WPB * 64> kc, vc;   // K and V tiles of an R problem
-        TileCopy<T, DT, ROWSM, WPM * 64> qc;       // Q^T tile of an L problem
+        u32x4 a[CNT];                              // R: K tile chunks; L: Q^T tile chunks
+        u32x4 b[CNT];                              // last R: V tile chunks
         V8 xq[KS];                                 // Q rows: first R step / Z step
         float kb;                                  // key bias of staging row `tix` (R)
         unsigned qok;                              // 4 bits: query rows l0 + 4q + v are real and unmasked (L)
     };
+    // start the loads of this thread's chunks of a tile of a problem with `nth` threads: rowoff(row)
+    // is the row's byte offset in `src` or kOob; columns at or beyond D read as zero
+    template <class RowOff>
+    static __device__ __forceinline__ void tile_issue(u32x4 (&val)[CNT], rsrc_t src, int D, RowOff rowoff, int tix, int nth) {
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) {
+            const int c = tix + i * nth;
+            const int row = c / CH, ch = c % CH;
+            const unsigned ro = rowoff(row);
+            val[i] = bload16<true>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
+        }
+    }
+    static __device__ __forceinline__ void tile_commit(T* tile, const u32x4 (&val)[CNT], int tix, int nth) {
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) {
+            const int c = tix + i * nth;
+            *reinterpret_cast<u32x4*>(tile + (c / CH) * LD + (c % CH) * 8) = val[i];
+        }
+    }
 
     struct Round {
         int head;   // E*H fits int32 (validated by the host)
@@ -131,9 +155,9 @@ struct Resident {
             const int m = rd.rnd * PPB + slot;
             if (m >= M) return;
             const int t0 = m * B - P.pad_off;
-            pre.kc.template issue<true>(S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
+            tile_issue(pre.a, S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix, WPB * 64);
             if (rd.p == nph - 2)
-                pre.vc.template issue<true>(S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix);
+                tile_issue(pre.b, S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix, WPB * 64);
             if (rd.p == 0) {
                 const int j = 16 * wig + c.r;
                 load_x<T, DT, true>(pre.xq, S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, c.q);
@@ -147,7 +171,7 @@ struct Resident {
                 const int l = 16 * wig + c.r;
                 load_x<T, DT, true>(pre.xq, S.q, l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob, D, c.q);
             } else {                 // L round: the Q^T tile and the query mask of the strip's rows
-                pre.qc.template issue<true>(S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
+                tile_issue(pre.a, S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix, WPM * 64);
                 unsigned ok = 0;
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
@@ -157,6 +181,15 @@ struct Resident {
                 pre.qok = ok;
             }
         }
+    }
+
+    // Orders the staging writes of a problem's waves before their reads.  A problem that a single
+    // wave owns needs no workgroup barrier for that: the LDS executes one wave's instructions in
+    // order, so only the compiler has to be kept from moving them.
+    template <int WP>
+    static __device__ __forceinline__ void problem_sync() {
+        if constexpr (WP == 1) __builtin_amdgcn_wave_barrier();
+        else __syncthreads();
     }
 
     // ---------------------------------------------------------------- the three kinds of rounds
@@ -172,11 +205,11 @@ struct Resident {
         T* Vt = Kt + ROWSB * LD;
         float* kbias = reinterpret_cast<float*>(Vt + ROWSB * LD);
         if (active) {
-            pre.kc.commit(Kt, tix);
-            if (with_v) pre.vc.commit(Vt, tix);
+            tile_commit(Kt, pre.a, tix, WPB * 64);
+            if (with_v) tile_commit(Vt, pre.b, tix, WPB * 64);
             if (tix < ROWSB) kbias[tix] = pre.kb;
         }
-        __syncthreads();
+        problem_sync<WPB>();
         if (active) {
             const int j = 16 * wig + r;
             const bool jv = j < B;
@@ -262,13 +295,13 @@ struct Resident {
         float* cb = reinterpret_cast<float*>(PT + ROWSM * LDP);
         float* crp = cb + ROWSM;
         if (active) {
-            pre.qc.commit(Qt, tix);
+            tile_commit(Qt, pre.a, tix, WPM * 64);
             if (tix < ROWSM) cb[tix] = tix < M ? -kLog2e * c.cLs[j * M + tix] : kNegBig;
             constexpr int PH = ROWS2M > ROWSM ? ROWS2M - ROWSM : 1;   // phantom query-block columns that phase 2 reads
             if (ROWS2M > ROWSM)
                 for (int i = tix; i < ROWSM * PH; i += WPM * 64) PT[(i / PH) * LDP + ROWSM + i % PH] = from_f<T>(0.f);
         }
-        __syncthreads();
+        problem_sync<WPM>();
         if (active) {
             const int l0 = 16 * wig;
             V8 xa[KS];
@@ -324,7 +357,7 @@ struct Resident {
                 if (q == 0) crp[wig * ROWSM + 16 * kt + r] = s;
             }
         }
-        __syncthreads();
+        problem_sync<WPM>();
         if (active) {
             const int k = 16 * wig + r;   // this wave's tile of key blocks
             const bool kv = k < M;
@@ -367,7 +400,7 @@ struct Resident {
         const int r = c.r, q = c.q;
         float* cb = reinterpret_cast<float*>(c.stage + slot * kSlotL);
         if (active && tix < ROWSM) cb[tix] = tix < M ? -kLog2e * c.cLs[j * M + tix] : kNegBig;
-        __syncthreads();
+        problem_sync<WPM>();
         if (active) {
             const int e = rd.head / P.H, h = rd.head % P.H;
             const Slices S = make_slices<T>(P, e, h, 0);
