@@ -192,6 +192,16 @@ struct Resident {
         else __syncthreads();
     }
 
+    // End of a round.  What a round writes to the state is read in the NEXT phase, and its staging
+    // is reused by the next round: the workgroup barrier is needed after the last round of a phase
+    // and whenever several waves share a problem's staging; single-wave problems in the middle of a
+    // phase run on (their staging accesses are ordered within the wave).
+    template <int WP>
+    static __device__ __forceinline__ void round_end(const Problem& P, const Round& rd) {
+        if (WP > 1 || rd.rnd + 1 == rounds_of(P, rd.p)) __syncthreads();
+        else __builtin_amdgcn_wave_barrier();
+    }
+
     // ---------------------------------------------------------------- the three kinds of rounds
     // R round: al_cl_ref / al_y_cl_ref (ma/ma_torch.py:10-23, :38-52) on the LDS state
     static __device__ __forceinline__ void round_r(const Problem& P, const Round& rd, const Pre& pre, const Ctx& c) {
@@ -279,7 +289,7 @@ struct Resident {
                 if (jv) lds_store_row(c.SY + lrow * LD, O, q);
             }
         }
-        __syncthreads();
+        round_end<WPB>(P, rd);
     }
 
     // L round: ar_cr_ref (ma/ma_torch.py:26-35) on the LDS state
@@ -388,7 +398,7 @@ struct Resident {
                 }
             }
         }
-        __syncthreads();
+        round_end<WPM>(P, rd);
     }
 
     // Z round: z_ref (ma/ma_torch.py:55-62) and the final slice (:106-108)
@@ -457,7 +467,7 @@ struct Resident {
             }
             store_row<T, DT>(S.out, l < M ? tok_off(t, P.N, S.ost) : kOob, D, O, q);   // padded query rows are dropped
         }
-        __syncthreads();
+        round_end<WPM>(P, rd);
     }
 
     static __device__ __forceinline__ void execute(const Problem& P, const Round& rd, const Pre& pre, const Ctx& c) {
