@@ -350,6 +350,16 @@ __device__ __forceinline__ bool token_kept(const Problem& P, int t, unsigned mas
     return static_cast<unsigned>(t) < static_cast<unsigned>(P.N) && (P.mask == nullptr || mask_byte != 0u);
 }
 
+// Orders the LDS tile writes of a problem's waves before their reads.  A problem that a single
+// wave owns (16-row problems) needs no workgroup barrier for that: the LDS executes one wave's
+// instructions in order, so only the compiler has to be kept from moving them.  Every barrier
+// inside a problem body goes through this, so all waves of a workgroup agree on whether they meet.
+template <int WPP>
+__device__ __forceinline__ void problem_sync() {
+    if constexpr (WPP == 1) __builtin_amdgcn_wave_barrier();
+    else __syncthreads();
+}
+
 // ============================================================================
 // The three block problems.  Each is split in three parts so that a caller can
 // overlap memory latency with other work:
@@ -427,7 +437,7 @@ struct RProb {
             if (with_v) pre.vc.commit(Vt, tix);
             if (tix < ROWS) kbias[tix] = (tix < P.B && token_kept(P, m * P.B - P.pad_off + tix, pre.km)) ? 0.f : kNegBig;
         }
-        __syncthreads();
+        problem_sync<WPP>();
         if (!active) return;
         for (int strip = wig; strip < NWT; strip += WPP) {
             const int j = 16 * strip + r;
@@ -554,7 +564,7 @@ struct ZProb {
             st.yc.commit(Yt, tix);
             if (tix < ROWS) cb[tix] = st.cbv;
         }
-        __syncthreads();
+        problem_sync<WPP>();
         if (!active) return;
         for (int strip = wig; strip < NWT; strip += WPP) {
             const int l = 16 * strip + r;
@@ -670,7 +680,7 @@ struct LProb {
             if (ROWS2 > ROWS)
                 for (int i = tix; i < ROWS * PH; i += nth) PT[(i / PH) * LDP + ROWS + i % PH] = from_f<T>(0.f);
         }
-        __syncthreads();
+        problem_sync<WPP>();
         if (active) {
             // phase 1: L[l, k] for 16-row strips of l; lane holds column k = 16kt + r, rows l0 + 4q + v
             float crsum[NWT];
@@ -737,7 +747,7 @@ struct LProb {
                 if (q == 0) crp[wig * ROWS + 16 * kt + r] = sv;
             }
         }
-        __syncthreads();
+        problem_sync<WPP>();
         if (active) {
             // phase 2: aR[k, :] = sum_l round(L[l,k]) Qt[l, :] for 16-wide tiles of k
             for (int kt = wig; kt < NWT; kt += WPP) {

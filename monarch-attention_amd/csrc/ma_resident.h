@@ -183,15 +183,6 @@ struct Resident {
         }
     }
 
-    // Orders the staging writes of a problem's waves before their reads.  A problem that a single
-    // wave owns needs no workgroup barrier for that: the LDS executes one wave's instructions in
-    // order, so only the compiler has to be kept from moving them.
-    template <int WP>
-    static __device__ __forceinline__ void problem_sync() {
-        if constexpr (WP == 1) __builtin_amdgcn_wave_barrier();
-        else __syncthreads();
-    }
-
     // End of a round.  What a round writes to the state is read in the NEXT phase, and its staging
     // is reused by the next round: the workgroup barrier is needed after the last round of a phase
     // and whenever several waves share a problem's staging; single-wave problems in the middle of a
