@@ -382,15 +382,16 @@ struct RProb {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
     static constexpr int WPP = Split<NWT>::WPP;
+    static constexpr int SPW = NWT / WPP;   // strips per wave: 2 for blocks of more than 64 rows (strip = wig + i * WPP)
     static constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
     struct Pre {
         TileCopy<T, DT, ROWS, WPP * 64> kc, vc;
-        V8 xq[G::KS];   // first step: the first strip's Q rows
-        unsigned km;    // mask byte of the key token of tile row `tix`
+        V8 xq[SPW][G::KS];   // first step: the Q rows of this wave's strips
+        unsigned km;         // mask byte of the key token of tile row `tix`
     };
     struct St {
-        V8 xa[G::KS];   // later steps: the first strip's aR rows
-        float cr;
+        V8 xa[SPW][G::KS];   // later steps: the aR rows of this wave's strips
+        float cr[SPW];
     };
 
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int e, int m, bool first,
@@ -402,8 +403,11 @@ struct RProb {
         pre.kc.template issue<true>(S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
         if (with_v) pre.vc.template issue<true>(S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix);
         if (first) {
-            const int j = 16 * wig + (lane & 15);
-            load_x<T, DT, true>(pre.xq, S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, lane >> 4);
+#pragma unroll
+            for (int i = 0; i < SPW; ++i) {
+                const int j = 16 * (wig + i * WPP) + (lane & 15);
+                load_x<T, DT, true>(pre.xq[i], S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, lane >> 4);
+            }
         }
         pre.km = mask_load(S, P, t0 + tix, tix < B);
     }
@@ -419,8 +423,11 @@ struct RProb {
 
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int m, bool first, int wig,
                                                  int lane) {
-        st.cr = 1.0f;
-        if (active && !first) load_state_strip(P, S, st.xa, st.cr, m, wig, lane);
+#pragma unroll
+        for (int i = 0; i < SPW; ++i) {
+            st.cr[i] = 1.0f;
+            if (active && !first) load_state_strip(P, S, st.xa[i], st.cr[i], m, wig + i * WPP, lane);
+        }
     }
 
     static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
@@ -439,20 +446,15 @@ struct RProb {
         }
         problem_sync<WPP>();
         if (!active) return;
-        for (int strip = wig; strip < NWT; strip += WPP) {
+#pragma unroll
+        for (int si = 0; si < SPW; ++si) {
+            const int strip = wig + si * WPP;
             const int j = 16 * strip + r;
             const bool jv = j < B;
             V8 xb[G::KS];
-            float cr = 1.0f;
-            if (strip == wig) {
 #pragma unroll
-                for (int ks = 0; ks < G::KS; ++ks) xb[ks] = first ? pre.xq[ks] : st.xa[ks];
-                cr = st.cr;
-            } else if (first) {   // blocks of more than 64 rows: a second strip per wave
-                load_x<T, DT, true>(xb, S.q, jv ? tok_off(m * B + j - P.pad_off, P.N, S.qst) : kOob, D, q);
-            } else {
-                load_state_strip(P, S, xb, cr, m, strip, lane);
-            }
+            for (int ks = 0; ks < G::KS; ++ks) xb[ks] = first ? pre.xq[si][ks] : st.xa[si][ks];
+            const float cr = st.cr[si];
             const float cj = (P.sm_scale * kLog2e) * rcp(cr + P.eps);  // logits in log2 units
 
             f32x4 C[NWT];
@@ -526,8 +528,9 @@ struct ZProb {
     using V8 = typename Ops<T>::v8;
     static constexpr int WPP = Split<NWT>::WPP;
     static constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
+    static constexpr int SPW = NWT / WPP;   // strips per wave (strip = wig + i * WPP)
     struct Pre {
-        V8 xq[G::KS];   // the first strip's Q rows
+        V8 xq[SPW][G::KS];   // the Q rows of this wave's strips
     };
     struct St {
         TileCopy<T, DT, ROWS, WPP * 64> ac, yc;
@@ -539,7 +542,9 @@ struct ZProb {
         load_x<T, DT, true>(xb, S.q, l < P.M ? tok_off(l * P.B + j - P.pad_off, P.N, S.qst) : kOob, P.D, lane >> 4);
     }
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int j, int wig, int lane) {
-        if (active) load_strip(P, S, pre.xq, j, wig, lane);
+        if (!active) return;
+#pragma unroll
+        for (int i = 0; i < SPW; ++i) load_strip(P, S, pre.xq[i], j, wig + i * WPP, lane);
     }
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
         if (!active) return;
@@ -566,17 +571,15 @@ struct ZProb {
         }
         problem_sync<WPP>();
         if (!active) return;
-        for (int strip = wig; strip < NWT; strip += WPP) {
+#pragma unroll
+        for (int si = 0; si < SPW; ++si) {
+            const int strip = wig + si * WPP;
             const int l = 16 * strip + r;
             const int t = l * B + j - P.pad_off;
             const bool lv = l < M;
             V8 xb[G::KS];
-            if (strip == wig) {
 #pragma unroll
-                for (int ks = 0; ks < G::KS; ++ks) xb[ks] = pre.xq[ks];
-            } else {
-                load_strip(P, S, xb, j, strip, lane);
-            }
+            for (int ks = 0; ks < G::KS; ++ks) xb[ks] = pre.xq[si][ks];
             f32x4 C[NWT];
 #pragma unroll
             for (int wt = 0; wt < NWT; ++wt) {
