@@ -4,7 +4,7 @@
 // first step to the last.  Nothing but Q, K, V is read from memory and nothing
 // but the output is written: the state never leaves the compute unit.
 //
-// It applies when the state fits: three Np x D tiles (aL, aR, Y) plus the
+// It applies when the state fits: two or three Np x D tiles (aL, aR, Y) plus the
 // operand staging of the problems in flight within the 160 KB of LDS, i.e. heads
 // of up to ~256 padded tokens at D = 64, and blocks / block counts of at most 64.
 //
@@ -21,7 +21,8 @@
 // State layout in LDS (row pitch LD, like the operand tiles):
 //   SA  aL rows (j, m) -> j*M + m      read as the "aL[j]" tile of the L / Z problems
 //   SX  aR rows (m, j) -> m*B + j      read as the "aR[m]" rows of the R problems
-//   SY  Y  rows (j, m) -> j*M + m      read (transposed) by the Z problems
+//   SY  Y  rows (j, m) -> j*M + m      read (transposed) by the Z problems; in aR's place when
+//       the last R phase is a single round (see y_on_x), else a tile of its own
 //   cLs[j*M + m], cRs[m*B + j] (fp32), ZR: one row of zeros that stands in for
 //   rows beyond the tile tails (k >= M, j >= B).
 #pragma once
@@ -46,14 +47,19 @@ struct Resident {
     static constexpr size_t kStageL = (ROWSM * LD + ROWSM * LDP) * sizeof(T) + (1 + WPM) * ROWSM * sizeof(float);
     static constexpr size_t kSlotR = (kStageR + 15) / 16 * 16, kSlotL = (kStageL + 15) / 16 * 16;
 
-    static __host__ __device__ size_t state_bytes(int Np) {   // SA, SX, SY, ZR, cLs, cRs
+    // Y is written by the last R phase, which is also the last reader of aR.  When that phase is
+    // a single round (all its block problems run at once) its waves read their aR rows first, meet
+    // at a barrier, and only then write Y - so Y can take aR's place and the state is two tiles.
+    // It costs that barrier, so it is only used where three tiles do not fit (the launcher decides).
+    static __host__ __device__ bool y_on_x_possible(int M) { return M <= PPB; }
+    static __host__ __device__ size_t state_bytes(int Np, bool y_on_x) {   // SA, SX, (SY,) ZR, cLs, cRs
         const size_t np4 = (static_cast<size_t>(Np) + 3) / 4 * 4;
-        return (3 * static_cast<size_t>(Np) + 1) * LD * sizeof(T) + 2 * np4 * sizeof(float);
+        return ((y_on_x ? 2 : 3) * static_cast<size_t>(Np) + 1) * LD * sizeof(T) + 2 * np4 * sizeof(float);
     }
     // staging is only needed for the problems a round can actually hold
-    static __host__ __device__ size_t lds_bytes(int Np, int M, int B) {
+    static __host__ __device__ size_t lds_bytes(int Np, int M, int B, bool y_on_x) {
         const size_t sr = static_cast<size_t>(M < PPB ? M : PPB) * kSlotR, sl = static_cast<size_t>(B < PPM ? B : PPM) * kSlotL;
-        return state_bytes(Np) + (sr > sl ? sr : sl);
+        return state_bytes(Np, y_on_x) + (sr > sl ? sr : sl);
     }
 
     // registers that carry one round's global loads from issue to execute
@@ -99,6 +105,7 @@ struct Resident {
         float *cLs, *cRs;
         char* stage;
         int wave, lane, r, q;
+        bool y_on_x;   // Y shares the LDS of aR
     };
 
     static __device__ __forceinline__ int rounds_of(const Problem& P, int p) {
@@ -211,11 +218,11 @@ struct Resident {
             if (tix < ROWSB) kbias[tix] = pre.kb;
         }
         problem_sync<WPB>();
+        const int j = 16 * wig + r;
+        const bool jv = j < B;
+        V8 xb[KS];
+        float cr = 1.0f;
         if (active) {
-            const int j = 16 * wig + r;
-            const bool jv = j < B;
-            V8 xb[KS];
-            float cr = 1.0f;
             if (first) {
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) xb[ks] = pre.xq[ks];
@@ -225,6 +232,11 @@ struct Resident {
                 for (int ks = 0; ks < KS; ++ks) xb[ks] = lds_row8<T>(xrow + 32 * ks + 8 * q);
                 if (jv) cr = c.cRs[m * B + j];
             }
+        }
+        // Y takes the place of aR (see the kernel): every wave has read its aR rows before any
+        // wave writes Y rows.  Uniform condition; the barrier also waits for the reads' data.
+        if (c.y_on_x && with_v && !first) __syncthreads();
+        if (active) {
             const float cj = (P.sm_scale * kLog2e) * rcp(cr + P.eps);
             f32x4 C[NTB];
 #pragma unroll
@@ -469,18 +481,20 @@ struct Resident {
 };
 
 template <class T, int DT, int NTB, int NTM, int W>
-__global__ __launch_bounds__(64 * W) void resident_fwd_mfma(Problem P) {
+__global__ __launch_bounds__(64 * W) void resident_fwd_mfma(Problem P, int y_on_x) {
     using RS = Resident<T, DT, NTB, NTM, W>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int Np = P.M * P.B;
     typename RS::Ctx c;
     c.SA = reinterpret_cast<T*>(smem);
+    c.y_on_x = y_on_x != 0;
+    const int tiles = c.y_on_x ? 2 : 3;
     c.SX = c.SA + Np * RS::LD;
-    c.SY = c.SX + Np * RS::LD;
-    c.ZR = c.SY + Np * RS::LD;
+    c.SY = c.y_on_x ? c.SX : c.SX + Np * RS::LD;
+    c.ZR = c.SA + tiles * Np * RS::LD;
     c.cLs = reinterpret_cast<float*>(c.ZR + RS::LD);
     c.cRs = c.cLs + (Np + 3) / 4 * 4;
-    c.stage = smem + RS::state_bytes(Np);
+    c.stage = smem + RS::state_bytes(Np, c.y_on_x);
     c.wave = wave_id();
     c.lane = threadIdx.x & 63;
     c.r = c.lane & 15;
@@ -491,7 +505,7 @@ __global__ __launch_bounds__(64 * W) void resident_fwd_mfma(Problem P) {
     // written and must not hold leftovers (0 * NaN) of whatever used the LDS before.
     if constexpr (16 * DT < 32 * RS::KS) {
         constexpr int kTail = 32 * RS::KS - 16 * DT;
-        for (int i = threadIdx.x; i < 3 * Np * kTail; i += 64 * W) c.SA[(i / kTail) * RS::LD + 16 * DT + i % kTail] = from_f<T>(0.f);
+        for (int i = threadIdx.x; i < tiles * Np * kTail; i += 64 * W) c.SA[(i / kTail) * RS::LD + 16 * DT + i % kTail] = from_f<T>(0.f);
     }
     __syncthreads();
 

@@ -18,7 +18,13 @@ template <class T, int DT, int NTB, int NTM, int W>
 int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
     using RS = Resident<T, DT, NTB, NTM, W>;
     const int Np = P.M * P.B;
-    const size_t lds = RS::lds_bytes(Np, P.M, P.B);
+    // Y in a tile of its own if that fits, else in aR's place where the kernel allows it
+    bool y_on_x = false;
+    size_t lds = RS::lds_bytes(Np, P.M, P.B, false);
+    if (lds > kLdsPerCu && RS::y_on_x_possible(P.M)) {
+        y_on_x = true;
+        lds = RS::lds_bytes(Np, P.M, P.B, true);
+    }
     if (lds > kLdsPerCu) return MA_ERR_UNSUPPORTED;   // the head's state does not fit in LDS
     if (dry_run) return MA_OK;
     auto kernel = resident_fwd_mfma<T, DT, NTB, NTM, W>;
@@ -41,7 +47,7 @@ int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
     const long long per_cu = lds * 2 <= kLdsPerCu ? 2 : 1;
     long long grid = caps.cus * per_cu;
     if (grid > heads) grid = heads;
-    hipLaunchKernelGGL((resident_fwd_mfma<T, DT, NTB, NTM, W>), dim3(grid), dim3(64 * W), lds, s, P);
+    hipLaunchKernelGGL((resident_fwd_mfma<T, DT, NTB, NTM, W>), dim3(grid), dim3(64 * W), lds, s, P, y_on_x ? 1 : 0);
     return static_cast<int>(hipGetLastError());
 }
 
