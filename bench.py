@@ -52,7 +52,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("cM", 1, "fused_fwd_mfma"): 71_980_000,
     ("cM", 1, "chain_fwd_mfma"): 70_300_000,
     ("c3", 2, "chain_fwd_mfma"): 175_100_000,
-    ("c2", 2, "resident_fwd_mfma"): 111_960_000,
+    ("c2", 2, "resident_fwd_mfma"): 102_330_000,
 }
 
 
