@@ -74,25 +74,26 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
     __shared__ int same_xcd;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int nph = 2 * P.T;
-    const long long heads = static_cast<long long>(P.E) * P.H;
+    const int heads = P.E * P.H;   // E * H * Np fits int32 (validated by the host)
 
     // task of this workgroup: phases in grid order, heads of this XCD, tasks of the head
-    const int xcd = blockIdx.x & 7, ix = blockIdx.x >> 3;
-    const int perR = plan.hx * plan.tR, perL = plan.hx * plan.tL;
-    const int step = ix / (perR + perL), rem = ix % (perR + perL);
+    const unsigned xcd = blockIdx.x & 7, ix = blockIdx.x >> 3;
+    const unsigned perR = plan.hx * plan.tR, perL = plan.hx * plan.tL;
+    const unsigned step = ix / (perR + perL), rem = ix % (perR + perL);
     const bool odd = rem >= perR;
     const int p = 2 * step + (odd ? 1 : 0);
-    const int tasks = odd ? plan.tL : plan.tR;
-    const int idx = odd ? rem - perR : rem;
-    const long long head = xcd + 8ll * (idx / tasks);
+    const unsigned tasks = odd ? plan.tL : plan.tR;
+    const unsigned idx = odd ? rem - perR : rem;
+    const int head = xcd + 8 * (idx / tasks);
     const int task = idx % tasks;
     if (p >= nph || head >= heads) return;
-    const int e = static_cast<int>(head / P.H), h = static_cast<int>(head % P.H);
+    const int e = static_cast<unsigned>(head) / static_cast<unsigned>(P.H), h = static_cast<unsigned>(head) % static_cast<unsigned>(P.H);
 
-    unsigned* flags = P.sync + kSyncWords + head * plan.stride;   // this head's flag words, phase after phase
+    unsigned* flags = P.sync + kSyncWords + static_cast<size_t>(head) * plan.stride;   // this head's flag words, phase after phase
     unsigned* error = P.sync + 1;
-    const int off = step * (plan.tR + plan.tL) + (odd ? plan.tR : 0);                    // this phase's flags
-    const int prev_off = odd ? step * (plan.tR + plan.tL) : (step - 1) * (plan.tR + plan.tL) + plan.tR;
+    const int per_step = plan.tR + plan.tL, st = static_cast<int>(step);
+    const int off = st * per_step + (odd ? plan.tR : 0);                    // this phase's flags
+    const int prev_off = odd ? st * per_step : (st - 1) * per_step + plan.tR;   // only used for p > 0
     const int prev_count = odd ? plan.tR : plan.tL;
     const unsigned my_xcc = xcc_id();
 

@@ -823,14 +823,16 @@ __global__ __launch_bounds__(kThreads) void r_step_mfma(Problem P, int first, in
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
-    const long long total = static_cast<long long>(P.E) * P.H * P.M;
-    long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;
+    // E * H * Np fits int32 (validated by the host), so all problem indices are 32-bit
+    const unsigned total = static_cast<unsigned>(P.E) * P.H * P.M;
+    unsigned pid = blockIdx.x * PPW + slot;
     const bool active = pid < total;
     if (!active) pid = 0;
-    const int m = pid % P.M;
-    const int h = (pid / P.M) % P.H;
-    const int e = pid / (static_cast<long long>(P.M) * P.H);
-    r_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::R, active, e, h, static_cast<long long>(e) * P.H + h, m, first != 0,
+    const int m = pid % static_cast<unsigned>(P.M);
+    const unsigned eh = pid / static_cast<unsigned>(P.M);
+    const int h = eh % static_cast<unsigned>(P.H);
+    const int e = eh / static_cast<unsigned>(P.H);
+    r_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::R, active, e, h, static_cast<long long>(eh), m, first != 0,
                           with_v != 0, wig, lane);
 }
 
@@ -840,14 +842,15 @@ __global__ __launch_bounds__(kThreads) void l_step_mfma(Problem P) {
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
-    const long long total = static_cast<long long>(P.E) * P.H * P.B;
-    long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;
+    const unsigned total = static_cast<unsigned>(P.E) * P.H * P.B;
+    unsigned pid = blockIdx.x * PPW + slot;
     const bool active = pid < total;
     if (!active) pid = 0;
-    const int j = pid % P.B;
-    const int h = (pid / P.B) % P.H;
-    const int e = pid / (static_cast<long long>(P.B) * P.H);
-    l_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::L, active, e, h, static_cast<long long>(e) * P.H + h, j, wig, lane);
+    const int j = pid % static_cast<unsigned>(P.B);
+    const unsigned eh = pid / static_cast<unsigned>(P.B);
+    const int h = eh % static_cast<unsigned>(P.H);
+    const int e = eh / static_cast<unsigned>(P.H);
+    l_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::L, active, e, h, static_cast<long long>(eh), j, wig, lane);
 }
 
 template <class T, int DT, int NWT>
@@ -856,14 +859,15 @@ __global__ __launch_bounds__(kThreads) void z_step_mfma(Problem P) {
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
-    const long long total = static_cast<long long>(P.E) * P.H * P.B;
-    long long pid = static_cast<long long>(blockIdx.x) * PPW + slot;
+    const unsigned total = static_cast<unsigned>(P.E) * P.H * P.B;
+    unsigned pid = blockIdx.x * PPW + slot;
     const bool active = pid < total;
     if (!active) pid = 0;
-    const int j = pid % P.B;
-    const int h = (pid / P.B) % P.H;
-    const int e = pid / (static_cast<long long>(P.B) * P.H);
-    z_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::Z, active, e, h, static_cast<long long>(e) * P.H + h, j, wig, lane);
+    const int j = pid % static_cast<unsigned>(P.B);
+    const unsigned eh = pid / static_cast<unsigned>(P.B);
+    const int h = eh % static_cast<unsigned>(P.H);
+    const int e = eh / static_cast<unsigned>(P.H);
+    z_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::Z, active, e, h, static_cast<long long>(eh), j, wig, lane);
 }
 
 }  // namespace mfma
