@@ -69,8 +69,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build measures ONE GPU (heads are independent; see DESIGN.md for how the path "
-                 "would shard) - run with --gpus 1")
+        sys.exit("bench.py: this build measures ONE GPU (heads are independent problems: more GPUs would each take "
+                 "a share of E*H with no communication) - run with --gpus 1")
 
     import torch
 
