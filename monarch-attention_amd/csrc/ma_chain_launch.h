@@ -16,7 +16,7 @@ int launch_chain_one(const Problem& P, bool sync_ready, hipStream_t s) {
     using FL = FusedLds<T, DT, NTB, NTM, W>;   // the three kinds of block problems share one LDS allocation
     if (FL::bytes > 160 * 1024) return MA_ERR_UNSUPPORTED;
     auto kernel = chain_fwd_mfma<T, DT, NTB, NTM, W>;
-    static const int lds_err = set_lds_limit(kernel, FL::bytes);
+    const int lds_err = set_lds_limit(kernel, FL::bytes);
     if (lds_err) return lds_err;
     const long long heads = static_cast<long long>(P.E) * P.H;
     ChainPlan pl;

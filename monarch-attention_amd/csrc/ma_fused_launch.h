@@ -41,9 +41,10 @@ int launch_fused_w(const Problem& P, bool sync_ready, hipStream_t s) {
     struct Caps {
         int err = 0, capacity = 0;
     };
+    const int lds_err = set_lds_limit(kernel, FL::bytes);
+    if (lds_err) return lds_err;
     static const Caps caps = [&] {
         Caps c;
-        c.err = set_lds_limit(kernel, FL::bytes);
         int dev = 0, cus = 0, per_cu = 0;
         if (!c.err) c.err = static_cast<int>(hipGetDevice(&dev));
         if (!c.err) c.err = static_cast<int>(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));

@@ -3,6 +3,9 @@
 // instantiations compile in parallel.
 #pragma once
 
+#include <map>
+#include <mutex>
+
 #include "ma_mfma.h"
 
 namespace ma {
@@ -14,10 +17,24 @@ inline int nt_class(int n) {
     return t <= 1 ? 1 : t <= 2 ? 2 : t <= 4 ? 4 : 8;
 }
 
+// Raises a kernel's dynamic-LDS limit to `bytes`, once per (kernel, device): the attribute belongs
+// to the device's copy of the code object, so a process that drives several devices needs it on
+// each of them.  Returns 0 or a hipError_t.
 template <class K>
 int set_lds_limit(K kernel, size_t bytes) {
-    return static_cast<int>(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+    static std::mutex mu;
+    static std::map<const void*, unsigned> done;   // kernel -> bit d set: limit raised on device d
+    int dev = 0;
+    const hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return static_cast<int>(err);
+    const void* key = reinterpret_cast<const void*>(kernel);
+    const unsigned bit = 1u << (dev & 31);
+    std::lock_guard<std::mutex> lock(mu);
+    unsigned& mask = done[key];
+    if (mask & bit) return 0;
+    const int rc = static_cast<int>(hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+    if (rc == 0) mask |= bit;
+    return rc;
 }
 
 // calls f(dt_tag, nt_tag) with integral_constant tags for the problem's classes
@@ -45,7 +62,7 @@ int launch_r(const Problem& P, bool first, bool with_v, hipStream_t s) {
         constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
         constexpr int PPW = Split<NWT>::PPW;
         constexpr size_t lds = PPW * Lds<T, DT, NWT>::R;
-        static const int attr = set_lds_limit(r_step_mfma<T, DT, NWT>, lds);
+        const int attr = set_lds_limit(r_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
         const long long problems = static_cast<long long>(P.E) * P.H * P.M;
         hipLaunchKernelGGL((r_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P,
@@ -60,7 +77,7 @@ int launch_l(const Problem& P, hipStream_t s) {
         constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
         constexpr int PPW = Split<NWT>::PPW;
         constexpr size_t lds = PPW * Lds<T, DT, NWT>::L;
-        static const int attr = set_lds_limit(l_step_mfma<T, DT, NWT>, lds);
+        const int attr = set_lds_limit(l_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
         const long long problems = static_cast<long long>(P.E) * P.H * P.B;
         hipLaunchKernelGGL((l_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P);
@@ -74,7 +91,7 @@ int launch_z(const Problem& P, hipStream_t s) {
         constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
         constexpr int PPW = Split<NWT>::PPW;
         constexpr size_t lds = PPW * Lds<T, DT, NWT>::Z;
-        static const int attr = set_lds_limit(z_step_mfma<T, DT, NWT>, lds);
+        const int attr = set_lds_limit(z_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
         const long long problems = static_cast<long long>(P.E) * P.H * P.B;
         hipLaunchKernelGGL((z_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P);

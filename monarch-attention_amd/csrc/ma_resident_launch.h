@@ -31,9 +31,10 @@ int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
     struct Caps {
         int err = 0, cus = 0;
     };
+    const int lds_err = set_lds_limit(kernel, kLdsPerCu);
+    if (lds_err) return lds_err;
     static const Caps caps = [&] {
         Caps c;
-        c.err = set_lds_limit(kernel, kLdsPerCu);
         int dev = 0;
         if (!c.err) c.err = static_cast<int>(hipGetDevice(&dev));
         if (!c.err) c.err = static_cast<int>(hipDeviceGetAttribute(&c.cus, hipDeviceAttributeMultiprocessorCount, dev));
