@@ -129,6 +129,27 @@ bool mfma_supported(const ma_fwd_params* p) {
     return true;
 }
 
+// What the fp32 MFMA stage kernels need: fp32 q, k, v, Dv == D, 16-byte row chunks (D % 4 == 0,
+// every row start 16-byte aligned), block problems within the tiles and the LDS.
+bool mfma32_supported(const ma_fwd_params* p) {
+    if (p->dtype_qk != MA_F32 || p->dtype_v != MA_F32) return false;
+    if (p->Dv != p->D || p->D % 4 != 0 || p->D > 128) return false;
+    const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+    if (p->B > 128 || M > 128) return false;
+    for (int i = 0; i < 3; ++i)
+        if (p->q_stride[i] % 4 || p->k_stride[i] % 4 || p->v_stride[i] % 4 || p->out_stride[i] % 4) return false;
+    if (reinterpret_cast<uintptr_t>(p->q) % 16 || reinterpret_cast<uintptr_t>(p->k) % 16 ||
+        reinterpret_cast<uintptr_t>(p->v) % 16 || reinterpret_cast<uintptr_t>(p->out) % 16)
+        return false;
+    const unsigned long long lim = 0xFFFF0000ull;
+    const unsigned long long n1 = static_cast<unsigned long long>(p->N - 1), db = 4ull * p->D;
+    if (n1 * p->q_stride[2] * 4 + db >= lim || n1 * p->k_stride[2] * 4 + db >= lim || n1 * p->v_stride[2] * 4 + db >= lim ||
+        n1 * p->out_stride[2] * 4 + db >= lim || static_cast<unsigned long long>(M) * p->B * db >= lim ||
+        n1 * static_cast<unsigned long long>(p->mask_stride[1]) >= lim)
+        return false;
+    return mfma32_lds_needed(p->D, p->B, static_cast<int>(M)) <= 160 * 1024;
+}
+
 int run_resident(const Problem& P, int dtype_qk, bool dry_run, hipStream_t s) {
     const bool h = dtype_qk == MA_F16;
     const int D = P.D;
@@ -161,14 +182,16 @@ bool resident_fits(const ma_fwd_params* p) {
 // beat it for few heads and the chained kernel for many.
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
+    const bool fast32 = mfma32_supported(p);   // fp32 operands: per-stage launches only
     const long long heads = static_cast<long long>(p->E) * p->H;
     switch (p->variant) {
         case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
-        case MA_VARIANT_STAGED: return fast ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_STAGED: return fast || fast32 ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_FUSED: return fast ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_CHAINED: return fast ? MA_VARIANT_CHAINED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_RESIDENT: return fast && resident_fits(p) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
         default:
+            if (fast32) return MA_VARIANT_STAGED;
             if (!fast) return MA_VARIANT_GENERIC;
             if (heads >= 128 && resident_fits(p)) return MA_VARIANT_RESIDENT;
             if (heads >= 32 && p->B <= 64 && (static_cast<long long>(p->N) + p->B - 1) / p->B <= 64) return MA_VARIANT_CHAINED;
@@ -207,14 +230,17 @@ int run_chain(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
 
 int run_r(const Prepared& pr, const ma_fwd_params* p, bool first, bool with_v, hipStream_t s) {
     if (pr.variant == MA_VARIANT_GENERIC) return launch_generic_r(pr.P, p->dtype_qk, p->dtype_v, first, with_v, s);
+    if (p->dtype_qk == MA_F32) return launch_mfma32_r(pr.P, first, with_v, s);
     return p->dtype_qk == MA_F16 ? launch_mfma_r_f16(pr.P, first, with_v, s) : launch_mfma_r_bf16(pr.P, first, with_v, s);
 }
 int run_l(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
     if (pr.variant == MA_VARIANT_GENERIC) return launch_generic_l(pr.P, p->dtype_qk, s);
+    if (p->dtype_qk == MA_F32) return launch_mfma32_l(pr.P, s);
     return p->dtype_qk == MA_F16 ? launch_mfma_l_f16(pr.P, s) : launch_mfma_l_bf16(pr.P, s);
 }
 int run_z(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
     if (pr.variant == MA_VARIANT_GENERIC) return launch_generic_z(pr.P, p->dtype_qk, p->dtype_v, s);
+    if (p->dtype_qk == MA_F32) return launch_mfma32_z(pr.P, s);
     return p->dtype_qk == MA_F16 ? launch_mfma_z_f16(pr.P, s) : launch_mfma_z_bf16(pr.P, s);
 }
 

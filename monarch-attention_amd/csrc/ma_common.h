@@ -60,6 +60,13 @@ int launch_mfma_r_bf16(const Problem& P, bool first, bool with_v, hipStream_t s)
 int launch_mfma_l_bf16(const Problem& P, hipStream_t s);
 int launch_mfma_z_bf16(const Problem& P, hipStream_t s);
 
+// fp32 MFMA stage kernels (v_mfma_f32_16x16x4_f32; Dv == D <= 128, D % 4 == 0, B, M <= 128,
+// 16-byte aligned rows) and the LDS their largest stage needs for a shape.
+int launch_mfma32_r(const Problem& P, bool first, bool with_v, hipStream_t s);
+int launch_mfma32_l(const Problem& P, hipStream_t s);
+int launch_mfma32_z(const Problem& P, hipStream_t s);
+size_t mfma32_lds_needed(int D, int B, int M);
+
 // Fused forward (one launch), by dtype and head-dim class (D <= 32/64/80/128).
 // sync_ready: the workspace's sync area is known to be zero.
 int launch_fused_f16_d2(const Problem& P, bool sync_ready, hipStream_t s);

@@ -1,0 +1,6 @@
+// Z-step MFMA kernels, fp32 operands.
+#include "ma_mfma32_launch.h"
+
+namespace ma {
+int launch_mfma32_z(const Problem& P, hipStream_t s) { return mfma32::launch_z(P, s); }
+}  // namespace ma

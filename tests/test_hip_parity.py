@@ -238,8 +238,10 @@ def test_empty_and_invalid_inputs_raise():
     q, k, v = to_dev(*seeded_qkv(1, 2, 32, 64, torch.float16))
     with pytest.raises(ValueError):
         monarch_attention_hip(q, k, v, None, 1, 16, False, variant="nope")
-    with pytest.raises(NotImplementedError):                 # fp32 cannot run on the MFMA kernels: no silent fallback
-        monarch_attention_hip(q.float(), k.float(), v.float(), None, 1, 16, False, variant="staged")
+    with pytest.raises(NotImplementedError):                 # fp32 has stage kernels only: no silent fallback
+        monarch_attention_hip(q.float(), k.float(), v.float(), None, 1, 16, False, variant="chained")
+    with pytest.raises(NotImplementedError):                 # an fp32 V with fp16 q / k is for the generic kernels
+        monarch_attention_hip(q, k, v.float(), None, 1, 16, False, variant="staged")
     with pytest.raises(NotImplementedError):
         with torch.enable_grad():
             monarch_attention_hip(q.requires_grad_(), k, v, None, 1, 16, False)
