@@ -68,18 +68,34 @@ struct Lds32 {
     static constexpr size_t L = (2 * TILE + ROWS * LDP + (1 + Split<NWT>::WPP) * ROWS) * sizeof(float);
 };
 
-// Cooperative global -> LDS copy of `rows` rows (the tile has ROWS; the rest is zero-filled through
-// the bounds check) of 16-byte chunks by nth threads.  rowoff(row) = byte offset of the row in src or kOob.
-template <int DTF, int ROWS, class RowOff>
-__device__ __forceinline__ void copy_tile(float* tile, rsrc_t src, int D, RowOff rowoff, int tix, int nth) {
-    constexpr int CH = 4 * DTF;   // chunks per row
-    for (int c = tix; c < ROWS * CH; c += nth) {
-        const int row = c / CH, ch = c % CH;
-        const unsigned ro = rowoff(row);
-        const u32x4 v = bload16<true>(src, (ch * 4 < D) ? ro + ch * 16 : kOob);
-        *reinterpret_cast<u32x4*>(tile + row * Geom32<DTF>::LD + ch * 4) = v;
+// Cooperative global -> LDS copy of a ROWS-row tile of 16-byte chunks by NTH threads, in two halves
+// so that a problem can put ALL its loads in flight before it waits for any of them: issue() starts
+// the loads into registers, commit() writes them to LDS.  rowoff(row) = byte offset of the row in
+// src or kOob (rows beyond the problem and columns at or beyond D are zero-filled by the bounds check).
+template <int DTF, int ROWS, int NTH>
+struct TileCopy32 {
+    static constexpr int CH = 4 * DTF;   // chunks per row
+    static constexpr int CNT = ROWS * CH / NTH;
+    static_assert(ROWS * CH % NTH == 0, "tile chunks must divide evenly among the threads");
+    u32x4 val[CNT];
+    template <class RowOff>
+    __device__ __forceinline__ void issue(rsrc_t src, int D, RowOff rowoff, int tix) {
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) {
+            const int c = tix + i * NTH;
+            const int row = c / CH, ch = c % CH;
+            const unsigned ro = rowoff(row);
+            val[i] = bload16<true>(src, (ch * 4 < D) ? ro + ch * 16 : kOob);
+        }
     }
-}
+    __device__ __forceinline__ void commit(float* tile, int tix) const {
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) {
+            const int c = tix + i * NTH;
+            *reinterpret_cast<u32x4*>(tile + (c / CH) * Geom32<DTF>::LD + (c % CH) * 4) = val[i];
+        }
+    }
+};
 
 // this lane's 16-byte pieces (columns 16 t + 4 q ..) of the row at byte offset ro (or kOob)
 template <int DTF>
@@ -165,8 +181,13 @@ __global__ __launch_bounds__(64 * Split<NWT>::WPP) void r_step_f32(Problem P, in
     const unsigned db = static_cast<unsigned>(D) * 4u;
     const int t0 = m * B - P.pad_off;
 
-    copy_tile<DTF, ROWS>(Kt, S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix, 64 * WPP);
-    if (with_v) copy_tile<DTF, ROWS>(Vt, S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix, 64 * WPP);
+    {
+        TileCopy32<DTF, ROWS, 64 * WPP> kc, vc;
+        kc.issue(S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
+        if (with_v) vc.issue(S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix);
+        kc.commit(Kt, tix);
+        if (with_v) vc.commit(Vt, tix);
+    }
     for (int i = tix; i < ROWS; i += 64 * WPP)
         kbias[i] = (i < B && token_kept(P, t0 + i, mask_load(S, P, t0 + i, i < B))) ? 0.f : kNegBig;
     __syncthreads();
@@ -256,8 +277,13 @@ __global__ __launch_bounds__(64 * Split<NWT>::WPP) void z_step_f32(Problem P) {
     const unsigned db = static_cast<unsigned>(D) * 4u;
     const unsigned row0 = static_cast<unsigned>(j * M);
 
-    copy_tile<DTF, ROWS>(At, S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix, 64 * WPP);
-    copy_tile<DTF, ROWS>(Yt, S.Y, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix, 64 * WPP);
+    {
+        TileCopy32<DTF, ROWS, 64 * WPP> ac, yc;
+        ac.issue(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        yc.issue(S.Y, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        ac.commit(At, tix);
+        yc.commit(Yt, tix);
+    }
     for (int k = tix; k < ROWS; k += 64 * WPP) cb[k] = k < M ? -kLog2e * bloadf<true>(S.cL, (row0 + k) * 4u) : kNegBig;
     __syncthreads();
 
@@ -319,8 +345,13 @@ __global__ __launch_bounds__(64 * Split<NWT>::WPP) void l_step_f32(Problem P) {
     const unsigned db = static_cast<unsigned>(D) * 4u;
     const unsigned row0 = static_cast<unsigned>(j * M);
 
-    copy_tile<DTF, ROWS>(Qt, S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix, 64 * WPP);
-    copy_tile<DTF, ROWS>(At, S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix, 64 * WPP);
+    {
+        TileCopy32<DTF, ROWS, 64 * WPP> qc, ac;
+        qc.issue(S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
+        ac.issue(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        qc.commit(Qt, tix);
+        ac.commit(At, tix);
+    }
     for (int k = tix; k < ROWS; k += 64 * WPP) cb[k] = k < M ? -kLog2e * bloadf<true>(S.cL, (row0 + k) * 4u) : kNegBig;
     __syncthreads();
 
