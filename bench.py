@@ -39,9 +39,13 @@ CONFIGS = {  # name: (E, H, N, D, B, T, dtype, scale)  - BASELINE.json configs +
     "c3": (16, 12, 512, 64, 32, 2, "bf16", 1.0),
     "c4": (8, 16, 1024, 72, 32, 3, "f16", 1.0),
     "c5": (1, 16, 16384, 64, 128, 3, "f16", 1.0),
+    # model shapes beyond the BASELINE configs (fp32 goes through the fp32 matrix-core stage kernels)
+    "gps": (1, 2, 7600, 48, 128, 2, "f32", 1.0),
+    "c3f32": (16, 12, 512, 64, 32, 2, "f32", 1.0),
 }
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
+MFMA_PEAK_TFLOPS_F32 = 157.3   # dense fp32
 
 # HBM-side bytes per launch of the dominant kernels on the metric workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for a plain
@@ -191,7 +195,7 @@ def main():
                    "flop_per_fwd": flops, "compulsory_bytes_per_fwd": cbytes, "rotating_input_sets": nbuf},
         "stream_ms_per_step": round(ev_ms, 5),
         "fwd_hbm_frac": round(cbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-        "fwd_mfma_frac": round(flops / (ev_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 5),
+        "fwd_mfma_frac": round(flops / (ev_ms * 1e-3) / 1e12 / (MFMA_PEAK_TFLOPS_F32 if dt == "f32" else MFMA_PEAK_TFLOPS), 5),
         "roofline": roofline,
     }
 
