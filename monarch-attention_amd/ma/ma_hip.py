@@ -137,6 +137,33 @@ def make_params(q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B
     return p
 
 
+# Filling a ma_fwd_params field by field costs more host time than a small forward takes on the
+# GPU, and a model calls the operator with the same few shapes over and over: the filled block
+# (and the workspace size the library reports for it) is kept per call signature, and a call only
+# copies it and patches the pointers.
+_PARAM_CACHE: dict[tuple, tuple] = {}
+_PARAM_CACHE_MAX = 256
+
+
+def _params_for(lib, q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B: int, pre_pad: bool,
+                variant: str) -> tuple:
+    key = (q.shape, q.stride(), k.stride(), v.shape, v.stride(), out.stride(),
+           None if mask_u8 is None else mask_u8.stride(), q.dtype, v.dtype, T, B, bool(pre_pad), variant)
+    hit = _PARAM_CACHE.get(key)
+    if hit is None:
+        tmpl = make_params(q, k, v, mask_u8, out, T, B, pre_pad, variant)
+        nbytes = lib.ma_fwd_workspace_bytes(tmpl)
+        if nbytes == 0:   # invalid problem: let the library say why
+            L.check(lib.ma_fwd_workspace_layout(tmpl, L.WsLayout()), "monarch_attention_hip")
+        if len(_PARAM_CACHE) >= _PARAM_CACHE_MAX:
+            _PARAM_CACHE.clear()
+        hit = _PARAM_CACHE[key] = (bytes(tmpl), nbytes)
+    p = L.FwdParams.from_buffer_copy(hit[0])
+    p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    p.mask = mask_u8.data_ptr() if mask_u8 is not None else None
+    return p, hit[1]
+
+
 def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, T: int, B: int,
                           pre_pad: bool, *, variant: str | None = None) -> Tensor:
     """MonarchAttention forward on the current HIP stream; returns a new
@@ -157,10 +184,7 @@ def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | N
     E, H, N, _ = q.shape
     with torch.cuda.device(q.device):
         out = _empty_like_layout(v, (E, H, N, v.shape[-1]))
-        p = make_params(q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
-        nbytes = lib.ma_fwd_workspace_bytes(p)
-        if nbytes == 0:
-            L.check(lib.ma_fwd_workspace_layout(p, L.WsLayout()), "monarch_attention_hip")
+        p, nbytes = _params_for(lib, q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
         stream = torch.cuda.current_stream(q.device).cuda_stream
         ws = _workspace(q.device, stream, nbytes)
         p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
