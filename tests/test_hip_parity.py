@@ -408,3 +408,45 @@ def test_full_size_properties(E, H, N, D, B, T, dt, variant):
     gen = run_hip(q[sub], k[sub], v[sub], None, T, B, False, "generic")
     assert_parity(out[sub].cpu(), gen.cpu(), dt, "vs generic")
     assert sync_status() == 0
+
+
+# ---------------------------------------------------------------- seeded random shapes, every variant
+def _random_cases(n, seed):
+    import random
+    rng = random.Random(seed)
+    cases = []
+    for i in range(n):
+        dt = rng.choice(["f16", "f16", "bf16", "f32"])
+        D = rng.choice([8, 16, 24, 32, 40, 48, 56, 64, 72, 80, 96, 128] if dt != "f32" else [4, 8, 12, 16, 32, 36, 48, 64, 100, 128])
+        B = rng.choice([1, 2, 3, 5, 8, 14, 16, 17, 24, 31, 32, 33, 48, 64, 65, 96, 128])
+        M = rng.choice([1, 2, 3, 4, 7, 8, 15, 16, 17, 31, 32, 33, 64] if B <= 32 else [1, 2, 3, 5, 8, 9])
+        N = max(1, M * B - rng.randrange(0, B))           # ragged last block most of the time
+        E, H = rng.choice([1, 1, 2, 3]), rng.choice([1, 2, 3, 5])
+        T = rng.choice([1, 1, 2, 2, 3, 4])
+        pre = rng.random() < 0.5
+        masked = rng.random() < 0.4
+        cases.append((i, E, H, N, D, B, T, pre, dt, masked))
+    return cases
+
+
+@pytest.mark.parametrize("idx,E,H,N,D,B,T,pre,dt,masked", _random_cases(200, seed=2024))
+def test_random_shapes_every_variant(idx, E, H, N, D, B, T, pre, dt, masked):
+    """Seeded random problems over the whole argument space (ragged N, odd block
+    sizes and counts, every head-dim class, both pad sides, key masks, 1..4
+    steps): every variant that accepts the problem must meet the parity gate,
+    and AUTO / GENERIC must accept all of them."""
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt], scale=0.7, seed=100 + idx)
+    mask = block_safe_mask(E, N, B, seed=idx) if masked else None
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=dt != "f32")
+    ran = []
+    for variant in VARIANTS:
+        try:
+            out = monarch_attention_hip(*to_dev(q, k, v, mask), T, B, pre, variant=variant)
+        except NotImplementedError:
+            assert variant not in ("auto", "generic")
+            continue
+        torch.cuda.synchronize()
+        assert_parity(out.cpu(), ref, dt, f"case {idx} {(E, H, N, D, B, T, pre, dt, masked)} / {variant}")
+        ran.append(variant)
+    assert "auto" in ran and "generic" in ran
+    assert sync_status() == 0
