@@ -38,6 +38,8 @@ int check_shape(const ma_fwd_params* p) {
         if (p->N > 1) return MA_ERR_STRIDE;  // rows of q / k overlap
     }
     if (p->N > 1 && (p->v_stride[2] < p->Dv || p->out_stride[2] < p->Dv)) return MA_ERR_STRIDE;
+    // inputs may be broadcast over batch / heads (stride 0); output slices must not coincide
+    if ((p->E > 1 && p->out_stride[0] == 0) || (p->H > 1 && p->out_stride[1] == 0)) return MA_ERR_STRIDE;
     if (p->mask_stride[0] < 0 || p->mask_stride[1] < 0) return MA_ERR_STRIDE;
     if (!(p->eps >= 0.0f)) return MA_ERR_SHAPE;
     return MA_OK;

@@ -97,6 +97,13 @@ def test_overlapping_rows_and_negative_strides_are_rejected():
     p = good_params()
     p.v_stride = (C.c_int64 * 3)(-1, 800, 16)
     assert lib.ma_fwd(p, None) == L.MA_ERR_STRIDE
+    p = good_params()
+    if p.H > 1:                                       # output slices of different heads may not coincide
+        p.out_stride = (C.c_int64 * 3)(p.out_stride[0], 0, p.out_stride[2])
+        assert lib.ma_fwd(p, None) == L.MA_ERR_STRIDE
+    p = good_params()
+    p.k_stride = (C.c_int64 * 3)(0, 0, p.k_stride[2])  # inputs may be broadcast over batch and heads
+    assert lib.ma_fwd_workspace_bytes(p) > 0
 
 
 def test_pointer_and_workspace_checks_precede_any_launch():

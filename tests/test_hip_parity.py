@@ -314,6 +314,20 @@ def test_permuted_views_as_models_pass_them(dt, variant):
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
+def test_broadcast_keys_and_values(variant):
+    """k and v shared by all heads and batch entries (expanded views, stride 0):
+    read in place, same result as with materialised copies."""
+    E, H, N, D, B, T = 2, 6, 160, 64, 32, 2
+    q, k, v = seeded_qkv(E, H, N, D, torch.float16)
+    k1, v1 = k[:1, :1], v[:1, :1]
+    ref = monarch_attention_oracle(q, k1.expand(E, H, N, D).contiguous(), v1.expand(E, H, N, D).contiguous(), None, T, B, False,
+                                   upcast=True)
+    qd, kd, vd = to_dev(q, k1, v1)
+    out = run_hip(qd, kd.expand(E, H, N, D), vd.expand(E, H, N, D), None, T, B, False, variant)
+    assert_parity(out.cpu(), ref, "f16")
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("kind", ["bool", "int64", "float"])
 def test_mask_dtypes(kind, variant):
     E, H, N, D, B, T = 2, 2, 384, 64, 32, 2
