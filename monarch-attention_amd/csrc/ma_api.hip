@@ -170,6 +170,26 @@ bool resident_fits(const ma_fwd_params* p) {
     return run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
 }
 
+// Can the chained kernel take the problem?  Mirrors the launcher's limits: at most 128 tasks per
+// head and phase (one poll covers 128 flags), the heads' flag words fit their part of the sync area,
+// the grid is a 31-bit count.  Four waves per workgroup; a block problem of n rows takes
+// min(ceil(n / 16), 4) waves, rounded up to a power of two.
+bool chain_fits(const ma_fwd_params* p) {
+    auto tasks = [](long long count, long long rows) {
+        const long long strips = (rows + 15) / 16;
+        const long long waves = strips <= 1 ? 1 : strips <= 2 ? 2 : 4;
+        const long long per_wg = 4 / waves;
+        return (count + per_wg - 1) / per_wg;
+    };
+    const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+    const long long tR = tasks(M, p->B), tL = tasks(p->B, M);
+    const long long heads = static_cast<long long>(p->E) * p->H;
+    const long long stride = p->T * (tR + tL) + 1;
+    if (tR > 128 || tL > 128) return false;
+    if (heads * stride > static_cast<long long>(kChainSyncBytes / 4)) return false;
+    return 8 * ((heads + 7) / 8) * p->T * (tR + tL) <= 0x7fffffffLL;
+}
+
 // The variant a problem resolves to.  AUTO: the MFMA kernels when the problem
 // qualifies; among them (measured on MI355X)
 //  * the resident kernel when a head's state fits in LDS and there are enough
@@ -190,13 +210,13 @@ int select_variant(const ma_fwd_params* p) {
         case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
         case MA_VARIANT_STAGED: return fast || fast32 ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_FUSED: return fast ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
-        case MA_VARIANT_CHAINED: return fast ? MA_VARIANT_CHAINED : MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_CHAINED: return fast && chain_fits(p) ? MA_VARIANT_CHAINED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_RESIDENT: return fast && resident_fits(p) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
         default:
             if (fast32) return MA_VARIANT_STAGED;
             if (!fast) return MA_VARIANT_GENERIC;
             if (heads >= 128 && resident_fits(p)) return MA_VARIANT_RESIDENT;
-            if (heads >= 32 && p->B <= 64 && (static_cast<long long>(p->N) + p->B - 1) / p->B <= 64) return MA_VARIANT_CHAINED;
+            if (heads >= 32 && p->B <= 64 && (static_cast<long long>(p->N) + p->B - 1) / p->B <= 64 && chain_fits(p)) return MA_VARIANT_CHAINED;
             return MA_VARIANT_STAGED;
     }
 }

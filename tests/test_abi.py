@@ -165,6 +165,7 @@ def test_auto_variant_policy():
     assert auto(16, 12, 512, 64, 32) == "chained"      # state of a 512-token head does not fit in LDS
     assert auto(8, 16, 1024, 72, 32) == "chained"
     assert auto(4, 16, 16384, 64, 128) == "staged"      # many heads, but 128-row problems
+    assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for
     assert auto(2, 2, 197, 64, 16) == "staged"          # few heads
     assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "staged"       # fp32 MFMA stage kernels
     assert auto(1, 2, 7600, 48, 128, dt=L.MA_F32) == "staged"
