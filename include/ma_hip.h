@@ -149,6 +149,18 @@ int ma_r_step(const ma_fwd_params* p, int first, int with_v, void* stream);
 int ma_l_step(const ma_fwd_params* p, void* stream);
 int ma_z_step(const ma_fwd_params* p, void* stream);
 
+/* Dense attention matrix: replaces MonarchAttention.get_matrix
+ * (ma/monarch_attention.py:61-66), which runs the forward pass on an fp32
+ * identity.  The same T steps run on q, k and the mask, then every entry
+ * A[(l,j),(k,i)] = Lz[j][l,k] * R[k][j,i] is written once, in fp32: no N x N
+ * identity, no (E,H,Np,N) Y state.  `A` is a contiguous (E,H,N,N) fp32 device
+ * array.  Of *p the fields v, out, Dv, dtype_v, v_stride and out_stride are not
+ * read; size the workspace for Dv = D and dtype_v = dtype_qk.  Variants AUTO,
+ * GENERIC and STAGED (they select the kernels of the T steps);
+ * MA_ERR_UNSUPPORTED for the one-launch variants and for padded sequences
+ * beyond what one workgroup's LDS holds (M*B + 64*M floats <= 160 KB). */
+int ma_matrix(const ma_fwd_params* p, float* A, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -379,4 +379,39 @@ int ma_fwd(const ma_fwd_params* p, void* stream) {
     return run_z(pr, p, s);
 }
 
+int ma_matrix(const ma_fwd_params* p, float* A, void* stream) {
+    if (p == nullptr || A == nullptr) return MA_ERR_NULL;
+    if (reinterpret_cast<uintptr_t>(A) % 4) return MA_ERR_STRIDE;
+    // the T steps on q and k alone: v and out are stand-ins that no stage of this call touches
+    ma_fwd_params pp = *p;
+    pp.v = pp.q;
+    pp.out = A;
+    pp.Dv = pp.D;
+    pp.dtype_v = pp.dtype_qk;
+    for (int i = 0; i < 3; ++i) pp.v_stride[i] = pp.out_stride[i] = pp.q_stride[i];
+    if (pp.E > 1 && pp.out_stride[0] == 0) pp.out_stride[0] = 1;   // q may be broadcast; the stand-in
+    if (pp.H > 1 && pp.out_stride[1] == 0) pp.out_stride[1] = 1;   // output must pass the overlap check
+    if (pp.variant != MA_VARIANT_AUTO && pp.variant != MA_VARIANT_GENERIC && pp.variant != MA_VARIANT_STAGED)
+        return pp.variant < MA_VARIANT_AUTO || pp.variant > MA_VARIANT_CHAINED ? MA_ERR_VARIANT : MA_ERR_UNSUPPORTED;
+    if (pp.variant == MA_VARIANT_AUTO) {
+        const int st = check_shape(&pp);
+        if (st != MA_OK) return st;
+        pp.variant = mfma_supported(&pp) || mfma32_supported(&pp) ? MA_VARIANT_STAGED : MA_VARIANT_GENERIC;
+    }
+    Prepared pr;
+    int st = prepare(&pp, &pr);
+    if (st != MA_OK) return st;
+    if (!generic_matrix_fits(pr.P)) return MA_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int t = 0; t < pp.T - 1; ++t) {
+        st = run_r(pr, &pp, t == 0, false, s);
+        if (st) return st;
+        st = run_l(pr, &pp, s);
+        if (st) return st;
+    }
+    st = run_r(pr, &pp, pp.T == 1, false, s);
+    if (st) return st;
+    return launch_generic_matrix(pr.P, pp.dtype_qk, A, pp.T == 1, s);
+}
+
 }  // extern "C"

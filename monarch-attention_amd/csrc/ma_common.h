@@ -50,6 +50,10 @@ __device__ __forceinline__ float round_to<float>(float x) { return x; }
 int launch_generic_r(const Problem& P, int dt_qk, int dt_v, bool first, bool with_v, hipStream_t s);
 int launch_generic_l(const Problem& P, int dt_qk, hipStream_t s);
 int launch_generic_z(const Problem& P, int dt_qk, int dt_v, hipStream_t s);
+// dense (E,H,N,N) fp32 matrix from the state of the last R step; MA_ERR_UNSUPPORTED beyond the LDS
+constexpr size_t kMatrixLdsBytes = 160 * 1024;
+bool generic_matrix_fits(const Problem& P);
+int launch_generic_matrix(const Problem& P, int dt_qk, float* A, bool first, hipStream_t s);
 
 // MFMA stage kernels (fp16 / bf16, Dv == D <= 128, D % 8 == 0, B, M <= 128,
 // 16-byte aligned rows).

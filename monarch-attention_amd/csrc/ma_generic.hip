@@ -283,6 +283,83 @@ __global__ __launch_bounds__(kThreads) void z_step_kernel(Problem P, int TL) {
     }
 }
 
+// Dense attention matrix, written directly: row (l, j) of block-row j is
+// A[(l,j), (k,i)] = Lz[j][l,k] * R[k][j,i], which is what the forward pass
+// returns for an fp32 identity as v (ma/monarch_attention.py:61-66: Y is then R
+// itself and the Z step's sum over k has one non-zero term).  Needs aL, cL of
+// the last R step (and aR, cR of the last L step when T > 1) in the workspace.
+// One workgroup: TL query blocks l of one (e,h,j).  LDS: R[M][B], then U[TL][M].
+template <class TQ>
+__global__ __launch_bounds__(kThreads) void matrix_kernel(Problem P, float* A, int TL, int first) {
+    extern __shared__ float lds[];
+    const int M = P.M, D = P.D, B = P.B;
+    int e, h, j, lt;
+    decode_bj(P, (M + TL - 1) / TL, e, h, j, lt);
+    const int l0 = lt * TL, rows = min(TL, M - l0);
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    float* R = lds;
+    float* U = lds + M * B;
+
+    // logits of query row j against every key block k (ma_torch.py:11-13)
+    for (int idx = threadIdx.x; idx < M * B; idx += kThreads) {
+        const int k = idx / B;
+        const long long row = (eh * M + k) * B + j;
+        const TQ* x = first ? tok_row<TQ>(P.q, P.qs, e, h, k * B + j - P.pad_off, P.N)
+                            : reinterpret_cast<const TQ*>(P.aR) + row * D;
+        const int ti = idx - P.pad_off;
+        const TQ* kr = tok_row<TQ>(P.k, P.ks, e, h, ti, P.N);
+        float s = P.sm_scale * round_to<TQ>(dot_rows(x, kr, D));
+        const float c = first ? 1.0f : P.cR[row];
+        s = s / (c + P.eps);
+        if (!token_ok(P, e, ti)) s = -INFINITY;
+        R[idx] = s;
+    }
+    lz_logits<TQ>(P, U, e, h, j, l0, rows);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int k = wave; k < M; k += kWaves) {  // ma_torch.py:14-18
+        float* S = R + k * B;
+        float mx = -INFINITY;
+        for (int i = lane; i < B; i += 64) mx = fmaxf(mx, S[i]);
+        mx = fmaxf(wave_max(mx), P.eps);
+        float sum = 0.f;
+        for (int i = lane; i < B; i += 64) {
+            const float p = expf(S[i] - mx);
+            S[i] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum) + P.eps;
+        for (int i = lane; i < B; i += 64) S[i] = fmaxf(S[i] / sum, kTiny);
+    }
+    for (int ll = wave; ll < rows; ll += kWaves) {  // ma_torch.py:58-59
+        float* Ul = U + ll * M;
+        float mx = -INFINITY;
+        for (int k = lane; k < M; k += 64) mx = fmaxf(mx, Ul[k]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int k = lane; k < M; k += 64) {
+            const float p = expf(Ul[k] - mx);
+            Ul[k] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum);
+        for (int k = lane; k < M; k += 64) Ul[k] = Ul[k] / sum;
+    }
+    __syncthreads();
+
+    for (int ll = 0; ll < rows; ++ll) {
+        const int tq = (l0 + ll) * B + j - P.pad_off;
+        if (tq < 0 || tq >= P.N) continue;  // padded query rows are dropped
+        float* out = A + (eh * P.N + tq) * P.N;
+        const float* Ul = U + ll * M;
+        for (int idx = threadIdx.x; idx < M * B; idx += kThreads) {
+            const int tk = idx - P.pad_off;
+            if (tk >= 0 && tk < P.N) out[tk] = Ul[idx / B] * R[idx];
+        }
+    }
+}
+
 // rows per workgroup so that rows * width floats fit the LDS budget
 int tile_rows(int width, int want) {
     const long long budget = 48 * 1024 / 4;
@@ -344,6 +421,29 @@ int launch_generic_z(const Problem& P, int dt_qk, int dt_v, hipStream_t s) {
             hipLaunchKernelGGL((z_step_kernel<TQ, TV>), dim3(grid), dim3(kThreads), lds, s, P, TL);
             return static_cast<int>(hipGetLastError());
         });
+    });
+}
+
+bool generic_matrix_fits(const Problem& P) {
+    const int TL = tile_rows(P.M, 64);
+    const size_t lds = (static_cast<size_t>(P.M) * P.B + static_cast<size_t>(TL) * P.M) * sizeof(float);
+    const long long grid = static_cast<long long>(P.E) * P.H * P.B * ((P.M + TL - 1) / TL);
+    return lds <= kMatrixLdsBytes && grid <= 0x7FFFFFFFLL;
+}
+
+int launch_generic_matrix(const Problem& P, int dt_qk, float* A, bool first, hipStream_t s) {
+    if (!generic_matrix_fits(P)) return MA_ERR_UNSUPPORTED;
+    const int TL = tile_rows(P.M, 64);
+    const size_t lds = (static_cast<size_t>(P.M) * P.B + static_cast<size_t>(TL) * P.M) * sizeof(float);
+    const long long grid = static_cast<long long>(P.E) * P.H * P.B * ((P.M + TL - 1) / TL);
+    return dispatch_qk(dt_qk, [&](auto tq) {
+        using TQ = decltype(tq);
+        const int rc = static_cast<int>(hipFuncSetAttribute(reinterpret_cast<const void*>(matrix_kernel<TQ>),
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                            static_cast<int>(kMatrixLdsBytes)));
+        if (rc) return rc;
+        hipLaunchKernelGGL((matrix_kernel<TQ>), dim3(grid), dim3(kThreads), lds, s, P, A, TL, first ? 1 : 0);
+        return static_cast<int>(hipGetLastError());
     });
 }
 

@@ -44,7 +44,8 @@ class WsLayout(C.Structure):
 MA_FLAG_SYNC_READY = 1
 
 EXPORTS = ("ma_abi_version", "ma_strerror", "ma_fwd_workspace_layout", "ma_fwd_workspace_bytes",
-           "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_r_step", "ma_l_step", "ma_z_step")
+           "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_r_step", "ma_l_step", "ma_z_step",
+           "ma_matrix")
 
 _lock = threading.Lock()
 _lib = None
@@ -91,6 +92,8 @@ def load() -> C.CDLL:
         lib.ma_l_step.argtypes = [P, C.c_void_p]
         lib.ma_z_step.restype = C.c_int
         lib.ma_z_step.argtypes = [P, C.c_void_p]
+        lib.ma_matrix.restype = C.c_int
+        lib.ma_matrix.argtypes = [P, C.c_void_p, C.c_void_p]
         got = lib.ma_abi_version()
         if got != ABI_VERSION:
             raise ImportError(f"libma_hip.so has ABI version {got}, this binding needs {ABI_VERSION}")

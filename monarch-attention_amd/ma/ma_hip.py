@@ -172,15 +172,7 @@ def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | N
     _check_inputs(q, k, v, attn_mask, T, B)
     lib = L.load()
     q, k, v = _inner_contiguous(q), _inner_contiguous(k), _inner_contiguous(v)
-    mask_u8 = None
-    if attn_mask is not None:
-        # truthiness, as torch.logical_and sees it (ma/ma_torch.py:98).  bool / uint8 / int8 masks
-        # are already one byte per token with "non-zero = keep": the kernels read them in place
-        # (any strides); other dtypes are reduced to bytes by one small elementwise kernel.
-        if attn_mask.dtype in (torch.bool, torch.uint8, torch.int8):
-            mask_u8 = attn_mask.view(torch.uint8)
-        else:
-            mask_u8 = (attn_mask != 0).to(torch.uint8)
+    mask_u8 = _mask_bytes(attn_mask)
     E, H, N, _ = q.shape
     with torch.cuda.device(q.device):
         out = _empty_like_layout(v, (E, H, N, v.shape[-1]))
@@ -191,3 +183,45 @@ def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | N
         p.flags = L.MA_FLAG_SYNC_READY
         L.check(lib.ma_fwd(p, stream), "ma_fwd")
     return out
+
+
+def _mask_bytes(attn_mask):
+    """One byte per token, non-zero = keep: truthiness as torch.logical_and sees it
+    (ma/ma_torch.py:98).  bool / uint8 / int8 masks already are that and are read in place
+    (any strides); other dtypes are reduced to bytes by one small elementwise kernel."""
+    if attn_mask is None:
+        return None
+    if attn_mask.dtype in (torch.bool, torch.uint8, torch.int8):
+        return attn_mask.view(torch.uint8)
+    return (attn_mask != 0).to(torch.uint8)
+
+
+def monarch_matrix_hip(q: Tensor, k: Tensor, attn_mask: Tensor | None, T: int, B: int, pre_pad: bool, *,
+                       variant: str | None = None) -> Tensor:
+    """Dense ``(E, H, N, N)`` fp32 attention matrix of q and k: what the forward
+    pass returns for an fp32 identity as v (``MonarchAttention.get_matrix``,
+    ma/monarch_attention.py:61-66), written entry by entry by ``ma_matrix``
+    without the identity and without the ``(E, H, Np, N)`` intermediate.
+    ``variant`` ('auto', 'generic' or 'staged') selects the kernels of the T
+    steps.  Raises ``NotImplementedError`` when the padded sequence is beyond
+    what the kernel holds on chip."""
+    _check_inputs(q, k, q, attn_mask, T, B)
+    lib = L.load()
+    q, k = _inner_contiguous(q), _inner_contiguous(k)
+    mask_u8 = _mask_bytes(attn_mask)
+    E, H, N, _ = q.shape
+    with torch.cuda.device(q.device):
+        A = torch.empty((E, H, N, N), dtype=torch.float32, device=q.device)
+        p = make_params(q, k, q, mask_u8, A, T, B, pre_pad, variant or DEFAULT_VARIANT)
+        nbytes = lib.ma_fwd_workspace_bytes(p)
+        if nbytes == 0:
+            L.check(lib.ma_fwd_workspace_layout(p, L.WsLayout()), "monarch_matrix_hip")
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        ws = _workspace(q.device, stream, nbytes)
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+        p.flags = L.MA_FLAG_SYNC_READY
+        st = lib.ma_matrix(p, A.data_ptr(), stream)
+        if st == L.MA_ERR_UNSUPPORTED:
+            raise NotImplementedError("ma_matrix: " + L.strerror(st))
+        L.check(st, "ma_matrix")
+    return A

@@ -19,7 +19,7 @@ from enum import Enum
 import torch
 import torch.nn as nn
 
-from .ma_hip import monarch_attention_hip
+from .ma_hip import monarch_attention_hip, monarch_matrix_hip
 
 Tensor = torch.Tensor
 
@@ -79,9 +79,18 @@ class MonarchAttention(nn.Module):
         return self._impl_fn(query, key, value, attention_mask, self.num_steps, self.block_size, pre_pad)
 
     def get_matrix(self, query, key, attention_mask=None):
-        """Dense ``(E,H,N,N)`` attention matrix: the forward pass applied to an
-        fp32 identity (reference ``:61-66``)."""
+        """Dense ``(E,H,N,N)`` fp32 attention matrix: the forward pass applied to
+        an fp32 identity (reference ``:61-66``).  The ``"hip"`` implementation
+        writes the matrix directly (no identity, no ``(E,H,Np,N)`` intermediate)
+        and takes the identity route only for sequences its matrix kernel does
+        not hold on chip; other implementations always take that route."""
         E, H, N, _ = query.shape
+        if self._impl_fn is monarch_attention_hip:
+            pre_pad = self.pad_type == PadType.pre
+            try:
+                return monarch_matrix_hip(query, key, attention_mask, self.num_steps, self.block_size, pre_pad)
+            except NotImplementedError:
+                pass
         eye = torch.eye(N, device=query.device).expand(E, H, N, N)
         return self.forward(query, key, eye, attention_mask)
 

@@ -124,6 +124,18 @@ def test_pointer_and_workspace_checks_precede_any_launch():
         assert fn(good_params(), None) == L.MA_ERR_NULL
     assert lib.ma_r_step(good_params(), 1, 0, None) == L.MA_ERR_NULL
     assert lib.ma_fwd(None, None) == L.MA_ERR_NULL
+    # ma_matrix: NULL output, NULL q / k, missing workspace, one-launch variants
+    assert lib.ma_matrix(good_params(), None, None) == L.MA_ERR_NULL
+    assert lib.ma_matrix(good_params(), 0x20000, None) == L.MA_ERR_NULL
+    pm = good_params()
+    pm.q = pm.k = 0x10000
+    assert lib.ma_matrix(pm, 0x20002, None) == L.MA_ERR_STRIDE         # fp32 output must be 4-byte aligned
+    assert lib.ma_matrix(pm, 0x20000, None) == L.MA_ERR_WORKSPACE      # v / out are not needed
+    for name in ("fused", "resident", "chained"):
+        pm.variant = L.VARIANTS[name]
+        assert lib.ma_matrix(pm, 0x20000, None) == L.MA_ERR_UNSUPPORTED
+    pm.variant = 99
+    assert lib.ma_matrix(pm, 0x20000, None) == L.MA_ERR_VARIANT
 
 
 def test_select_variant_reports_a_known_variant():

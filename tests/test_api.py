@@ -51,6 +51,21 @@ def test_register_impl_and_argument_marshalling():
         api._IMPLEMENTATIONS.pop("fake")
 
 
+def test_get_matrix_takes_the_identity_route_when_the_matrix_kernel_declines(monkeypatch):
+    calls = []
+
+    def decline(*args, **kwargs):
+        calls.append(args)
+        raise NotImplementedError("padded sequence too long")
+
+    monkeypatch.setattr(api, "monarch_matrix_hip", decline)
+    q, k = torch.zeros(1, 1, 6, 4), torch.ones(1, 1, 6, 4)
+    # CPU tensors: the forward pass of "hip" refuses them, which shows that it was reached
+    with pytest.raises(ValueError, match="GPU"):
+        MonarchAttention(3, 1, "pre").get_matrix(q, k)
+    assert len(calls) == 1 and calls[0][3:] == (1, 3, True)
+
+
 def _qkv(dtype=torch.float16):
     return (torch.randn(1, 2, 8, 4, dtype=dtype) for _ in range(3))
 
