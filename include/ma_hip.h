@@ -161,6 +161,34 @@ int ma_z_step(const ma_fwd_params* p, void* stream);
  * beyond what one workgroup's LDS holds (M*B + 64*M floats <= 160 KB). */
 int ma_matrix(const ma_fwd_params* p, float* A, void* stream);
 
+/* Backward pass.  The reference has no backward code: it differentiates
+ * monarch_attention_torch (ma/ma_torch.py:65-108) with PyTorch autograd, which
+ * is what training through the operator uses (experiments/gps/train.py:34).
+ * ma_bwd is that derivative: given the inputs of a forward call and the
+ * gradient of its output it writes the gradients of q, k and v.  The forward
+ * state is not kept between the two calls: ma_bwd runs the T steps again
+ * (kernels chosen by fwd.variant: AUTO, GENERIC or STAGED), keeping every
+ * step's state in its workspace, then walks the steps backwards in fp32.
+ *   fwd            the forward call's arguments; fwd.out is not read;
+ *                  fwd.workspace / workspace_bytes: >= ma_bwd_workspace_bytes()
+ *   dout           (E,H,N,Dv) dtype_v, element strides dout_stride
+ *   dq, dk / dv    (E,H,N,D) dtype_qk / (E,H,N,Dv) dtype_v, written in full
+ * MA_ERR_UNSUPPORTED for the one-launch variants and for M > 6144 or B > 4096. */
+typedef struct ma_bwd_params {
+    ma_fwd_params fwd;
+    const void* dout;
+    void* dq;
+    void* dk;
+    void* dv;
+    int64_t dout_stride[3];
+    int64_t dq_stride[3];
+    int64_t dk_stride[3];
+    int64_t dv_stride[3];
+} ma_bwd_params;
+
+uint64_t ma_bwd_workspace_bytes(const ma_bwd_params* p);
+int ma_bwd(const ma_bwd_params* p, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -279,6 +279,57 @@ int prepare(const ma_fwd_params* p, Prepared* out) {
     return MA_OK;
 }
 
+
+// Workspace of the backward pass: every step's forward state, the state gradients, and padded
+// fp32 accumulators of the input gradients.
+struct BwdLayout {
+    uint64_t aL, cL, aR, cR, Y, stats;      // aL / cL: T slots; aR / cR: T - 1 slots (steps 1..T-1)
+    uint64_t gaR, gcR, gaL, gcL, gY, dq, dk, dv;
+    uint64_t slot_a, slot_c;                // bytes of one aL / aR slot and of one cL / cR slot
+    uint64_t total;
+};
+
+int bwd_prepare(const ma_bwd_params* b, ma_fwd_params* pp, BwdLayout* L) {
+    if (b == nullptr) return MA_ERR_NULL;
+    *pp = b->fwd;
+    // the forward output is not needed: a stand-in that passes the checks and is never written
+    pp->out = b->dv;
+    for (int i = 0; i < 3; ++i) pp->out_stride[i] = b->dv_stride[i];
+    int st = check_shape(pp);
+    if (st != MA_OK) return st;
+    if (pp->variant != MA_VARIANT_AUTO && pp->variant != MA_VARIANT_GENERIC && pp->variant != MA_VARIANT_STAGED) return MA_ERR_UNSUPPORTED;
+    for (int i = 0; i < 3; ++i)
+        if (b->dout_stride[i] < 0 || b->dq_stride[i] < 0 || b->dk_stride[i] < 0 || b->dv_stride[i] < 0) return MA_ERR_STRIDE;
+    if (pp->N > 1 && (b->dout_stride[2] < pp->Dv || b->dv_stride[2] < pp->Dv || b->dq_stride[2] < pp->D || b->dk_stride[2] < pp->D))
+        return MA_ERR_STRIDE;
+    if ((pp->E > 1 && (b->dq_stride[0] == 0 || b->dk_stride[0] == 0 || b->dv_stride[0] == 0)) ||
+        (pp->H > 1 && (b->dq_stride[1] == 0 || b->dk_stride[1] == 0 || b->dv_stride[1] == 0)))
+        return MA_ERR_STRIDE;
+    const uint64_t M = (static_cast<uint64_t>(pp->N) + pp->B - 1) / pp->B;
+    const uint64_t rows = static_cast<uint64_t>(pp->E) * pp->H * M * pp->B;
+    const uint64_t sq = elt_size(pp->dtype_qk), sv = elt_size(pp->dtype_v), T = pp->T;
+    L->slot_a = align_up(rows * pp->D * sq);
+    L->slot_c = align_up(rows * 4);
+    uint64_t off = 0;
+    L->aL = off; off += T * L->slot_a;
+    L->cL = off; off += T * L->slot_c;
+    L->aR = off; off += (T - 1) * L->slot_a;
+    L->cR = off; off += (T - 1) * L->slot_c;
+    L->Y = off; off = align_up(off + rows * pp->Dv * sv);
+    L->stats = off; off = align_up(off + rows * 8);
+    L->gaR = off; off = align_up(off + rows * pp->D * 4);
+    L->gcR = off; off = align_up(off + rows * 4);
+    L->gaL = off; off = align_up(off + rows * pp->D * 4);
+    L->gcL = off; off = align_up(off + rows * 4);
+    L->gY = off; off = align_up(off + rows * pp->Dv * 4);
+    // dq, dk, dv are contiguous: one fill kernel zeroes the three
+    L->dq = off; off += rows * pp->D * 4;
+    L->dk = off; off += rows * pp->D * 4;
+    L->dv = off; off = align_up(off + rows * pp->Dv * 4);
+    L->total = off;
+    return MA_OK;
+}
+
 }  // namespace
 
 int launch_zero_sync(unsigned* sync, hipStream_t s) {
@@ -412,6 +463,95 @@ int ma_matrix(const ma_fwd_params* p, float* A, void* stream) {
     st = run_r(pr, &pp, pp.T == 1, false, s);
     if (st) return st;
     return launch_generic_matrix(pr.P, pp.dtype_qk, A, pp.T == 1, s);
+}
+
+uint64_t ma_bwd_workspace_bytes(const ma_bwd_params* b) {
+    ma_fwd_params pp;
+    BwdLayout L;
+    return bwd_prepare(b, &pp, &L) == MA_OK ? L.total : 0;
+}
+
+int ma_bwd(const ma_bwd_params* b, void* stream) {
+    ma_fwd_params pp;
+    BwdLayout L;
+    int st = bwd_prepare(b, &pp, &L);
+    if (st != MA_OK) return st;
+    if (!pp.q || !pp.k || !pp.v || !b->dout || !b->dq || !b->dk || !b->dv) return MA_ERR_NULL;
+    if (!pp.workspace || reinterpret_cast<uintptr_t>(pp.workspace) % kAlign || pp.workspace_bytes < L.total) return MA_ERR_WORKSPACE;
+    const uintptr_t aq = elt_size(pp.dtype_qk), av = elt_size(pp.dtype_v);
+    if (reinterpret_cast<uintptr_t>(pp.q) % aq || reinterpret_cast<uintptr_t>(pp.k) % aq || reinterpret_cast<uintptr_t>(b->dq) % aq ||
+        reinterpret_cast<uintptr_t>(b->dk) % aq || reinterpret_cast<uintptr_t>(pp.v) % av || reinterpret_cast<uintptr_t>(b->dout) % av ||
+        reinterpret_cast<uintptr_t>(b->dv) % av)
+        return MA_ERR_STRIDE;
+    if (pp.variant == MA_VARIANT_AUTO) pp.variant = mfma_supported(&pp) || mfma32_supported(&pp) ? MA_VARIANT_STAGED : MA_VARIANT_GENERIC;
+    const int v = select_variant(&pp);
+    if (v < 0) return v;
+
+    char* ws = static_cast<char*>(pp.workspace);
+    ma_ws_layout none;
+    std::memset(&none, 0, sizeof(none));
+    Prepared pr;
+    pr.P = make_problem(&pp, none);
+    pr.variant = v;
+    Problem& P = pr.P;
+    if (!bwd_fits(P)) return MA_ERR_UNSUPPORTED;
+    P.Y = ws + L.Y;
+    P.stats = reinterpret_cast<float*>(ws + L.stats);
+    P.sync = nullptr;
+    const int T = pp.T;
+    auto at_step = [&](int t) {   // state pointers of step t: aR_t, cR_t in, aL_t, cL_t out
+        P.aL = ws + L.aL + t * L.slot_a;
+        P.cL = reinterpret_cast<float*>(ws + L.cL + t * L.slot_c);
+        // step 0 takes aR = q, cR = 1 from the inputs: its state pointers only have to be valid
+        P.aR = ws + (t > 0 ? L.aR + (t - 1) * L.slot_a : L.aL);
+        P.cR = reinterpret_cast<float*>(ws + (t > 0 ? L.cR + (t - 1) * L.slot_c : L.cL));
+    };
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    // forward again, every step's state kept
+    for (int t = 0; t < T; ++t) {
+        at_step(t);
+        st = run_r(pr, &pp, t == 0, t == T - 1, s);
+        if (st) return st;
+        if (t < T - 1) {   // the L step reads aL_t, cL_t and writes aR_{t+1}, cR_{t+1}
+            P.aR = ws + L.aR + t * L.slot_a;
+            P.cR = reinterpret_cast<float*>(ws + L.cR + t * L.slot_c);
+            st = run_l(pr, &pp, s);
+            if (st) return st;
+        }
+    }
+
+    BwdBuffers G;
+    G.gaR = reinterpret_cast<float*>(ws + L.gaR); G.gcR = reinterpret_cast<float*>(ws + L.gcR);
+    G.gaL = reinterpret_cast<float*>(ws + L.gaL); G.gcL = reinterpret_cast<float*>(ws + L.gcL);
+    G.gY = reinterpret_cast<float*>(ws + L.gY);
+    G.dq = reinterpret_cast<float*>(ws + L.dq); G.dk = reinterpret_cast<float*>(ws + L.dk); G.dv = reinterpret_cast<float*>(ws + L.dv);
+    G.dout = static_cast<const char*>(b->dout);
+    for (int i = 0; i < 3; ++i) G.dos[i] = b->dout_stride[i];
+    const long long rows = static_cast<long long>(P.E) * P.H * P.M * P.B;
+    st = launch_bwd_zero(G.dq, rows * (2LL * P.D + P.Dv), s);
+    if (st) return st;
+
+    at_step(T - 1);
+    st = launch_bwd_z(P, G, pp.dtype_qk, pp.dtype_v, s);
+    if (st) return st;
+    for (int t = T - 1; t >= 0; --t) {
+        at_step(t);
+        st = launch_bwd_r(P, G, pp.dtype_qk, pp.dtype_v, t == 0, t == T - 1, s);
+        if (st) return st;
+        if (t > 0) {   // L step t-1: state aL_{t-1}, cL_{t-1}; gradients gaR, gcR of its outputs
+            at_step(t - 1);
+            st = launch_bwd_l(P, G, pp.dtype_qk, s);
+            if (st) return st;
+        }
+    }
+    long long qs[3], ks[3], vs[3];
+    for (int i = 0; i < 3; ++i) { qs[i] = b->dq_stride[i]; ks[i] = b->dk_stride[i]; vs[i] = b->dv_stride[i]; }
+    st = launch_bwd_out(G.dq, b->dq, qs, pp.dtype_qk, P, P.D, s);
+    if (st) return st;
+    st = launch_bwd_out(G.dk, b->dk, ks, pp.dtype_qk, P, P.D, s);
+    if (st) return st;
+    return launch_bwd_out(G.dv, b->dv, vs, pp.dtype_v, P, P.Dv, s);
 }
 
 }  // extern "C"

@@ -55,6 +55,27 @@ constexpr size_t kMatrixLdsBytes = 160 * 1024;
 bool generic_matrix_fits(const Problem& P);
 int launch_generic_matrix(const Problem& P, int dt_qk, float* A, bool first, hipStream_t s);
 
+// Backward pass (FMA kernels).  Gradients of the per-step state and the padded fp32 accumulators
+// of the input gradients; `dout` is the caller's output gradient (v dtype, element strides dos).
+struct BwdBuffers {
+    float* gaR;   // (E,H,M,B,D)
+    float* gcR;   // (E,H,M,B)
+    float* gaL;   // (E,H,B,M,D)
+    float* gcL;   // (E,H,B,M)
+    float* gY;    // (E,H,B,M,Dv)
+    float* dq;    // (E,H,Np,D)   accumulated over the stages, zeroed first
+    float* dk;    // (E,H,Np,D)
+    float* dv;    // (E,H,Np,Dv)
+    const char* dout;
+    long long dos[3];
+};
+bool bwd_fits(const Problem& P);
+int launch_bwd_zero(float* p, long long n, hipStream_t s);
+int launch_bwd_z(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, hipStream_t s);
+int launch_bwd_l(const Problem& P, const BwdBuffers& G, int dt_qk, hipStream_t s);
+int launch_bwd_r(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, bool first, bool with_v, hipStream_t s);
+int launch_bwd_out(const float* src, void* dst, const long long* st, int dt, const Problem& P, int W, hipStream_t s);
+
 // MFMA stage kernels (fp16 / bf16, Dv == D <= 128, D % 8 == 0, B, M <= 128,
 // 16-byte aligned rows).
 int launch_mfma_r_f16(const Problem& P, bool first, bool with_v, hipStream_t s);

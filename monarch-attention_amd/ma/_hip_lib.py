@@ -36,6 +36,15 @@ class FwdParams(C.Structure):
     ]
 
 
+class BwdParams(C.Structure):
+    """struct ma_bwd_params"""
+    _fields_ = [
+        ("fwd", FwdParams), ("dout", C.c_void_p), ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
+        ("dout_stride", C.c_int64 * 3), ("dq_stride", C.c_int64 * 3), ("dk_stride", C.c_int64 * 3),
+        ("dv_stride", C.c_int64 * 3),
+    ]
+
+
 class WsLayout(C.Structure):
     """struct ma_ws_layout (byte offsets into the workspace)"""
     _fields_ = [(n, C.c_uint64) for n in ("aR", "cR", "aL", "cL", "Y", "stats", "sync", "total")]
@@ -45,7 +54,7 @@ MA_FLAG_SYNC_READY = 1
 
 EXPORTS = ("ma_abi_version", "ma_strerror", "ma_fwd_workspace_layout", "ma_fwd_workspace_bytes",
            "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_r_step", "ma_l_step", "ma_z_step",
-           "ma_matrix")
+           "ma_matrix", "ma_bwd_workspace_bytes", "ma_bwd")
 
 _lock = threading.Lock()
 _lib = None
@@ -94,6 +103,10 @@ def load() -> C.CDLL:
         lib.ma_z_step.argtypes = [P, C.c_void_p]
         lib.ma_matrix.restype = C.c_int
         lib.ma_matrix.argtypes = [P, C.c_void_p, C.c_void_p]
+        lib.ma_bwd_workspace_bytes.restype = C.c_uint64
+        lib.ma_bwd_workspace_bytes.argtypes = [C.POINTER(BwdParams)]
+        lib.ma_bwd.restype = C.c_int
+        lib.ma_bwd.argtypes = [C.POINTER(BwdParams), C.c_void_p]
         got = lib.ma_abi_version()
         if got != ABI_VERSION:
             raise ImportError(f"libma_hip.so has ABI version {got}, this binding needs {ABI_VERSION}")

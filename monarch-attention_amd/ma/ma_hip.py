@@ -94,9 +94,6 @@ def _check_inputs(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int) ->
             raise ValueError("attn_mask must be on the same device as q")
     if q.device.type != "cuda":
         raise ValueError(f"the 'hip' implementation needs tensors on a GPU, got {q.device}")
-    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
-        raise NotImplementedError("the 'hip' implementation is forward-only: call it under torch.no_grad() "
-                                  "or detach the inputs")
 
 
 def _inner_contiguous(t: Tensor) -> Tensor:
@@ -168,8 +165,17 @@ def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | N
                           pre_pad: bool, *, variant: str | None = None) -> Tensor:
     """MonarchAttention forward on the current HIP stream; returns a new
     ``(E, H, N, Dv)`` tensor of ``v.dtype`` in v's memory layout (contiguous for
-    contiguous v; backed by ``(E, N, H, Dv)`` when v is such a permuted view)."""
+    contiguous v; backed by ``(E, N, H, Dv)`` when v is such a permuted view).
+    Differentiable with respect to q, k and v: when one of them requires grad
+    (and grad mode is on) the call is recorded as one autograd node whose
+    backward is ``ma_bwd``."""
     _check_inputs(q, k, v, attn_mask, T, B)
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return _MonarchAttentionHip.apply(q, k, v, attn_mask, T, B, bool(pre_pad), variant)
+    return _forward(q, k, v, attn_mask, T, B, pre_pad, variant)
+
+
+def _forward(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int, pre_pad: bool, variant) -> Tensor:
     lib = L.load()
     q, k, v = _inner_contiguous(q), _inner_contiguous(k), _inner_contiguous(v)
     mask_u8 = _mask_bytes(attn_mask)
@@ -225,3 +231,53 @@ def monarch_matrix_hip(q: Tensor, k: Tensor, attn_mask: Tensor | None, T: int, B
             raise NotImplementedError("ma_matrix: " + L.strerror(st))
         L.check(st, "ma_matrix")
     return A
+
+
+def monarch_attention_hip_backward(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dout: Tensor, T: int,
+                                   B: int, pre_pad: bool, *, variant: str | None = None):
+    """Gradients ``(dq, dk, dv)`` of ``monarch_attention_hip(q, k, v, attn_mask, T, B, pre_pad)``
+    for the output gradient ``dout`` - what autograd through the reference's
+    ``monarch_attention_torch`` (ma/ma_torch.py:65-108) yields.  ``ma_bwd`` runs
+    the T steps again (``variant`` 'auto', 'generic' or 'staged' picks their
+    kernels) and then the backward kernels, all on the current stream."""
+    _check_inputs(q, k, v, attn_mask, T, B)
+    if dout.shape != v.shape or dout.device != v.device:
+        raise ValueError(f"dout must have the shape of the output {tuple(v.shape)}, got {tuple(dout.shape)}")
+    lib = L.load()
+    q, k, v = _inner_contiguous(q), _inner_contiguous(k), _inner_contiguous(v)
+    dout = _inner_contiguous(dout.to(v.dtype))
+    mask_u8 = _mask_bytes(attn_mask)
+    with torch.cuda.device(q.device):
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        b = L.BwdParams()
+        b.fwd = make_params(q, k, v, mask_u8, dv, T, B, pre_pad, variant or DEFAULT_VARIANT)
+        b.dout, b.dq, b.dk, b.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+        for name, t in (("dout_stride", dout), ("dq_stride", dq), ("dk_stride", dk), ("dv_stride", dv)):
+            setattr(b, name, (L.C.c_int64 * 3)(*t.stride()[:3]))
+        nbytes = lib.ma_bwd_workspace_bytes(b)
+        if nbytes == 0:
+            L.check(lib.ma_fwd_workspace_layout(b.fwd, L.WsLayout()), "monarch_attention_hip_backward")
+            raise NotImplementedError("ma_bwd does not support this problem (variant or block shape)")
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        # the backward workspace holds every step's state: allocated per call and freed after it
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+        b.fwd.workspace, b.fwd.workspace_bytes = ws.data_ptr(), ws.numel()
+        L.check(lib.ma_bwd(b, stream), "ma_bwd")
+    return dq, dk, dv
+
+
+class _MonarchAttentionHip(torch.autograd.Function):
+    """One autograd node per operator call: forward ``ma_fwd``, backward ``ma_bwd``."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, attn_mask, T, B, pre_pad, variant):
+        ctx.save_for_backward(q, k, v, attn_mask)
+        ctx.args = (T, B, pre_pad, variant if variant in ("auto", "generic", "staged") else None)
+        return _forward(q, k, v, attn_mask, T, B, pre_pad, variant)
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, attn_mask = ctx.saved_tensors
+        T, B, pre_pad, variant = ctx.args
+        dq, dk, dv = monarch_attention_hip_backward(q, k, v, attn_mask, dout, T, B, pre_pad, variant=variant)
+        return dq, dk, dv, None, None, None, None, None

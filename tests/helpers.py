@@ -36,6 +36,25 @@ def load_golden(name: str) -> dict:
                 out=_unpack(z["out"], vdt), E=E, H=H, N=N, D=D, Dv=Dv)
 
 
+GRAD_DIR = os.path.join(GOLDEN_DIR, "grads")
+
+
+def grad_golden_names():
+    return sorted(os.path.basename(p)[:-4] for p in glob.glob(os.path.join(GRAD_DIR, "*.npz")))
+
+
+def load_grad_golden(name: str) -> dict:
+    """One committed gradient fixture: inputs, the weights w of the loss
+    sum(out * w) (= the output gradient) and the gradients autograd through
+    the reference produced on the CPU."""
+    z = np.load(os.path.join(GRAD_DIR, name + ".npz"), allow_pickle=False)
+    E, H, N, D, Dv, B, T, pre = (int(x) for x in z["meta"])
+    dt = str(z["dt"])
+    t = {n: _unpack(z[n], dt) for n in ("q", "k", "v", "w", "dq", "dk", "dv")}
+    mask = torch.from_numpy(z["mask"].copy()) if "mask" in z.files else None
+    return dict(name=name, mask=mask, T=T, B=B, pre=bool(pre), dt=dt, **t)
+
+
 def seeded_qkv(E, H, N, D, dtype, Dv=None, scale=1.0, seed=0):
     """fp32 CPU randn in the order q, k, v (as ma/tests/test_ma.py:11-15),
     then scaled and cast."""
