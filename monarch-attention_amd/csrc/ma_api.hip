@@ -483,6 +483,7 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
         reinterpret_cast<uintptr_t>(b->dk) % aq || reinterpret_cast<uintptr_t>(pp.v) % av || reinterpret_cast<uintptr_t>(b->dout) % av ||
         reinterpret_cast<uintptr_t>(b->dv) % av)
         return MA_ERR_STRIDE;
+    const bool fma_only = pp.variant == MA_VARIANT_GENERIC;
     if (pp.variant == MA_VARIANT_AUTO) pp.variant = mfma_supported(&pp) || mfma32_supported(&pp) ? MA_VARIANT_STAGED : MA_VARIANT_GENERIC;
     const int v = select_variant(&pp);
     if (v < 0) return v;
@@ -526,6 +527,7 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
     G.gaL = reinterpret_cast<float*>(ws + L.gaL); G.gcL = reinterpret_cast<float*>(ws + L.gcL);
     G.gY = reinterpret_cast<float*>(ws + L.gY);
     G.dq = reinterpret_cast<float*>(ws + L.dq); G.dk = reinterpret_cast<float*>(ws + L.dk); G.dv = reinterpret_cast<float*>(ws + L.dv);
+    G.fma_only = fma_only ? 1 : 0;
     G.dout = static_cast<const char*>(b->dout);
     for (int i = 0; i < 3; ++i) G.dos[i] = b->dout_stride[i];
     const long long rows = static_cast<long long>(P.E) * P.H * P.M * P.B;

@@ -346,6 +346,10 @@ int launch_bwd_zero(float* p, long long n, hipStream_t s) {
 }
 
 int launch_bwd_z(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, hipStream_t s) {
+    if (!G.fma_only && dt_qk == dt_v) {
+        const int st = launch_bwd_lz_mfma(P, G, dt_qk, true, s);
+        if (st != MA_ERR_UNSUPPORTED) return st;
+    }
     const int TL = tile_rows(2 * P.M, P.M);
     const size_t lds = 2ull * TL * P.M * sizeof(float);
     return dispatch_qk(dt_qk, [&](auto tq) {
@@ -359,6 +363,10 @@ int launch_bwd_z(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, hip
 }
 
 int launch_bwd_l(const Problem& P, const BwdBuffers& G, int dt_qk, hipStream_t s) {
+    if (!G.fma_only) {
+        const int st = launch_bwd_lz_mfma(P, G, dt_qk, false, s);
+        if (st != MA_ERR_UNSUPPORTED) return st;
+    }
     const int TL = tile_rows(2 * P.M, P.M);
     const size_t lds = 2ull * TL * P.M * sizeof(float);
     return dispatch_qk(dt_qk, [&](auto tq) {
@@ -369,6 +377,10 @@ int launch_bwd_l(const Problem& P, const BwdBuffers& G, int dt_qk, hipStream_t s
 }
 
 int launch_bwd_r(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, bool first, bool with_v, hipStream_t s) {
+    if (!G.fma_only && dt_qk == dt_v) {
+        const int st = launch_bwd_r_mfma(P, G, dt_qk, first, with_v, s);
+        if (st != MA_ERR_UNSUPPORTED) return st;
+    }
     const int TJ = tile_rows(3 * P.B, P.B);
     const size_t lds = 3ull * TJ * P.B * sizeof(float);
     return dispatch_qk(dt_qk, [&](auto tq) {

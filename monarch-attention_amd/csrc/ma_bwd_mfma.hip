@@ -1,0 +1,452 @@
+// Backward stages on the matrix cores (v_mfma_f32_16x16x4_f32), for every
+// operand dtype: a workgroup stages the operand tiles of its block problem in
+// LDS as fp32 (zero-padded to the tile grid), and every product of the stage
+// derivative - the formulas are at the top of ma_bwd.hip - is a small GEMM
+// between LDS matrices, read with arbitrary row / column strides so that
+// transposed operands cost nothing.  Selected when the tiles of a problem fit
+// the LDS and q, k, v share a dtype; the FMA kernels of ma_bwd.hip cover the
+// rest.  Ownership and summation order are as there: a workgroup owns every
+// row it accumulates into, so results are reproducible bit for bit.
+#include "ma_generic_dev.h"
+#include "ma_mfma_launch.h"
+
+namespace ma {
+namespace {
+
+using f32x4 = float __attribute__((ext_vector_type(4)));
+
+constexpr int kPad = 4;              // floats added to every LDS row (spreads the rows over the banks)
+constexpr size_t kLdsBudget = 156 * 1024;
+
+__host__ __device__ constexpr int up(int x, int m) { return (x + m - 1) / m * m; }
+
+// acc[t] += sum_k A(r,k) B(k, 16 t + c) for one 16-row strip of up to four 16-column tiles.
+// A(r,k) = A[r*ars + k*acs], B(k,c) = B[k*brs + c*bcs]; K is a multiple of 4.  Lane (r = lane % 16,
+// q = lane / 16) feeds A(r, k0+q) and B(k0+q, r); acc[t][v] is C(4q+v, 16t+r).
+__device__ __forceinline__ void strip_mma(f32x4 (&acc)[4], int nt, const float* A, int ars, int acs, const float* B, int brs,
+                                          int bcs, int K) {
+    const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+    const float* a = A + r * ars + q * acs;
+    const float* b = B + q * brs + r * bcs;
+    for (int k0 = 0; k0 < K; k0 += 4) {
+        const float av = a[k0 * acs];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < nt) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[k0 * brs + 16 * t * bcs], acc[t], 0, 0, 0);
+    }
+}
+
+// f(row, col, value) for every element of the strip
+template <class F>
+__device__ __forceinline__ void strip_each(const f32x4 (&acc)[4], int nt, int r0, int c0, F&& f) {
+    const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        if (t < nt) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) f(r0 + 4 * q + v, c0 + 16 * t + r, acc[t][v]);
+        }
+}
+
+// Strips of a rows x cols output (both multiples of 16) dealt to the waves; body(r0, c0, nt).
+// A strip is as wide as lets every wave have one (1, 2 or 4 tiles).
+template <int NTH, class F>
+__device__ __forceinline__ void for_strips(int rows, int cols, F&& body) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tiles = (rows / 16) * (cols / 16);
+    const int wt = tiles >= 4 * (NTH / 64) ? 4 : tiles >= 2 * (NTH / 64) ? 2 : 1;
+    const int cg = (cols / 16 + wt - 1) / wt, total = (rows / 16) * cg;
+    for (int s = wave; s < total; s += NTH / 64) {
+        const int rt = s / cg, g = s % cg;
+        body(16 * rt, 16 * wt * g, min(wt, cols / 16 - wt * g));
+    }
+}
+
+__device__ __forceinline__ void zero_acc(f32x4 (&acc)[4]) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+// rows x width floats (row stride ld) <- rows of a (.., rows, W) tensor of dtype T, converted; rows
+// for which row_ptr(i) is null and columns >= W are zero.
+// A wave takes whole rows, its lanes the columns.
+template <int NTH, class T, class RowPtr>
+__device__ __forceinline__ void stage_rows(float* dst, int ld, int rows, int width, int W, float scale, RowPtr&& row_ptr) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll 2
+    for (int i = threadIdx.x >> 6; i < rows; i += NTH / 64) {
+        const T* p = row_ptr(i);
+        for (int d = lane; d < width; d += 64) dst[i * ld + d] = (p != nullptr && d < W) ? scale * to_f(p[d]) : 0.f;
+    }
+}
+
+// softmax over columns [0, cols) of every row of U[rows][ld], in place (entries may be -inf)
+template <int NTH>
+__device__ __forceinline__ void softmax_rows_lds(float* U, int ld, int rows, int cols) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int ll = wave; ll < rows; ll += NTH / 64) {
+        float* Ul = U + ll * ld;
+        float mx = -INFINITY;
+        for (int k = lane; k < cols; k += 64) mx = fmaxf(mx, Ul[k]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int k = lane; k < cols; k += 64) {
+            const float p = expf(Ul[k] - mx);
+            Ul[k] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum);
+        for (int k = lane; k < cols; k += 64) Ul[k] = Ul[k] / sum;
+    }
+}
+
+// ---------------------------------------------------------------- Z and L stages
+// One workgroup per (e,h,j), TL query blocks l at a time (TL a multiple of 16).
+// LDS: aL[M16][ldd], W[M16][ldw] (Z: Y_j; L: gaR_j), cl[M16], cw[M16] (L: gcR_j), Qt[TL][ldd],
+// dO[TL][ldw] (Z only), qok[TL], U[TL][ldm], Gg[TL][ldm].
+template <class TQ, bool kZ, int NTH>
+__global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int TL) {
+    extern __shared__ float lds[];
+    const int M = P.M, D = P.D, B = P.B, W = kZ ? P.Dv : P.D;
+    const int M16 = up(M, 16), D16 = up(D, 16), W16 = up(W, 16);
+    const int ldd = D16 + kPad, ldw = W16 + kPad, ldm = M16 + kPad;
+    int w = blockIdx.x;
+    const int j = w % B; w /= B;
+    const int h = w % P.H, e = w / P.H;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const long long jm = (eh * B + j) * M;
+    float* aLt = lds;
+    float* Wt = aLt + M16 * ldd;
+    float* cl = Wt + M16 * ldw;
+    float* cw = cl + M16;
+    float* Qt = cw + M16;
+    float* dO = Qt + TL * ldd;
+    float* qok = dO + (kZ ? TL * ldw : 0);
+    float* U = qok + TL;
+    float* Gg = U + TL * ldm;
+
+    const TQ* aL = reinterpret_cast<const TQ*>(P.aL) + jm * D;
+    stage_rows<NTH, TQ>(aLt, ldd, M16, D16, D, 1.f, [&](int k) { return k < M ? aL + k * D : nullptr; });
+    if (kZ) {
+        const TQ* Y = reinterpret_cast<const TQ*>(P.Y) + jm * W;
+        stage_rows<NTH, TQ>(Wt, ldw, M16, W16, W, 1.f, [&](int k) { return k < M ? Y + k * static_cast<long long>(W) : nullptr; });
+    } else {
+        stage_rows<NTH, float>(Wt, ldw, M16, W16, W, 1.f,
+                          [&](int k) { return k < M ? G.gaR + ((eh * M + k) * B + j) * D : nullptr; });
+    }
+    for (int k = threadIdx.x; k < M16; k += NTH) {
+        cl[k] = k < M ? P.cL[jm + k] : 0.f;
+        cw[k] = (!kZ && k < M) ? G.gcR[(eh * M + k) * B + j] : 0.f;
+    }
+
+    for (int l0 = 0; l0 < M; l0 += TL) {
+        stage_rows<NTH, TQ>(Qt, ldd, TL, D16, D, 1.f, [&](int ll) {
+            return l0 + ll < M ? tok_row<TQ>(P.q, P.qs, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
+        });
+        if (kZ)
+            stage_rows<NTH, TQ>(dO, ldw, TL, W16, W, 1.f, [&](int ll) {
+                return l0 + ll < M ? tok_row<TQ>(G.dout, G.dos, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
+            });
+        for (int ll = threadIdx.x; ll < TL; ll += NTH)
+            qok[ll] = (l0 + ll < M && token_ok(P, e, (l0 + ll) * B + j - P.pad_off)) ? 1.f : 0.f;
+        __syncthreads();
+
+        // U = round(Qt aL^T) - cL, -inf in the columns beyond M
+        for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, Qt + r0 * ldd, ldd, 1, aLt + c0 * ldd, 1, ldd, up(D, 4));
+            strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) { U[ll * ldm + k] = k < M ? round_to<TQ>(x) - cl[k] : -INFINITY; });
+        });
+        __syncthreads();
+        softmax_rows_lds<NTH>(U, ldm, TL, M16);
+        // Z: gLz = dO Y^T;  L: gLm = mask_q (Qt gaR^T + gcR)
+        for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, (kZ ? dO : Qt) + r0 * ldw, ldw, 1, Wt + c0 * ldw, 1, ldw, up(W, 4));
+            strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) {
+                if (!kZ) x = (k < M && qok[ll] != 0.f) ? x + cw[k] : 0.f;
+                Gg[ll * ldm + k] = x;
+            });
+        });
+        __syncthreads();
+        {   // dU = p (g - sum g p); afterwards U holds the rounded (L: query-masked) probabilities
+            const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+            for (int ll = wave; ll < TL; ll += NTH / 64) {
+                float dot = 0.f;
+                for (int k = lane; k < M16; k += 64) dot = fmaf(Gg[ll * ldm + k], U[ll * ldm + k], dot);
+                dot = wave_sum(dot);
+                const float keep = kZ ? 1.f : qok[ll];
+                for (int k = lane; k < M16; k += 64) {
+                    const float p = U[ll * ldm + k];
+                    Gg[ll * ldm + k] = p * (Gg[ll * ldm + k] - dot);
+                    U[ll * ldm + k] = keep * round_to<TQ>(p);
+                }
+            }
+        }
+        __syncthreads();
+        if (kZ) {   // gY (+)= round(Lz)^T dO
+            for_strips<NTH>(M16, W16, [&](int r0, int c0, int nt) {
+                f32x4 acc[4];
+                zero_acc(acc);
+                strip_mma(acc, nt, U + r0, 1, ldm, dO + c0, ldw, 1, TL);
+                strip_each(acc, nt, r0, c0, [&](int k, int d, float x) {
+                    if (k < M && d < W) {
+                        float* p = G.gY + (jm + k) * W + d;
+                        *p = (l0 ? *p : 0.f) + x;
+                    }
+                });
+            });
+        }
+        // gaL (+)= dU^T Qt
+        for_strips<NTH>(M16, D16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, Gg + r0, 1, ldm, Qt + c0, ldd, 1, TL);
+            strip_each(acc, nt, r0, c0, [&](int k, int d, float x) {
+                if (k < M && d < D) {
+                    float* p = G.gaL + (jm + k) * D + d;
+                    *p = (l0 ? *p : 0.f) + x;
+                }
+            });
+        });
+        for (int k = threadIdx.x; k < M; k += NTH) {   // gcL (+)= -sum_l dU
+            float acc = l0 ? G.gcL[jm + k] : 0.f;
+            for (int ll = 0; ll < TL; ++ll) acc -= Gg[ll * ldm + k];
+            G.gcL[jm + k] = acc;
+        }
+        // dq rows (l, j) += dU aL  (L: + round(Lm) gaR)
+        for_strips<NTH>(TL, D16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, Gg + r0 * ldm, ldm, 1, aLt + c0, ldd, 1, M16);
+            if (!kZ) strip_mma(acc, nt, U + r0 * ldm, ldm, 1, Wt + c0, ldw, 1, M16);
+            strip_each(acc, nt, r0, c0, [&](int ll, int d, float x) {
+                if (l0 + ll < M && d < D) G.dq[(eh * M * B + (l0 + ll) * B + j) * D + d] += x;
+            });
+        });
+        __syncthreads();
+    }
+}
+
+size_t lz_lds_floats(const Problem& P, bool z, int TL) {
+    const int M16 = up(P.M, 16), D16 = up(P.D, 16), W16 = up(z ? P.Dv : P.D, 16);
+    const size_t ldd = D16 + kPad, ldw = W16 + kPad, ldm = M16 + kPad;
+    return M16 * ldd + M16 * ldw + 2 * M16 + TL * ldd + (z ? TL * ldw : 0) + TL + 2 * TL * ldm;
+}
+
+// ---------------------------------------------------------------- R stage
+// One workgroup per key block (e,h,k), TJ query rows j at a time (TJ a multiple of 16).
+// LDS: Kt[B16][ldd], Vt[B16][ldv], kok[B16], X[TJ][ldd], Ga[TJ][ldd] (sm * gaL), Gy[TJ][ldv], c[TJ],
+// gcl[TJ], S[TJ][ldb], R[TJ][ldb], Gg[TJ][ldb].
+template <class TQ, int NTH>
+__global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int TJ, int first, int with_v) {
+    extern __shared__ float lds[];
+    const int B = P.B, M = P.M, D = P.D, Dv = P.Dv;
+    const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
+    const int ldd = D16 + kPad, ldv = V16 + kPad, ldb = B16 + kPad;
+    int w = blockIdx.x;
+    const int k = w % M; w /= M;
+    const int h = w % P.H, e = w / P.H;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const TQ* aR = reinterpret_cast<const TQ*>(P.aR) + (eh * M + k) * B * D;
+    const float* cR = P.cR + (eh * M + k) * B;
+    const float sm = P.sm_scale;
+    float* Kt = lds;
+    float* Vt = Kt + B16 * ldd;
+    float* kok = Vt + (with_v ? B16 * ldv : 0);
+    float* X = kok + B16;
+    float* Ga = X + TJ * ldd;
+    float* Gy = Ga + TJ * ldd;
+    float* c = Gy + (with_v ? TJ * ldv : 0);
+    float* gcl = c + TJ;
+    float* S = gcl + TJ;
+    float* R = S + TJ * ldb;
+    float* Gg = R + TJ * ldb;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    stage_rows<NTH, TQ>(Kt, ldd, B16, D16, D, 1.f,
+                   [&](int i) { return i < B ? tok_row<TQ>(P.k, P.ks, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
+    if (with_v)
+        stage_rows<NTH, TQ>(Vt, ldv, B16, V16, Dv, 1.f,
+                       [&](int i) { return i < B ? tok_row<TQ>(P.v, P.vs, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
+    for (int i = threadIdx.x; i < B16; i += NTH) kok[i] = (i < B && token_ok(P, e, k * B + i - P.pad_off)) ? 1.f : 0.f;
+
+    for (int j0 = 0; j0 < B; j0 += TJ) {
+        stage_rows<NTH, TQ>(X, ldd, TJ, D16, D, 1.f, [&](int jj) -> const TQ* {
+            if (j0 + jj >= B) return nullptr;
+            return first ? tok_row<TQ>(P.q, P.qs, e, h, k * B + j0 + jj - P.pad_off, P.N) : aR + (j0 + jj) * D;
+        });
+        stage_rows<NTH, float>(Ga, ldd, TJ, D16, D, sm,
+                          [&](int jj) { return j0 + jj < B ? G.gaL + ((eh * B + j0 + jj) * M + k) * D : nullptr; });
+        if (with_v)
+            stage_rows<NTH, float>(Gy, ldv, TJ, V16, Dv, 1.f, [&](int jj) {
+                return j0 + jj < B ? G.gY + ((eh * B + j0 + jj) * M + k) * static_cast<long long>(Dv) : nullptr;
+            });
+        for (int jj = threadIdx.x; jj < TJ; jj += NTH) {
+            const bool in = j0 + jj < B;
+            c[jj] = ((first || !in) ? 1.0f : cR[j0 + jj]) + P.eps;
+            gcl[jj] = in ? G.gcL[(eh * B + j0 + jj) * M + k] : 0.f;
+        }
+        __syncthreads();
+
+        // S = sm round(X K^T) / c, -inf for masked / padded keys
+        for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, X + r0 * ldd, ldd, 1, Kt + c0 * ldd, 1, ldd, up(D, 4));
+            strip_each(acc, nt, r0, c0,
+                       [&](int jj, int i, float x) { S[jj * ldb + i] = kok[i] != 0.f ? sm * round_to<TQ>(x) / c[jj] : -INFINITY; });
+        });
+        __syncthreads();
+        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // probabilities (ma_torch.py:14-18); Gg <- 1 where the clamp did not act
+            float mx = -INFINITY;
+            for (int i = lane; i < B16; i += 64) mx = fmaxf(mx, S[jj * ldb + i]);
+            mx = fmaxf(wave_max(mx), P.eps);
+            float sum = 0.f;
+            for (int i = lane; i < B16; i += 64) {
+                const float p = expf(S[jj * ldb + i] - mx);
+                R[jj * ldb + i] = p;
+                sum += p;
+            }
+            sum = wave_sum(sum) + P.eps;
+            for (int i = lane; i < B16; i += 64) {
+                const float r = R[jj * ldb + i] / sum;
+                Gg[jj * ldb + i] = (i < B && r >= kTiny) ? 1.f : 0.f;
+                R[jj * ldb + i] = i < B ? fmaxf(r, kTiny) : 0.f;
+            }
+        }
+        __syncthreads();
+        // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act
+        for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, Ga + r0 * ldd, ldd, 1, Kt + c0 * ldd, 1, ldd, up(D, 4));
+            if (with_v) strip_mma(acc, nt, Gy + r0 * ldv, ldv, 1, Vt + c0 * ldv, 1, ldv, up(Dv, 4));
+            strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) {
+                float* g = Gg + jj * ldb + i;
+                *g = *g != 0.f ? fmaf(gcl[jj], logf(R[jj * ldb + i]) + 1.0f, x) : 0.f;
+            });
+        });
+        __syncthreads();
+        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // dS, gcR; Gg <- dDot = dS sm / c; R <- round(r)
+            float dot = 0.f;
+            for (int i = lane; i < B16; i += 64) dot = fmaf(Gg[jj * ldb + i], R[jj * ldb + i], dot);
+            dot = wave_sum(dot);
+            float gc = 0.f;
+            for (int i = lane; i < B16; i += 64) {
+                const float s = S[jj * ldb + i], r = R[jj * ldb + i];
+                const float ds = s == -INFINITY ? 0.f : r * (Gg[jj * ldb + i] - dot);
+                if (s != -INFINITY) gc = fmaf(-ds, s / c[jj], gc);
+                Gg[jj * ldb + i] = ds * sm / c[jj];
+                R[jj * ldb + i] = round_to<TQ>(r);
+            }
+            gc = wave_sum(gc);
+            if (!first && lane == 0 && j0 + jj < B) G.gcR[(eh * M + k) * B + j0 + jj] = gc;
+        }
+        __syncthreads();
+        // gaR = dDot K (first step: aR is q, the rows of block k of dq)
+        for_strips<NTH>(TJ, D16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, Gg + r0 * ldb, ldb, 1, Kt + c0, ldd, 1, B16);
+            strip_each(acc, nt, r0, c0, [&](int jj, int d, float x) {
+                if (j0 + jj < B && d < D) {
+                    const long long row = (eh * M + k) * B + j0 + jj;
+                    if (first) G.dq[row * D + d] += x;
+                    else G.gaR[row * D + d] = x;
+                }
+            });
+        });
+        // dK += round(r)^T (sm gaL) + dDot^T X
+        for_strips<NTH>(B16, D16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, R + r0, 1, ldb, Ga + c0, ldd, 1, TJ);
+            strip_mma(acc, nt, Gg + r0, 1, ldb, X + c0, ldd, 1, TJ);
+            strip_each(acc, nt, r0, c0, [&](int i, int d, float x) {
+                if (i < B && d < D) G.dk[((eh * M + k) * B + i) * D + d] += x;
+            });
+        });
+        if (with_v)   // dV += round(r)^T gY
+            for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
+                f32x4 acc[4];
+                zero_acc(acc);
+                strip_mma(acc, nt, R + r0, 1, ldb, Gy + c0, ldv, 1, TJ);
+                strip_each(acc, nt, r0, c0, [&](int i, int d, float x) {
+                    if (i < B && d < Dv) G.dv[((eh * M + k) * B + i) * static_cast<long long>(Dv) + d] += x;
+                });
+            });
+        __syncthreads();
+    }
+}
+
+size_t r_lds_floats(const Problem& P, bool with_v, int TJ) {
+    const int B16 = up(P.B, 16), D16 = up(P.D, 16), V16 = up(P.Dv, 16);
+    const size_t ldd = D16 + kPad, ldv = V16 + kPad, ldb = B16 + kPad;
+    return B16 * ldd + (with_v ? B16 * ldv : 0) + B16 + 2 * TJ * ldd + (with_v ? TJ * ldv : 0) + 2 * TJ + 3 * TJ * ldb;
+}
+
+// largest tile (multiple of 16, at most the padded extent) whose LDS fits; 0 if none
+template <class F>
+int pick_tile(int extent, F&& floats) {
+    for (int t = up(extent, 16); t >= 16; t -= 16)
+        if (floats(t) * sizeof(float) <= kLdsBudget) return t;
+    return 0;
+}
+
+// threads per workgroup for a stage whose probability matrix has `tiles` 16 x 16 tiles
+int threads_for(int tiles) { return tiles <= 2 ? 64 : tiles <= 8 ? 256 : 1024; }
+
+template <class F>
+int dispatch16(int dt, F&& f) {
+    switch (dt) {
+        case MA_F32: return f(float{});
+        case MA_F16: return f(f16{});
+        default: return f(bf16{});
+    }
+}
+
+}  // namespace
+
+// Each returns MA_ERR_UNSUPPORTED when the problem does not fit; the caller then takes the FMA kernel.
+int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z, hipStream_t s) {
+    const int TL = pick_tile(P.M, [&](int t) { return lz_lds_floats(P, z, t); });
+    if (TL == 0) return MA_ERR_UNSUPPORTED;
+    const size_t lds = lz_lds_floats(P, z, TL) * sizeof(float);
+    const int nth = threads_for((TL / 16) * (up(P.M, 16) / 16));
+    return dispatch16(dt_qk, [&](auto tq) {
+        using TQ = decltype(tq);
+        auto launch = [&](auto kernel) {
+            const int attr = mfma::set_lds_limit(kernel, kLdsBudget);
+            if (attr) return attr;
+            hipLaunchKernelGGL(kernel, dim3(P.E * P.H * P.B), dim3(nth), lds, s, P, G, TL);
+            return static_cast<int>(hipGetLastError());
+        };
+        if (nth == 64) return z ? launch(lz_bwd_mfma<TQ, true, 64>) : launch(lz_bwd_mfma<TQ, false, 64>);
+        if (nth == 256) return z ? launch(lz_bwd_mfma<TQ, true, 256>) : launch(lz_bwd_mfma<TQ, false, 256>);
+        return z ? launch(lz_bwd_mfma<TQ, true, 1024>) : launch(lz_bwd_mfma<TQ, false, 1024>);
+    });
+}
+
+int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool first, bool with_v, hipStream_t s) {
+    const int TJ = pick_tile(P.B, [&](int t) { return r_lds_floats(P, with_v, t); });
+    if (TJ == 0) return MA_ERR_UNSUPPORTED;
+    const size_t lds = r_lds_floats(P, with_v, TJ) * sizeof(float);
+    const int nth = threads_for((TJ / 16) * (up(P.B, 16) / 16));
+    return dispatch16(dt_qk, [&](auto tq) {
+        using TQ = decltype(tq);
+        auto launch = [&](auto kernel) {
+            const int attr = mfma::set_lds_limit(kernel, kLdsBudget);
+            if (attr) return attr;
+            hipLaunchKernelGGL(kernel, dim3(P.E * P.H * P.M), dim3(nth), lds, s, P, G, TJ, first ? 1 : 0, with_v ? 1 : 0);
+            return static_cast<int>(hipGetLastError());
+        };
+        if (nth == 64) return launch(r_bwd_mfma<TQ, 64>);
+        if (nth == 256) return launch(r_bwd_mfma<TQ, 256>);
+        return launch(r_bwd_mfma<TQ, 1024>);
+    });
+}
+
+}  // namespace ma
