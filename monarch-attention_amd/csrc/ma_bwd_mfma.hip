@@ -15,24 +15,49 @@ namespace {
 
 using f32x4 = float __attribute__((ext_vector_type(4)));
 
-constexpr int kPad = 4;              // floats added to every LDS row (spreads the rows over the banks)
+// Row stride of an LDS matrix with n (a multiple of 16) columns.  The GEMM operands are read both
+// as (row = lane % 16, column = lane / 16) and as (row = lane / 16, column = lane % 16); a stride of
+// 12 or 20 (mod 32) floats keeps the first pattern free of bank conflicts and the second nearly so.
+__host__ __device__ constexpr int ld_of(int n) { return n + (n % 32 == 0 ? 12 : 4); }
 constexpr size_t kLdsBudget = 156 * 1024;
 
 __host__ __device__ constexpr int up(int x, int m) { return (x + m - 1) / m * m; }
 
+// all-reduce over the wave on the VALU (DPP within 16-lane rows, lane swaps across them)
+__device__ __forceinline__ float wmax(float x) { return mfma::quad_rows_max(mfma::row16_max(x)); }
+__device__ __forceinline__ float wsum(float x) { return mfma::quad_rows_sum(mfma::row16_sum(x)); }
+
 // acc[t] += sum_k A(r,k) B(k, 16 t + c) for one 16-row strip of up to four 16-column tiles.
-// A(r,k) = A[r*ars + k*acs], B(k,c) = B[k*brs + c*bcs]; K is a multiple of 4.  Lane (r = lane % 16,
-// q = lane / 16) feeds A(r, k0+q) and B(k0+q, r); acc[t][v] is C(4q+v, 16t+r).
-__device__ __forceinline__ void strip_mma(f32x4 (&acc)[4], int nt, const float* A, int ars, int acs, const float* B, int brs,
-                                          int bcs, int K) {
+// A(r,k) = A[r*ars + k*acs], B(k,c) = B[k*brs + c*bcs]; K is a multiple of 16.  Lane (r = lane % 16,
+// q = lane / 16) feeds A(r, k0+q) and B(k0+q, r); acc[t][v] is C(4q+v, 16t+r).  The operands of four
+// k-steps are read before their MFMAs are issued, so that the LDS reads overlap.
+template <int NT>
+__device__ __forceinline__ void strip_mma_n(f32x4 (&acc)[4], const float* A, int ars, int acs, const float* B, int brs, int bcs,
+                                            int K) {
     const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
     const float* a = A + r * ars + q * acs;
     const float* b = B + q * brs + r * bcs;
-    for (int k0 = 0; k0 < K; k0 += 4) {
-        const float av = a[k0 * acs];
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        float av[4], bv[4][NT];
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (t < nt) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[k0 * brs + 16 * t * bcs], acc[t], 0, 0, 0);
+        for (int u = 0; u < 4; ++u) {
+            av[u] = a[(k0 + 4 * u) * acs];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) bv[u][t] = b[(k0 + 4 * u) * brs + 16 * t * bcs];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u][t], acc[t], 0, 0, 0);
+    }
+}
+__device__ __forceinline__ void strip_mma(f32x4 (&acc)[4], int nt, const float* A, int ars, int acs, const float* B, int brs,
+                                          int bcs, int K) {
+    switch (nt) {   // nt is the same for every lane of the wave
+        case 1: return strip_mma_n<1>(acc, A, ars, acs, B, brs, bcs, K);
+        case 2: return strip_mma_n<2>(acc, A, ars, acs, B, brs, bcs, K);
+        case 3: return strip_mma_n<3>(acc, A, ars, acs, B, brs, bcs, K);
+        default: return strip_mma_n<4>(acc, A, ars, acs, B, brs, bcs, K);
     }
 }
 
@@ -46,6 +71,28 @@ __device__ __forceinline__ void strip_each(const f32x4 (&acc)[4], int nt, int r0
 #pragma unroll
             for (int v = 0; v < 4; ++v) f(r0 + 4 * q + v, c0 + 16 * t + r, acc[t][v]);
         }
+}
+
+// *addr(row, col) = (accumulate ? *addr : 0) + value for every element of the strip whose addr is
+// not null.  All old values are loaded before the first store: the loads are in flight together
+// instead of one memory round trip per element.
+template <class F>
+__device__ __forceinline__ void strip_rmw(const f32x4 (&acc)[4], int nt, int r0, int c0, bool accumulate, F&& addr) {
+    const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+    float* p[16];
+    float old[16];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            p[4 * t + v] = t < nt ? addr(r0 + 4 * q + v, c0 + 16 * t + r) : nullptr;
+            old[4 * t + v] = (accumulate && p[4 * t + v] != nullptr) ? *p[4 * t + v] : 0.f;
+        }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            if (p[4 * t + v] != nullptr) *p[4 * t + v] = old[4 * t + v] + acc[t][v];
 }
 
 // Strips of a rows x cols output (both multiples of 16) dealt to the waves; body(r0, c0, nt).
@@ -69,14 +116,41 @@ __device__ __forceinline__ void zero_acc(f32x4 (&acc)[4]) {
 
 // rows x width floats (row stride ld) <- rows of a (.., rows, W) tensor of dtype T, converted; rows
 // for which row_ptr(i) is null and columns >= W are zero.
-// A wave takes whole rows, its lanes the columns.
+// Sixteen lanes take a row, four elements each (one 8- or 16-byte load where the row allows it),
+// so a wave loads four rows per instruction; two such groups are in flight together.
 template <int NTH, class T, class RowPtr>
 __device__ __forceinline__ void stage_rows(float* dst, int ld, int rows, int width, int W, float scale, RowPtr&& row_ptr) {
-    const int lane = threadIdx.x & 63;
-#pragma unroll 2
-    for (int i = threadIdx.x >> 6; i < rows; i += NTH / 64) {
-        const T* p = row_ptr(i);
-        for (int d = lane; d < width; d += 64) dst[i * ld + d] = (p != nullptr && d < W) ? scale * to_f(p[d]) : 0.f;
+    constexpr int NW = NTH / 64;
+    struct alignas(4 * sizeof(T)) Quad { T v[4]; };
+    const int lane = threadIdx.x & 63, sub = lane >> 4, c0 = lane & 15;
+    for (int i0 = 4 * (threadIdx.x >> 6) + sub; i0 < rows; i0 += 8 * NW) {
+        const T* p[2];
+        bool vec[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int i = i0 + 4 * NW * u;
+            p[u] = i < rows ? row_ptr(i) : nullptr;
+            vec[u] = W % 4 == 0 && reinterpret_cast<uintptr_t>(p[u]) % sizeof(Quad) == 0;
+        }
+        for (int c = c0; 4 * c < width; c += 16) {
+            float x[2][4];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                if (p[u] != nullptr && vec[u] && 4 * c < W) {
+                    const Quad qd = *reinterpret_cast<const Quad*>(p[u] + 4 * c);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x[u][e] = scale * to_f(qd.v[e]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x[u][e] = (p[u] != nullptr && 4 * c + e < W) ? scale * to_f(p[u][4 * c + e]) : 0.f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int i = i0 + 4 * NW * u;
+                if (i < rows) *reinterpret_cast<f32x4*>(dst + i * ld + 4 * c) = f32x4{x[u][0], x[u][1], x[u][2], x[u][3]};
+            }
+        }
     }
 }
 
@@ -88,14 +162,14 @@ __device__ __forceinline__ void softmax_rows_lds(float* U, int ld, int rows, int
         float* Ul = U + ll * ld;
         float mx = -INFINITY;
         for (int k = lane; k < cols; k += 64) mx = fmaxf(mx, Ul[k]);
-        mx = wave_max(mx);
+        mx = wmax(mx);
         float sum = 0.f;
         for (int k = lane; k < cols; k += 64) {
             const float p = expf(Ul[k] - mx);
             Ul[k] = p;
             sum += p;
         }
-        sum = wave_sum(sum);
+        sum = wsum(sum);
         for (int k = lane; k < cols; k += 64) Ul[k] = Ul[k] / sum;
     }
 }
@@ -109,7 +183,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
     extern __shared__ float lds[];
     const int M = P.M, D = P.D, B = P.B, W = kZ ? P.Dv : P.D;
     const int M16 = up(M, 16), D16 = up(D, 16), W16 = up(W, 16);
-    const int ldd = D16 + kPad, ldw = W16 + kPad, ldm = M16 + kPad;
+    const int ldd = ld_of(D16), ldw = ld_of(W16), ldm = ld_of(M16);
     int w = blockIdx.x;
     const int j = w % B; w /= B;
     const int h = w % P.H, e = w / P.H;
@@ -155,7 +229,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
         for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma(acc, nt, Qt + r0 * ldd, ldd, 1, aLt + c0 * ldd, 1, ldd, up(D, 4));
+            strip_mma(acc, nt, Qt + r0 * ldd, ldd, 1, aLt + c0 * ldd, 1, ldd, D16);
             strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) { U[ll * ldm + k] = k < M ? round_to<TQ>(x) - cl[k] : -INFINITY; });
         });
         __syncthreads();
@@ -164,7 +238,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
         for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma(acc, nt, (kZ ? dO : Qt) + r0 * ldw, ldw, 1, Wt + c0 * ldw, 1, ldw, up(W, 4));
+            strip_mma(acc, nt, (kZ ? dO : Qt) + r0 * ldw, ldw, 1, Wt + c0 * ldw, 1, ldw, W16);
             strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) {
                 if (!kZ) x = (k < M && qok[ll] != 0.f) ? x + cw[k] : 0.f;
                 Gg[ll * ldm + k] = x;
@@ -176,7 +250,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             for (int ll = wave; ll < TL; ll += NTH / 64) {
                 float dot = 0.f;
                 for (int k = lane; k < M16; k += 64) dot = fmaf(Gg[ll * ldm + k], U[ll * ldm + k], dot);
-                dot = wave_sum(dot);
+                dot = wsum(dot);
                 const float keep = kZ ? 1.f : qok[ll];
                 for (int k = lane; k < M16; k += 64) {
                     const float p = U[ll * ldm + k];
@@ -191,12 +265,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma(acc, nt, U + r0, 1, ldm, dO + c0, ldw, 1, TL);
-                strip_each(acc, nt, r0, c0, [&](int k, int d, float x) {
-                    if (k < M && d < W) {
-                        float* p = G.gY + (jm + k) * W + d;
-                        *p = (l0 ? *p : 0.f) + x;
-                    }
-                });
+                strip_rmw(acc, nt, r0, c0, l0 != 0,
+                          [&](int k, int d) -> float* { return (k < M && d < W) ? G.gY + (jm + k) * W + d : nullptr; });
             });
         }
         // gaL (+)= dU^T Qt
@@ -204,15 +274,12 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma(acc, nt, Gg + r0, 1, ldm, Qt + c0, ldd, 1, TL);
-            strip_each(acc, nt, r0, c0, [&](int k, int d, float x) {
-                if (k < M && d < D) {
-                    float* p = G.gaL + (jm + k) * D + d;
-                    *p = (l0 ? *p : 0.f) + x;
-                }
-            });
+            strip_rmw(acc, nt, r0, c0, l0 != 0,
+                      [&](int k, int d) -> float* { return (k < M && d < D) ? G.gaL + (jm + k) * D + d : nullptr; });
         });
         for (int k = threadIdx.x; k < M; k += NTH) {   // gcL (+)= -sum_l dU
             float acc = l0 ? G.gcL[jm + k] : 0.f;
+#pragma unroll 8
             for (int ll = 0; ll < TL; ++ll) acc -= Gg[ll * ldm + k];
             G.gcL[jm + k] = acc;
         }
@@ -222,8 +289,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             zero_acc(acc);
             strip_mma(acc, nt, Gg + r0 * ldm, ldm, 1, aLt + c0, ldd, 1, M16);
             if (!kZ) strip_mma(acc, nt, U + r0 * ldm, ldm, 1, Wt + c0, ldw, 1, M16);
-            strip_each(acc, nt, r0, c0, [&](int ll, int d, float x) {
-                if (l0 + ll < M && d < D) G.dq[(eh * M * B + (l0 + ll) * B + j) * D + d] += x;
+            strip_rmw(acc, nt, r0, c0, true, [&](int ll, int d) -> float* {
+                return (l0 + ll < M && d < D) ? G.dq + (eh * M * B + (l0 + ll) * B + j) * D + d : nullptr;
             });
         });
         __syncthreads();
@@ -232,7 +299,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
 
 size_t lz_lds_floats(const Problem& P, bool z, int TL) {
     const int M16 = up(P.M, 16), D16 = up(P.D, 16), W16 = up(z ? P.Dv : P.D, 16);
-    const size_t ldd = D16 + kPad, ldw = W16 + kPad, ldm = M16 + kPad;
+    const size_t ldd = ld_of(D16), ldw = ld_of(W16), ldm = ld_of(M16);
     return M16 * ldd + M16 * ldw + 2 * M16 + TL * ldd + (z ? TL * ldw : 0) + TL + 2 * TL * ldm;
 }
 
@@ -245,7 +312,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
     extern __shared__ float lds[];
     const int B = P.B, M = P.M, D = P.D, Dv = P.Dv;
     const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
-    const int ldd = D16 + kPad, ldv = V16 + kPad, ldb = B16 + kPad;
+    const int ldd = ld_of(D16), ldv = ld_of(V16), ldb = ld_of(B16);
     int w = blockIdx.x;
     const int k = w % M; w /= M;
     const int h = w % P.H, e = w / P.H;
@@ -295,7 +362,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
         for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma(acc, nt, X + r0 * ldd, ldd, 1, Kt + c0 * ldd, 1, ldd, up(D, 4));
+            strip_mma(acc, nt, X + r0 * ldd, ldd, 1, Kt + c0 * ldd, 1, ldd, D16);
             strip_each(acc, nt, r0, c0,
                        [&](int jj, int i, float x) { S[jj * ldb + i] = kok[i] != 0.f ? sm * round_to<TQ>(x) / c[jj] : -INFINITY; });
         });
@@ -303,14 +370,14 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
         for (int jj = wave; jj < TJ; jj += NTH / 64) {   // probabilities (ma_torch.py:14-18); Gg <- 1 where the clamp did not act
             float mx = -INFINITY;
             for (int i = lane; i < B16; i += 64) mx = fmaxf(mx, S[jj * ldb + i]);
-            mx = fmaxf(wave_max(mx), P.eps);
+            mx = fmaxf(wmax(mx), P.eps);
             float sum = 0.f;
             for (int i = lane; i < B16; i += 64) {
                 const float p = expf(S[jj * ldb + i] - mx);
                 R[jj * ldb + i] = p;
                 sum += p;
             }
-            sum = wave_sum(sum) + P.eps;
+            sum = wsum(sum) + P.eps;
             for (int i = lane; i < B16; i += 64) {
                 const float r = R[jj * ldb + i] / sum;
                 Gg[jj * ldb + i] = (i < B && r >= kTiny) ? 1.f : 0.f;
@@ -322,8 +389,8 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
         for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma(acc, nt, Ga + r0 * ldd, ldd, 1, Kt + c0 * ldd, 1, ldd, up(D, 4));
-            if (with_v) strip_mma(acc, nt, Gy + r0 * ldv, ldv, 1, Vt + c0 * ldv, 1, ldv, up(Dv, 4));
+            strip_mma(acc, nt, Ga + r0 * ldd, ldd, 1, Kt + c0 * ldd, 1, ldd, D16);
+            if (with_v) strip_mma(acc, nt, Gy + r0 * ldv, ldv, 1, Vt + c0 * ldv, 1, ldv, V16);
             strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) {
                 float* g = Gg + jj * ldb + i;
                 *g = *g != 0.f ? fmaf(gcl[jj], logf(R[jj * ldb + i]) + 1.0f, x) : 0.f;
@@ -333,7 +400,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
         for (int jj = wave; jj < TJ; jj += NTH / 64) {   // dS, gcR; Gg <- dDot = dS sm / c; R <- round(r)
             float dot = 0.f;
             for (int i = lane; i < B16; i += 64) dot = fmaf(Gg[jj * ldb + i], R[jj * ldb + i], dot);
-            dot = wave_sum(dot);
+            dot = wsum(dot);
             float gc = 0.f;
             for (int i = lane; i < B16; i += 64) {
                 const float s = S[jj * ldb + i], r = R[jj * ldb + i];
@@ -342,7 +409,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
                 Gg[jj * ldb + i] = ds * sm / c[jj];
                 R[jj * ldb + i] = round_to<TQ>(r);
             }
-            gc = wave_sum(gc);
+            gc = wsum(gc);
             if (!first && lane == 0 && j0 + jj < B) G.gcR[(eh * M + k) * B + j0 + jj] = gc;
         }
         __syncthreads();
@@ -351,12 +418,9 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma(acc, nt, Gg + r0 * ldb, ldb, 1, Kt + c0, ldd, 1, B16);
-            strip_each(acc, nt, r0, c0, [&](int jj, int d, float x) {
-                if (j0 + jj < B && d < D) {
-                    const long long row = (eh * M + k) * B + j0 + jj;
-                    if (first) G.dq[row * D + d] += x;
-                    else G.gaR[row * D + d] = x;
-                }
+            strip_rmw(acc, nt, r0, c0, first != 0, [&](int jj, int d) -> float* {
+                if (j0 + jj >= B || d >= D) return nullptr;
+                return (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0 + jj) * D + d;
             });
         });
         // dK += round(r)^T (sm gaL) + dDot^T X
@@ -365,17 +429,16 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             zero_acc(acc);
             strip_mma(acc, nt, R + r0, 1, ldb, Ga + c0, ldd, 1, TJ);
             strip_mma(acc, nt, Gg + r0, 1, ldb, X + c0, ldd, 1, TJ);
-            strip_each(acc, nt, r0, c0, [&](int i, int d, float x) {
-                if (i < B && d < D) G.dk[((eh * M + k) * B + i) * D + d] += x;
-            });
+            strip_rmw(acc, nt, r0, c0, true,
+                      [&](int i, int d) -> float* { return (i < B && d < D) ? G.dk + ((eh * M + k) * B + i) * D + d : nullptr; });
         });
         if (with_v)   // dV += round(r)^T gY
             for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma(acc, nt, R + r0, 1, ldb, Gy + c0, ldv, 1, TJ);
-                strip_each(acc, nt, r0, c0, [&](int i, int d, float x) {
-                    if (i < B && d < Dv) G.dv[((eh * M + k) * B + i) * static_cast<long long>(Dv) + d] += x;
+                strip_rmw(acc, nt, r0, c0, true, [&](int i, int d) -> float* {
+                    return (i < B && d < Dv) ? G.dv + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d : nullptr;
                 });
             });
         __syncthreads();
@@ -384,7 +447,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
 
 size_t r_lds_floats(const Problem& P, bool with_v, int TJ) {
     const int B16 = up(P.B, 16), D16 = up(P.D, 16), V16 = up(P.Dv, 16);
-    const size_t ldd = D16 + kPad, ldv = V16 + kPad, ldb = B16 + kPad;
+    const size_t ldd = ld_of(D16), ldv = ld_of(V16), ldb = ld_of(B16);
     return B16 * ldd + (with_v ? B16 * ldv : 0) + B16 + 2 * TJ * ldd + (with_v ? TJ * ldv : 0) + 2 * TJ + 3 * TJ * ldb;
 }
 
