@@ -42,6 +42,7 @@ CONFIGS = {  # name: (E, H, N, D, B, T, dtype, scale)  - BASELINE.json configs +
     # model shapes beyond the BASELINE configs (fp32 goes through the fp32 matrix-core stage kernels)
     "gps": (1, 2, 7600, 48, 128, 2, "f32", 1.0),
     "c3f32": (16, 12, 512, 64, 32, 2, "f32", 1.0),
+    "bart": (2, 16, 8192, 64, 64, 2, "bf16", 1.0),
 }
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
@@ -71,6 +72,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sdpa", action="store_true", help="skip the dense SDPA comparison")
     ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep")
+    ap.add_argument("--backward", action="store_true",
+                    help="time ma_bwd (gradients of q, k, v; runs the T steps again) instead of the forward metric")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE GPU (heads are independent problems: more GPUs would each take "
@@ -133,6 +136,25 @@ def main():
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
         return wall_ms, e0.elapsed_time(e1) / steps, ps, ws
+
+    if args.backward:
+        from ma.ma_hip import monarch_attention_hip_backward
+        q, k, v, _ = sets[0]
+        w = torch.randn(E, H, N, D, generator=gen).to(dtype).to(dev)
+        variant = args.variant if args.variant in ("auto", "generic", "staged") else "auto"
+        for _ in range(max(args.warmup // 10, 2)):
+            monarch_attention_hip_backward(q, k, v, None, w, T, B, False, variant=variant)
+        torch.cuda.synchronize()
+        steps = max(args.steps // 10, 5)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            monarch_attention_hip_backward(q, k, v, None, w, T, B, False, variant=variant)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        print(json.dumps({"metric": "ma_bwd_ms", "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": steps,
+                          "higher_is_better": False, "dtype": dt, "data": "synthetic",
+                          "config": {"workload": f"{args.config}: E{E} H{H} N{N} D{D} block {B} T={T}", "variant": variant}}))
+        return
 
     resolved = L.VARIANT_NAMES[lib.ma_fwd_select_variant(make_params(*sets[0][:3], None, sets[0][3], T, B, False, args.variant))]
     flops = forward_flops(E, H, N, D, D, B, T)
