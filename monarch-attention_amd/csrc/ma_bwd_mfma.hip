@@ -1,6 +1,7 @@
 // Backward stages on the matrix cores (v_mfma_f32_16x16x4_f32), for every
 // operand dtype: a workgroup stages the operand tiles of its block problem in
-// LDS as fp32 (zero-padded to the tile grid), and every product of the stage
+// LDS (zero-padded to the tile grid; tiles of q, k, v and of the 16-bit state in
+// their own dtype, gradients and probabilities as fp32), and every product of the stage
 // derivative - the formulas are at the top of ma_bwd.hip - is a small GEMM
 // between LDS matrices, read with arbitrary row / column strides so that
 // transposed operands cost nothing.  Selected when the tiles of a problem fit
@@ -9,6 +10,8 @@
 // row it accumulates into, so results are reproducible bit for bit.
 #include "ma_generic_dev.h"
 #include "ma_mfma_launch.h"
+
+#include <type_traits>
 
 namespace ma {
 namespace {
@@ -19,6 +22,12 @@ using f32x4 = float __attribute__((ext_vector_type(4)));
 // as (row = lane % 16, column = lane / 16) and as (row = lane / 16, column = lane % 16); a stride of
 // 12 or 20 (mod 32) floats keeps the first pattern free of bank conflicts and the second nearly so.
 __host__ __device__ constexpr int ld_of(int n) { return n + (n % 32 == 0 ? 12 : 4); }
+// The same for a matrix of T: 16-bit rows take a stride of 2 w elements with w = 9 (mod 16) 32-bit
+// words, which does for the two read patterns what 12 / 20 (mod 32) does for fp32.
+template <class T>
+__host__ __device__ constexpr int ld_t(int n) {
+    return sizeof(T) == 4 ? ld_of(n) : 2 * ((n / 2 + 6) / 16 * 16 + 9);
+}
 constexpr size_t kLdsBudget = 156 * 1024;
 
 __host__ __device__ constexpr int up(int x, int m) { return (x + m - 1) / m * m; }
@@ -31,19 +40,18 @@ __device__ __forceinline__ float wsum(float x) { return mfma::quad_rows_sum(mfma
 // A(r,k) = A[r*ars + k*acs], B(k,c) = B[k*brs + c*bcs]; K is a multiple of 16.  Lane (r = lane % 16,
 // q = lane / 16) feeds A(r, k0+q) and B(k0+q, r); acc[t][v] is C(4q+v, 16t+r).  The operands of four
 // k-steps are read before their MFMAs are issued, so that the LDS reads overlap.
-template <int NT>
-__device__ __forceinline__ void strip_mma_n(f32x4 (&acc)[4], const float* A, int ars, int acs, const float* B, int brs, int bcs,
-                                            int K) {
+template <int NT, class TA, class TB>
+__device__ __forceinline__ void strip_mma_n(f32x4 (&acc)[4], const TA* A, int ars, int acs, const TB* B, int brs, int bcs, int K) {
     const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
-    const float* a = A + r * ars + q * acs;
-    const float* b = B + q * brs + r * bcs;
+    const TA* a = A + r * ars + q * acs;
+    const TB* b = B + q * brs + r * bcs;
     for (int k0 = 0; k0 < K; k0 += 16) {
         float av[4], bv[4][NT];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            av[u] = a[(k0 + 4 * u) * acs];
+            av[u] = to_f(a[(k0 + 4 * u) * acs]);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) bv[u][t] = b[(k0 + 4 * u) * brs + 16 * t * bcs];
+            for (int t = 0; t < NT; ++t) bv[u][t] = to_f(b[(k0 + 4 * u) * brs + 16 * t * bcs]);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u)
@@ -51,8 +59,9 @@ __device__ __forceinline__ void strip_mma_n(f32x4 (&acc)[4], const float* A, int
             for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u][t], acc[t], 0, 0, 0);
     }
 }
-__device__ __forceinline__ void strip_mma(f32x4 (&acc)[4], int nt, const float* A, int ars, int acs, const float* B, int brs,
-                                          int bcs, int K) {
+template <class TA, class TB>
+__device__ __forceinline__ void strip_mma(f32x4 (&acc)[4], int nt, const TA* A, int ars, int acs, const TB* B, int brs, int bcs,
+                                          int K) {
     switch (nt) {   // nt is the same for every lane of the wave
         case 1: return strip_mma_n<1>(acc, A, ars, acs, B, brs, bcs, K);
         case 2: return strip_mma_n<2>(acc, A, ars, acs, B, brs, bcs, K);
@@ -114,14 +123,16 @@ __device__ __forceinline__ void zero_acc(f32x4 (&acc)[4]) {
     for (int t = 0; t < 4; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
-// rows x width floats (row stride ld) <- rows of a (.., rows, W) tensor of dtype T, converted; rows
-// for which row_ptr(i) is null and columns >= W are zero.
-// Sixteen lanes take a row, four elements each (one 8- or 16-byte load where the row allows it),
-// so a wave loads four rows per instruction; two such groups are in flight together.
-template <int NTH, class T, class RowPtr>
-__device__ __forceinline__ void stage_rows(float* dst, int ld, int rows, int width, int W, float scale, RowPtr&& row_ptr) {
+// rows x width elements of TD (row stride ld) <- rows of a (.., rows, W) tensor of dtype T; TD is T
+// itself (copied as is) or float (converted, times scale); rows for which row_ptr(i) is null and
+// columns >= W are zero.  Sixteen lanes take a row, four elements each (one 8- or 16-byte load where
+// the row allows it), so a wave loads four rows per instruction; two such groups are in flight
+// together.
+template <int NTH, class T, class TD, class RowPtr>
+__device__ __forceinline__ void stage_rows(TD* dst, int ld, int rows, int width, int W, float scale, RowPtr&& row_ptr) {
     constexpr int NW = NTH / 64;
     struct alignas(4 * sizeof(T)) Quad { T v[4]; };
+    struct alignas(2 * sizeof(T)) Pair { T a, b; };
     const int lane = threadIdx.x & 63, sub = lane >> 4, c0 = lane & 15;
     for (int i0 = 4 * (threadIdx.x >> 6) + sub; i0 < rows; i0 += 8 * NW) {
         const T* p[2];
@@ -133,22 +144,27 @@ __device__ __forceinline__ void stage_rows(float* dst, int ld, int rows, int wid
             vec[u] = W % 4 == 0 && reinterpret_cast<uintptr_t>(p[u]) % sizeof(Quad) == 0;
         }
         for (int c = c0; 4 * c < width; c += 16) {
-            float x[2][4];
+            Quad x[2];
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 if (p[u] != nullptr && vec[u] && 4 * c < W) {
-                    const Quad qd = *reinterpret_cast<const Quad*>(p[u] + 4 * c);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) x[u][e] = scale * to_f(qd.v[e]);
+                    x[u] = *reinterpret_cast<const Quad*>(p[u] + 4 * c);
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) x[u][e] = (p[u] != nullptr && 4 * c + e < W) ? scale * to_f(p[u][4 * c + e]) : 0.f;
+                    for (int e = 0; e < 4; ++e) x[u].v[e] = (p[u] != nullptr && 4 * c + e < W) ? p[u][4 * c + e] : from_f<T>(0.f);
                 }
             }
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int i = i0 + 4 * NW * u;
-                if (i < rows) *reinterpret_cast<f32x4*>(dst + i * ld + 4 * c) = f32x4{x[u][0], x[u][1], x[u][2], x[u][3]};
+                if (i >= rows) continue;
+                if constexpr (sizeof(TD) == 4) {
+                    *reinterpret_cast<f32x4*>(dst + i * ld + 4 * c) = f32x4{scale * to_f(x[u].v[0]), scale * to_f(x[u].v[1]),
+                                                                           scale * to_f(x[u].v[2]), scale * to_f(x[u].v[3])};
+                } else {   // 16-bit rows start on 4-byte boundaries only
+                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c) = Pair{x[u].v[0], x[u].v[1]};
+                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c + 2) = Pair{x[u].v[2], x[u].v[3]};
+                }
             }
         }
     }
@@ -175,38 +191,69 @@ __device__ __forceinline__ void softmax_rows_lds(float* U, int ld, int rows, int
 }
 
 // ---------------------------------------------------------------- Z and L stages
+// LDS of the Z / L stage for tiles of TL query blocks: byte offsets and row strides (elements).
+//   aL[M16][ldd] TQ, W[M16][ldw] (Z: Y_j, TQ; L: gaR_j, float), cl[M16], cw[M16] (L: gcR_j),
+//   Qt[TL][ldd] TQ, dO[TL][ldo] TQ (Z only), qok[TL], U[TL][ldm], Gg[TL][ldm]
+struct LzLayout {
+    int ldd, ldw, ldo, ldm;
+    unsigned aLt, Wt, cl, cw, Qt, dO, qok, U, Gg, total;
+};
+template <class TQ>
+__host__ __device__ inline LzLayout lz_layout(int M, int D, int W, bool z, int TL) {
+    const int M16 = up(M, 16), D16 = up(D, 16), W16 = up(W, 16);
+    LzLayout L;
+    L.ldd = ld_t<TQ>(D16);
+    L.ldw = z ? ld_t<TQ>(W16) : ld_of(W16);
+    L.ldo = ld_t<TQ>(W16);
+    L.ldm = ld_of(M16);
+    unsigned off = 0;
+    auto take = [&](size_t bytes) { const unsigned at = off; off += static_cast<unsigned>((bytes + 15) / 16 * 16); return at; };
+    L.aLt = take(sizeof(TQ) * M16 * L.ldd);
+    L.Wt = take((z ? sizeof(TQ) : sizeof(float)) * M16 * L.ldw);
+    L.cl = take(4 * M16);
+    L.cw = take(4 * M16);
+    L.Qt = take(sizeof(TQ) * TL * L.ldd);
+    L.dO = take(z ? sizeof(TQ) * TL * L.ldo : 0);
+    L.qok = take(4 * TL);
+    L.U = take(4 * TL * L.ldm);
+    L.Gg = take(4 * TL * L.ldm);
+    L.total = off;
+    return L;
+}
+
 // One workgroup per (e,h,j), TL query blocks l at a time (TL a multiple of 16).
-// LDS: aL[M16][ldd], W[M16][ldw] (Z: Y_j; L: gaR_j), cl[M16], cw[M16] (L: gcR_j), Qt[TL][ldd],
-// dO[TL][ldw] (Z only), qok[TL], U[TL][ldm], Gg[TL][ldm].
 template <class TQ, bool kZ, int NTH>
 __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int TL) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+    using TW = typename std::conditional<kZ, TQ, float>::type;
     const int M = P.M, D = P.D, B = P.B, W = kZ ? P.Dv : P.D;
     const int M16 = up(M, 16), D16 = up(D, 16), W16 = up(W, 16);
-    const int ldd = ld_of(D16), ldw = ld_of(W16), ldm = ld_of(M16);
+    const LzLayout L = lz_layout<TQ>(M, D, W, kZ, TL);
+    const int ldd = L.ldd, ldw = L.ldw, ldo = L.ldo, ldm = L.ldm;
     int w = blockIdx.x;
     const int j = w % B; w /= B;
     const int h = w % P.H, e = w / P.H;
     const long long eh = static_cast<long long>(e) * P.H + h;
     const long long jm = (eh * B + j) * M;
-    float* aLt = lds;
-    float* Wt = aLt + M16 * ldd;
-    float* cl = Wt + M16 * ldw;
-    float* cw = cl + M16;
-    float* Qt = cw + M16;
-    float* dO = Qt + TL * ldd;
-    float* qok = dO + (kZ ? TL * ldw : 0);
-    float* U = qok + TL;
-    float* Gg = U + TL * ldm;
+    TQ* aLt = reinterpret_cast<TQ*>(lds_raw + L.aLt);
+    TW* Wt = reinterpret_cast<TW*>(lds_raw + L.Wt);
+    float* cl = reinterpret_cast<float*>(lds_raw + L.cl);
+    float* cw = reinterpret_cast<float*>(lds_raw + L.cw);
+    TQ* Qt = reinterpret_cast<TQ*>(lds_raw + L.Qt);
+    TQ* dO = reinterpret_cast<TQ*>(lds_raw + L.dO);
+    float* qok = reinterpret_cast<float*>(lds_raw + L.qok);
+    float* U = reinterpret_cast<float*>(lds_raw + L.U);
+    float* Gg = reinterpret_cast<float*>(lds_raw + L.Gg);
 
     const TQ* aL = reinterpret_cast<const TQ*>(P.aL) + jm * D;
-    stage_rows<NTH, TQ>(aLt, ldd, M16, D16, D, 1.f, [&](int k) { return k < M ? aL + k * D : nullptr; });
+    stage_rows<NTH, TQ, TQ>(aLt, ldd, M16, D16, D, 1.f, [&](int k) { return k < M ? aL + k * D : nullptr; });
     if (kZ) {
         const TQ* Y = reinterpret_cast<const TQ*>(P.Y) + jm * W;
-        stage_rows<NTH, TQ>(Wt, ldw, M16, W16, W, 1.f, [&](int k) { return k < M ? Y + k * static_cast<long long>(W) : nullptr; });
+        stage_rows<NTH, TQ, TQ>(reinterpret_cast<TQ*>(Wt), ldw, M16, W16, W, 1.f,
+                                [&](int k) { return k < M ? Y + k * static_cast<long long>(W) : nullptr; });
     } else {
-        stage_rows<NTH, float>(Wt, ldw, M16, W16, W, 1.f,
-                          [&](int k) { return k < M ? G.gaR + ((eh * M + k) * B + j) * D : nullptr; });
+        stage_rows<NTH, float, float>(reinterpret_cast<float*>(Wt), ldw, M16, W16, W, 1.f,
+                                      [&](int k) { return k < M ? G.gaR + ((eh * M + k) * B + j) * D : nullptr; });
     }
     for (int k = threadIdx.x; k < M16; k += NTH) {
         cl[k] = k < M ? P.cL[jm + k] : 0.f;
@@ -214,11 +261,11 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
     }
 
     for (int l0 = 0; l0 < M; l0 += TL) {
-        stage_rows<NTH, TQ>(Qt, ldd, TL, D16, D, 1.f, [&](int ll) {
+        stage_rows<NTH, TQ, TQ>(Qt, ldd, TL, D16, D, 1.f, [&](int ll) {
             return l0 + ll < M ? tok_row<TQ>(P.q, P.qs, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
         });
         if (kZ)
-            stage_rows<NTH, TQ>(dO, ldw, TL, W16, W, 1.f, [&](int ll) {
+            stage_rows<NTH, TQ, TQ>(dO, ldo, TL, W16, W, 1.f, [&](int ll) {
                 return l0 + ll < M ? tok_row<TQ>(G.dout, G.dos, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
             });
         for (int ll = threadIdx.x; ll < TL; ll += NTH)
@@ -238,7 +285,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
         for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma(acc, nt, (kZ ? dO : Qt) + r0 * ldw, ldw, 1, Wt + c0 * ldw, 1, ldw, W16);
+            if (kZ) strip_mma(acc, nt, dO + r0 * ldo, ldo, 1, Wt + c0 * ldw, 1, ldw, W16);
+            else strip_mma(acc, nt, Qt + r0 * ldd, ldd, 1, Wt + c0 * ldw, 1, ldw, W16);
             strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) {
                 if (!kZ) x = (k < M && qok[ll] != 0.f) ? x + cw[k] : 0.f;
                 Gg[ll * ldm + k] = x;
@@ -264,7 +312,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             for_strips<NTH>(M16, W16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
-                strip_mma(acc, nt, U + r0, 1, ldm, dO + c0, ldw, 1, TL);
+                strip_mma(acc, nt, U + r0, 1, ldm, dO + c0, ldo, 1, TL);
                 strip_rmw(acc, nt, r0, c0, l0 != 0,
                           [&](int k, int d) -> float* { return (k < M && d < W) ? G.gY + (jm + k) * W + d : nullptr; });
             });
@@ -297,22 +345,51 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
     }
 }
 
-size_t lz_lds_floats(const Problem& P, bool z, int TL) {
-    const int M16 = up(P.M, 16), D16 = up(P.D, 16), W16 = up(z ? P.Dv : P.D, 16);
-    const size_t ldd = ld_of(D16), ldw = ld_of(W16), ldm = ld_of(M16);
-    return M16 * ldd + M16 * ldw + 2 * M16 + TL * ldd + (z ? TL * ldw : 0) + TL + 2 * TL * ldm;
-}
+template <class TQ>
+size_t lz_lds_bytes(const Problem& P, bool z, int TL) { return lz_layout<TQ>(P.M, P.D, z ? P.Dv : P.D, z, TL).total; }
 
 // ---------------------------------------------------------------- R stage
+// LDS of the R stage for tiles of TJ query rows: byte offsets and row strides (elements).
+//   Kt[B16][ldd] TQ, Vt[B16][ldv] TQ, kok[B16], X[TJ][ldd] TQ, Ga[TJ][lga] (sm * gaL), Gy[TJ][lgy],
+//   c[TJ], gcl[TJ], S[TJ][ldb], R[TJ][ldb], Gg[TJ][ldb]
+struct RLayout {
+    int ldd, ldv, lga, lgy, ldb;
+    unsigned Kt, Vt, kok, X, Ga, Gy, c, gcl, S, R, Gg, total;
+};
+template <class TQ>
+__host__ __device__ inline RLayout r_layout(int B, int D, int Dv, bool with_v, int TJ) {
+    const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
+    RLayout L;
+    L.ldd = ld_t<TQ>(D16);
+    L.ldv = ld_t<TQ>(V16);
+    L.lga = ld_of(D16);
+    L.lgy = ld_of(V16);
+    L.ldb = ld_of(B16);
+    unsigned off = 0;
+    auto take = [&](size_t bytes) { const unsigned at = off; off += static_cast<unsigned>((bytes + 15) / 16 * 16); return at; };
+    L.Kt = take(sizeof(TQ) * B16 * L.ldd);
+    L.Vt = take(with_v ? sizeof(TQ) * B16 * L.ldv : 0);
+    L.kok = take(4 * B16);
+    L.X = take(sizeof(TQ) * TJ * L.ldd);
+    L.Ga = take(4 * TJ * L.lga);
+    L.Gy = take(with_v ? 4 * TJ * L.lgy : 0);
+    L.c = take(4 * TJ);
+    L.gcl = take(4 * TJ);
+    L.S = take(4 * TJ * L.ldb);
+    L.R = take(4 * TJ * L.ldb);
+    L.Gg = take(4 * TJ * L.ldb);
+    L.total = off;
+    return L;
+}
+
 // One workgroup per key block (e,h,k), TJ query rows j at a time (TJ a multiple of 16).
-// LDS: Kt[B16][ldd], Vt[B16][ldv], kok[B16], X[TJ][ldd], Ga[TJ][ldd] (sm * gaL), Gy[TJ][ldv], c[TJ],
-// gcl[TJ], S[TJ][ldb], R[TJ][ldb], Gg[TJ][ldb].
 template <class TQ, int NTH>
 __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int TJ, int first, int with_v) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];
     const int B = P.B, M = P.M, D = P.D, Dv = P.Dv;
     const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
-    const int ldd = ld_of(D16), ldv = ld_of(V16), ldb = ld_of(B16);
+    const RLayout L = r_layout<TQ>(B, D, Dv, with_v != 0, TJ);
+    const int ldd = L.ldd, ldv = L.ldv, lga = L.lga, lgy = L.lgy, ldb = L.ldb;
     int w = blockIdx.x;
     const int k = w % M; w /= M;
     const int h = w % P.H, e = w / P.H;
@@ -320,35 +397,35 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
     const TQ* aR = reinterpret_cast<const TQ*>(P.aR) + (eh * M + k) * B * D;
     const float* cR = P.cR + (eh * M + k) * B;
     const float sm = P.sm_scale;
-    float* Kt = lds;
-    float* Vt = Kt + B16 * ldd;
-    float* kok = Vt + (with_v ? B16 * ldv : 0);
-    float* X = kok + B16;
-    float* Ga = X + TJ * ldd;
-    float* Gy = Ga + TJ * ldd;
-    float* c = Gy + (with_v ? TJ * ldv : 0);
-    float* gcl = c + TJ;
-    float* S = gcl + TJ;
-    float* R = S + TJ * ldb;
-    float* Gg = R + TJ * ldb;
+    TQ* Kt = reinterpret_cast<TQ*>(lds_raw + L.Kt);
+    TQ* Vt = reinterpret_cast<TQ*>(lds_raw + L.Vt);
+    float* kok = reinterpret_cast<float*>(lds_raw + L.kok);
+    TQ* X = reinterpret_cast<TQ*>(lds_raw + L.X);
+    float* Ga = reinterpret_cast<float*>(lds_raw + L.Ga);
+    float* Gy = reinterpret_cast<float*>(lds_raw + L.Gy);
+    float* c = reinterpret_cast<float*>(lds_raw + L.c);
+    float* gcl = reinterpret_cast<float*>(lds_raw + L.gcl);
+    float* S = reinterpret_cast<float*>(lds_raw + L.S);
+    float* R = reinterpret_cast<float*>(lds_raw + L.R);
+    float* Gg = reinterpret_cast<float*>(lds_raw + L.Gg);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-    stage_rows<NTH, TQ>(Kt, ldd, B16, D16, D, 1.f,
+    stage_rows<NTH, TQ, TQ>(Kt, ldd, B16, D16, D, 1.f,
                    [&](int i) { return i < B ? tok_row<TQ>(P.k, P.ks, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
     if (with_v)
-        stage_rows<NTH, TQ>(Vt, ldv, B16, V16, Dv, 1.f,
+        stage_rows<NTH, TQ, TQ>(Vt, ldv, B16, V16, Dv, 1.f,
                        [&](int i) { return i < B ? tok_row<TQ>(P.v, P.vs, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
     for (int i = threadIdx.x; i < B16; i += NTH) kok[i] = (i < B && token_ok(P, e, k * B + i - P.pad_off)) ? 1.f : 0.f;
 
     for (int j0 = 0; j0 < B; j0 += TJ) {
-        stage_rows<NTH, TQ>(X, ldd, TJ, D16, D, 1.f, [&](int jj) -> const TQ* {
+        stage_rows<NTH, TQ, TQ>(X, ldd, TJ, D16, D, 1.f, [&](int jj) -> const TQ* {
             if (j0 + jj >= B) return nullptr;
             return first ? tok_row<TQ>(P.q, P.qs, e, h, k * B + j0 + jj - P.pad_off, P.N) : aR + (j0 + jj) * D;
         });
-        stage_rows<NTH, float>(Ga, ldd, TJ, D16, D, sm,
+        stage_rows<NTH, float, float>(Ga, lga, TJ, D16, D, sm,
                           [&](int jj) { return j0 + jj < B ? G.gaL + ((eh * B + j0 + jj) * M + k) * D : nullptr; });
         if (with_v)
-            stage_rows<NTH, float>(Gy, ldv, TJ, V16, Dv, 1.f, [&](int jj) {
+            stage_rows<NTH, float, float>(Gy, lgy, TJ, V16, Dv, 1.f, [&](int jj) {
                 return j0 + jj < B ? G.gY + ((eh * B + j0 + jj) * M + k) * static_cast<long long>(Dv) : nullptr;
             });
         for (int jj = threadIdx.x; jj < TJ; jj += NTH) {
@@ -389,8 +466,8 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
         for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma(acc, nt, Ga + r0 * ldd, ldd, 1, Kt + c0 * ldd, 1, ldd, D16);
-            if (with_v) strip_mma(acc, nt, Gy + r0 * ldv, ldv, 1, Vt + c0 * ldv, 1, ldv, V16);
+            strip_mma(acc, nt, Ga + r0 * lga, lga, 1, Kt + c0 * ldd, 1, ldd, D16);
+            if (with_v) strip_mma(acc, nt, Gy + r0 * lgy, lgy, 1, Vt + c0 * ldv, 1, ldv, V16);
             strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) {
                 float* g = Gg + jj * ldb + i;
                 *g = *g != 0.f ? fmaf(gcl[jj], logf(R[jj * ldb + i]) + 1.0f, x) : 0.f;
@@ -427,7 +504,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
         for_strips<NTH>(B16, D16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma(acc, nt, R + r0, 1, ldb, Ga + c0, ldd, 1, TJ);
+            strip_mma(acc, nt, R + r0, 1, ldb, Ga + c0, lga, 1, TJ);
             strip_mma(acc, nt, Gg + r0, 1, ldb, X + c0, ldd, 1, TJ);
             strip_rmw(acc, nt, r0, c0, true,
                       [&](int i, int d) -> float* { return (i < B && d < D) ? G.dk + ((eh * M + k) * B + i) * D + d : nullptr; });
@@ -436,7 +513,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
-                strip_mma(acc, nt, R + r0, 1, ldb, Gy + c0, ldv, 1, TJ);
+                strip_mma(acc, nt, R + r0, 1, ldb, Gy + c0, lgy, 1, TJ);
                 strip_rmw(acc, nt, r0, c0, true, [&](int i, int d) -> float* {
                     return (i < B && d < Dv) ? G.dv + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d : nullptr;
                 });
@@ -445,17 +522,14 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
     }
 }
 
-size_t r_lds_floats(const Problem& P, bool with_v, int TJ) {
-    const int B16 = up(P.B, 16), D16 = up(P.D, 16), V16 = up(P.Dv, 16);
-    const size_t ldd = ld_of(D16), ldv = ld_of(V16), ldb = ld_of(B16);
-    return B16 * ldd + (with_v ? B16 * ldv : 0) + B16 + 2 * TJ * ldd + (with_v ? TJ * ldv : 0) + 2 * TJ + 3 * TJ * ldb;
-}
+template <class TQ>
+size_t r_lds_bytes(const Problem& P, bool with_v, int TJ) { return r_layout<TQ>(P.B, P.D, P.Dv, with_v, TJ).total; }
 
 // largest tile (multiple of 16, at most the padded extent) whose LDS fits; 0 if none
 template <class F>
-int pick_tile(int extent, F&& floats) {
+int pick_tile(int extent, F&& bytes) {
     for (int t = up(extent, 16); t >= 16; t -= 16)
-        if (floats(t) * sizeof(float) <= kLdsBudget) return t;
+        if (bytes(t) <= kLdsBudget) return t;
     return 0;
 }
 
@@ -475,12 +549,12 @@ int dispatch16(int dt, F&& f) {
 
 // Each returns MA_ERR_UNSUPPORTED when the problem does not fit; the caller then takes the FMA kernel.
 int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z, hipStream_t s) {
-    const int TL = pick_tile(P.M, [&](int t) { return lz_lds_floats(P, z, t); });
-    if (TL == 0) return MA_ERR_UNSUPPORTED;
-    const size_t lds = lz_lds_floats(P, z, TL) * sizeof(float);
-    const int nth = threads_for((TL / 16) * (up(P.M, 16) / 16));
     return dispatch16(dt_qk, [&](auto tq) {
         using TQ = decltype(tq);
+        const int TL = pick_tile(P.M, [&](int t) { return lz_lds_bytes<TQ>(P, z, t); });
+        if (TL == 0) return static_cast<int>(MA_ERR_UNSUPPORTED);
+        const size_t lds = lz_lds_bytes<TQ>(P, z, TL);
+        const int nth = threads_for((TL / 16) * (up(P.M, 16) / 16));
         auto launch = [&](auto kernel) {
             const int attr = mfma::set_lds_limit(kernel, kLdsBudget);
             if (attr) return attr;
@@ -494,12 +568,12 @@ int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z,
 }
 
 int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool first, bool with_v, hipStream_t s) {
-    const int TJ = pick_tile(P.B, [&](int t) { return r_lds_floats(P, with_v, t); });
-    if (TJ == 0) return MA_ERR_UNSUPPORTED;
-    const size_t lds = r_lds_floats(P, with_v, TJ) * sizeof(float);
-    const int nth = threads_for((TJ / 16) * (up(P.B, 16) / 16));
     return dispatch16(dt_qk, [&](auto tq) {
         using TQ = decltype(tq);
+        const int TJ = pick_tile(P.B, [&](int t) { return r_lds_bytes<TQ>(P, with_v, t); });
+        if (TJ == 0) return static_cast<int>(MA_ERR_UNSUPPORTED);
+        const size_t lds = r_lds_bytes<TQ>(P, with_v, TJ);
+        const int nth = threads_for((TJ / 16) * (up(P.B, 16) / 16));
         auto launch = [&](auto kernel) {
             const int attr = mfma::set_lds_limit(kernel, kLdsBudget);
             if (attr) return attr;

@@ -276,6 +276,7 @@ class _MonarchAttentionHip(torch.autograd.Function):
         return _forward(q, k, v, attn_mask, T, B, pre_pad, variant)
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, dout):
         q, k, v, attn_mask = ctx.saved_tensors
         T, B, pre_pad, variant = ctx.args
