@@ -181,12 +181,13 @@ __device__ __forceinline__ void softmax_rows_lds(float* U, int ld, int rows, int
         mx = wmax(mx);
         float sum = 0.f;
         for (int k = lane; k < cols; k += 64) {
-            const float p = expf(Ul[k] - mx);
+            const float p = __expf(Ul[k] - mx);
             Ul[k] = p;
             sum += p;
         }
         sum = wsum(sum);
-        for (int k = lane; k < cols; k += 64) Ul[k] = Ul[k] / sum;
+        const float inv = 1.0f / sum;
+        for (int k = lane; k < cols; k += 64) Ul[k] = Ul[k] * inv;
     }
 }
 
@@ -430,18 +431,18 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             });
         for (int jj = threadIdx.x; jj < TJ; jj += NTH) {
             const bool in = j0 + jj < B;
-            c[jj] = ((first || !in) ? 1.0f : cR[j0 + jj]) + P.eps;
+            c[jj] = 1.0f / (((first || !in) ? 1.0f : cR[j0 + jj]) + P.eps);   // c holds 1 / (cR + eps)
             gcl[jj] = in ? G.gcL[(eh * B + j0 + jj) * M + k] : 0.f;
         }
         __syncthreads();
 
-        // S = sm round(X K^T) / c, -inf for masked / padded keys
+        // S = sm round(X K^T) / (cR + eps), -inf for masked / padded keys
         for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma(acc, nt, X + r0 * ldd, ldd, 1, Kt + c0 * ldd, 1, ldd, D16);
             strip_each(acc, nt, r0, c0,
-                       [&](int jj, int i, float x) { S[jj * ldb + i] = kok[i] != 0.f ? sm * round_to<TQ>(x) / c[jj] : -INFINITY; });
+                       [&](int jj, int i, float x) { S[jj * ldb + i] = kok[i] != 0.f ? sm * round_to<TQ>(x) * c[jj] : -INFINITY; });
         });
         __syncthreads();
         for (int jj = wave; jj < TJ; jj += NTH / 64) {   // probabilities (ma_torch.py:14-18); Gg <- 1 where the clamp did not act
@@ -450,13 +451,13 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             mx = fmaxf(wmax(mx), P.eps);
             float sum = 0.f;
             for (int i = lane; i < B16; i += 64) {
-                const float p = expf(S[jj * ldb + i] - mx);
+                const float p = __expf(S[jj * ldb + i] - mx);
                 R[jj * ldb + i] = p;
                 sum += p;
             }
-            sum = wsum(sum) + P.eps;
+            const float inv = 1.0f / (wsum(sum) + P.eps);
             for (int i = lane; i < B16; i += 64) {
-                const float r = R[jj * ldb + i] / sum;
+                const float r = R[jj * ldb + i] * inv;
                 Gg[jj * ldb + i] = (i < B && r >= kTiny) ? 1.f : 0.f;
                 R[jj * ldb + i] = i < B ? fmaxf(r, kTiny) : 0.f;
             }
@@ -470,11 +471,11 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             if (with_v) strip_mma(acc, nt, Gy + r0 * lgy, lgy, 1, Vt + c0 * ldv, 1, ldv, V16);
             strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) {
                 float* g = Gg + jj * ldb + i;
-                *g = *g != 0.f ? fmaf(gcl[jj], logf(R[jj * ldb + i]) + 1.0f, x) : 0.f;
+                *g = *g != 0.f ? fmaf(gcl[jj], __logf(R[jj * ldb + i]) + 1.0f, x) : 0.f;
             });
         });
         __syncthreads();
-        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // dS, gcR; Gg <- dDot = dS sm / c; R <- round(r)
+        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // dS, gcR; Gg <- dDot = dS sm / (cR + eps); R <- round(r)
             float dot = 0.f;
             for (int i = lane; i < B16; i += 64) dot = fmaf(Gg[jj * ldb + i], R[jj * ldb + i], dot);
             dot = wsum(dot);
@@ -482,8 +483,8 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             for (int i = lane; i < B16; i += 64) {
                 const float s = S[jj * ldb + i], r = R[jj * ldb + i];
                 const float ds = s == -INFINITY ? 0.f : r * (Gg[jj * ldb + i] - dot);
-                if (s != -INFINITY) gc = fmaf(-ds, s / c[jj], gc);
-                Gg[jj * ldb + i] = ds * sm / c[jj];
+                if (s != -INFINITY) gc = fmaf(-ds, s * c[jj], gc);
+                Gg[jj * ldb + i] = ds * sm * c[jj];
                 R[jj * ldb + i] = round_to<TQ>(r);
             }
             gc = wsum(gc);
