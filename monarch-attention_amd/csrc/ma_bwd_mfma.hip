@@ -123,16 +123,15 @@ __device__ __forceinline__ void zero_acc(f32x4 (&acc)[4]) {
     for (int t = 0; t < 4; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
-// rows x width elements of TD (row stride ld) <- rows of a (.., rows, W) tensor of dtype T; TD is T
-// itself (copied as is) or float (converted, times scale); rows for which row_ptr(i) is null and
-// columns >= W are zero.  Sixteen lanes take a row, four elements each (one 8- or 16-byte load where
+// rows x width elements of TD (row stride ld) <- rows of a (.., rows, W) tensor of dtype T, converted
+// and multiplied by scale; rows for which row_ptr(i) is null and columns >= W are zero.  Sixteen lanes take a row, four elements each (one 8- or 16-byte load where
 // the row allows it), so a wave loads four rows per instruction; two such groups are in flight
 // together.
 template <int NTH, class T, class TD, class RowPtr>
 __device__ __forceinline__ void stage_rows(TD* dst, int ld, int rows, int width, int W, float scale, RowPtr&& row_ptr) {
     constexpr int NW = NTH / 64;
     struct alignas(4 * sizeof(T)) Quad { T v[4]; };
-    struct alignas(2 * sizeof(T)) Pair { T a, b; };
+    struct alignas(2 * sizeof(TD)) Pair { TD a, b; };
     const int lane = threadIdx.x & 63, sub = lane >> 4, c0 = lane & 15;
     for (int i0 = 4 * (threadIdx.x >> 6) + sub; i0 < rows; i0 += 8 * NW) {
         const T* p[2];
@@ -162,8 +161,10 @@ __device__ __forceinline__ void stage_rows(TD* dst, int ld, int rows, int width,
                     *reinterpret_cast<f32x4*>(dst + i * ld + 4 * c) = f32x4{scale * to_f(x[u].v[0]), scale * to_f(x[u].v[1]),
                                                                            scale * to_f(x[u].v[2]), scale * to_f(x[u].v[3])};
                 } else {   // 16-bit rows start on 4-byte boundaries only
-                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c) = Pair{x[u].v[0], x[u].v[1]};
-                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c + 2) = Pair{x[u].v[2], x[u].v[3]};
+                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c) =
+                        Pair{from_f<TD>(scale * to_f(x[u].v[0])), from_f<TD>(scale * to_f(x[u].v[1]))};
+                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c + 2) =
+                        Pair{from_f<TD>(scale * to_f(x[u].v[2])), from_f<TD>(scale * to_f(x[u].v[3]))};
                 }
             }
         }
@@ -346,9 +347,6 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
     }
 }
 
-template <class TQ>
-size_t lz_lds_bytes(const Problem& P, bool z, int TL) { return lz_layout<TQ>(P.M, P.D, z ? P.Dv : P.D, z, TL).total; }
-
 // ---------------------------------------------------------------- R stage
 // LDS of the R stage for tiles of TJ query rows: byte offsets and row strides (elements).
 //   Kt[B16][ldd] TQ, Vt[B16][ldv] TQ, kok[B16], X[TJ][ldd] TQ, Ga[TJ][lga] (sm * gaL), Gy[TJ][lgy],
@@ -523,15 +521,409 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
     }
 }
 
-template <class TQ>
-size_t r_lds_bytes(const Problem& P, bool with_v, int TJ) { return r_layout<TQ>(P.B, P.D, P.Dv, with_v, TJ).total; }
-
 // largest tile (multiple of 16, at most the padded extent) whose LDS fits; 0 if none
 template <class F>
 int pick_tile(int extent, F&& bytes) {
     for (int t = up(extent, 16); t >= 16; t -= 16)
         if (bytes(t) <= kLdsBudget) return t;
     return 0;
+}
+
+// ================================================================ fp16 / bf16 operands
+// The same stages with every GEMM operand as a 16-bit LDS matrix (row pitch n + 8 elements) and
+// v_mfma_f32_16x16x16_{f16,bf16}: a lane's four k-values are one 8-byte LDS read - a plain one
+// where k runs along the row, ds_read_b64_tr_b16 where it runs down the column (lane 4e+c of a
+// 16-lane group addresses row e, columns 4c..4c+3 of a 4 x 16 block and receives column lane%16).
+// Probabilities and their gradients are kept in fp32 for the softmax arithmetic and rounded to the
+// operand dtype for the products, which is where autograd through the reference rounds them too.
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+__host__ __device__ constexpr int ld16(int n) { return n + 8; }
+
+template <class T>
+struct Mma16;
+template <>
+struct Mma16<f16> {
+    static __device__ __forceinline__ f32x4 mma(i16x4 a, i16x4 b, f32x4 c) {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a), __builtin_bit_cast(h4, b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mma16<bf16> {
+    static __device__ __forceinline__ f32x4 mma(i16x4 a, i16x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+    }
+};
+
+template <bool TR, class T>
+__device__ __forceinline__ i16x4 lds_k4(const T* p) {
+    if constexpr (TR) {
+        typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
+        return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+    } else {
+        return *reinterpret_cast<const i16x4*>(p);
+    }
+}
+
+// acc[t] += sum_k A(r,k) B(k, 16 t + c) for one 16-row strip of NT 16-column tiles, K a multiple of 16.
+// TA = false: A is stored [row][k] (pitch lda) and points at the strip's first row; TA = true: A is
+// stored [k][row] and points at the strip's first column.  TB = false: B is stored [column][k] and
+// points at the first column's row; TB = true: B is stored [k][column] and points at the first column.
+template <int NT, bool TA, bool TB, class T>
+__device__ __forceinline__ void strip_mma16_n(f32x4 (&acc)[4], const T* A, int lda, const T* B, int ldb, int K) {
+    const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4, e = r >> 2, c = r & 3;
+    const T* a = TA ? A + (4 * q + e) * lda + 4 * c : A + r * lda + 4 * q;
+    const T* b = TB ? B + (4 * q + e) * ldb + 4 * c : B + r * ldb + 4 * q;
+    const int astep = TA ? 16 * lda : 16, bstep = TB ? 16 * ldb : 16, btile = TB ? 16 : 16 * ldb;
+#pragma unroll 2
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        const i16x4 av = lds_k4<TA>(a);
+        i16x4 bv[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) bv[t] = lds_k4<TB>(b + t * btile);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = Mma16<T>::mma(av, bv[t], acc[t]);
+        a += astep;
+        b += bstep;
+    }
+}
+template <bool TA, bool TB, class T>
+__device__ __forceinline__ void strip_mma16(f32x4 (&acc)[4], int nt, const T* A, int lda, const T* B, int ldb, int K) {
+    switch (nt) {   // nt is the same for every lane of the wave
+        case 1: return strip_mma16_n<1, TA, TB>(acc, A, lda, B, ldb, K);
+        case 2: return strip_mma16_n<2, TA, TB>(acc, A, lda, B, ldb, K);
+        case 3: return strip_mma16_n<3, TA, TB>(acc, A, lda, B, ldb, K);
+        default: return strip_mma16_n<4, TA, TB>(acc, A, lda, B, ldb, K);
+    }
+}
+
+// LDS of the 16-bit Z / L stage: aL[M16][ldd], W[M16][ldw] (Z: Y_j; L: gaR_j rounded), cl[M16],
+// cw[M16], Qt[TL][ldd], dO[TL][ldw] (Z), qok[TL], U[TL][ldm] f32, Gg[TL][ldm] f32, U16[TL][ldp],
+// G16[TL][ldp]
+struct LzLayout16 {
+    int ldd, ldw, ldm, ldp;
+    unsigned aLt, Wt, cl, cw, Qt, dO, qok, U, Gg, U16, G16, total;
+};
+__host__ __device__ inline LzLayout16 lz_layout16(int M, int D, int W, bool z, int TL) {
+    const int M16 = up(M, 16), D16 = up(D, 16), W16 = up(W, 16);
+    LzLayout16 L;
+    L.ldd = ld16(D16);
+    L.ldw = ld16(W16);
+    L.ldm = ld_of(M16);
+    L.ldp = ld16(M16);
+    unsigned off = 0;
+    auto take = [&](size_t bytes) { const unsigned at = off; off += static_cast<unsigned>((bytes + 15) / 16 * 16); return at; };
+    L.aLt = take(2 * M16 * L.ldd);
+    L.Wt = take(2 * M16 * L.ldw);
+    L.cl = take(4 * M16);
+    L.cw = take(4 * M16);
+    L.Qt = take(2 * TL * L.ldd);
+    L.dO = take(z ? 2 * TL * L.ldw : 0);
+    L.qok = take(4 * TL);
+    L.U = take(4 * TL * L.ldm);
+    L.Gg = take(4 * TL * L.ldm);
+    L.U16 = take(2 * TL * L.ldp);
+    L.G16 = take(2 * TL * L.ldp);
+    L.total = off;
+    return L;
+}
+
+template <class TQ, bool kZ, int NTH>
+__global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, int TL) {
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+    const int M = P.M, D = P.D, B = P.B, W = kZ ? P.Dv : P.D;
+    const int M16 = up(M, 16), D16 = up(D, 16), W16 = up(W, 16);
+    const LzLayout16 L = lz_layout16(M, D, W, kZ, TL);
+    const int ldd = L.ldd, ldw = L.ldw, ldm = L.ldm, ldp = L.ldp;
+    int w = blockIdx.x;
+    const int j = w % B; w /= B;
+    const int h = w % P.H, e = w / P.H;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const long long jm = (eh * B + j) * M;
+    TQ* aLt = reinterpret_cast<TQ*>(lds_raw + L.aLt);
+    TQ* Wt = reinterpret_cast<TQ*>(lds_raw + L.Wt);
+    float* cl = reinterpret_cast<float*>(lds_raw + L.cl);
+    float* cw = reinterpret_cast<float*>(lds_raw + L.cw);
+    TQ* Qt = reinterpret_cast<TQ*>(lds_raw + L.Qt);
+    TQ* dO = reinterpret_cast<TQ*>(lds_raw + L.dO);
+    float* qok = reinterpret_cast<float*>(lds_raw + L.qok);
+    float* U = reinterpret_cast<float*>(lds_raw + L.U);
+    float* Gg = reinterpret_cast<float*>(lds_raw + L.Gg);
+    TQ* U16 = reinterpret_cast<TQ*>(lds_raw + L.U16);
+    TQ* G16 = reinterpret_cast<TQ*>(lds_raw + L.G16);
+
+    const TQ* aL = reinterpret_cast<const TQ*>(P.aL) + jm * D;
+    stage_rows<NTH, TQ, TQ>(aLt, ldd, M16, D16, D, 1.f, [&](int k) { return k < M ? aL + k * D : nullptr; });
+    if (kZ) {
+        const TQ* Y = reinterpret_cast<const TQ*>(P.Y) + jm * W;
+        stage_rows<NTH, TQ, TQ>(Wt, ldw, M16, W16, W, 1.f, [&](int k) { return k < M ? Y + k * static_cast<long long>(W) : nullptr; });
+    } else {
+        stage_rows<NTH, float, TQ>(Wt, ldw, M16, W16, W, 1.f,
+                                   [&](int k) { return k < M ? G.gaR + ((eh * M + k) * B + j) * D : nullptr; });
+    }
+    for (int k = threadIdx.x; k < M16; k += NTH) {
+        cl[k] = k < M ? P.cL[jm + k] : 0.f;
+        cw[k] = (!kZ && k < M) ? G.gcR[(eh * M + k) * B + j] : 0.f;
+    }
+
+    for (int l0 = 0; l0 < M; l0 += TL) {
+        stage_rows<NTH, TQ, TQ>(Qt, ldd, TL, D16, D, 1.f, [&](int ll) {
+            return l0 + ll < M ? tok_row<TQ>(P.q, P.qs, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
+        });
+        if (kZ)
+            stage_rows<NTH, TQ, TQ>(dO, ldw, TL, W16, W, 1.f, [&](int ll) {
+                return l0 + ll < M ? tok_row<TQ>(G.dout, G.dos, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
+            });
+        for (int ll = threadIdx.x; ll < TL; ll += NTH)
+            qok[ll] = (l0 + ll < M && token_ok(P, e, (l0 + ll) * B + j - P.pad_off)) ? 1.f : 0.f;
+        __syncthreads();
+
+        // U = round(Qt aL^T) - cL, -inf in the columns beyond M
+        for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma16<false, false>(acc, nt, Qt + r0 * ldd, ldd, aLt + c0 * ldd, ldd, D16);
+            strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) { U[ll * ldm + k] = k < M ? round_to<TQ>(x) - cl[k] : -INFINITY; });
+        });
+        __syncthreads();
+        softmax_rows_lds<NTH>(U, ldm, TL, M16);
+        // Z: gLz = dO Y^T;  L: gLm = mask_q (Qt gaR^T + gcR)
+        for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            if (kZ) strip_mma16<false, false>(acc, nt, dO + r0 * ldw, ldw, Wt + c0 * ldw, ldw, W16);
+            else strip_mma16<false, false>(acc, nt, Qt + r0 * ldd, ldd, Wt + c0 * ldw, ldw, W16);
+            strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) {
+                if (!kZ) x = (k < M && qok[ll] != 0.f) ? x + cw[k] : 0.f;
+                Gg[ll * ldm + k] = x;
+            });
+        });
+        __syncthreads();
+        {   // dU = p (g - sum g p); U16 <- rounded (L: query-masked) probabilities, G16 <- rounded dU
+            const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+            for (int ll = wave; ll < TL; ll += NTH / 64) {
+                float dot = 0.f;
+                for (int k = lane; k < M16; k += 64) dot = fmaf(Gg[ll * ldm + k], U[ll * ldm + k], dot);
+                dot = wsum(dot);
+                const float keep = kZ ? 1.f : qok[ll];
+                for (int k = lane; k < M16; k += 64) {
+                    const float p = U[ll * ldm + k];
+                    const float du = p * (Gg[ll * ldm + k] - dot);
+                    Gg[ll * ldm + k] = du;
+                    G16[ll * ldp + k] = from_f<TQ>(du);
+                    U16[ll * ldp + k] = from_f<TQ>(keep * p);
+                }
+            }
+        }
+        __syncthreads();
+        if (kZ) {   // gY (+)= round(Lz)^T dO
+            for_strips<NTH>(M16, W16, [&](int r0, int c0, int nt) {
+                f32x4 acc[4];
+                zero_acc(acc);
+                strip_mma16<true, true>(acc, nt, U16 + r0, ldp, dO + c0, ldw, TL);
+                strip_rmw(acc, nt, r0, c0, l0 != 0,
+                          [&](int k, int d) -> float* { return (k < M && d < W) ? G.gY + (jm + k) * W + d : nullptr; });
+            });
+        }
+        // gaL (+)= dU^T Qt
+        for_strips<NTH>(M16, D16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma16<true, true>(acc, nt, G16 + r0, ldp, Qt + c0, ldd, TL);
+            strip_rmw(acc, nt, r0, c0, l0 != 0,
+                      [&](int k, int d) -> float* { return (k < M && d < D) ? G.gaL + (jm + k) * D + d : nullptr; });
+        });
+        for (int k = threadIdx.x; k < M; k += NTH) {   // gcL (+)= -sum_l dU
+            float acc = l0 ? G.gcL[jm + k] : 0.f;
+#pragma unroll 8
+            for (int ll = 0; ll < TL; ++ll) acc -= Gg[ll * ldm + k];
+            G.gcL[jm + k] = acc;
+        }
+        // dq rows (l, j) += dU aL  (L: + round(Lm) gaR)
+        for_strips<NTH>(TL, D16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma16<false, true>(acc, nt, G16 + r0 * ldp, ldp, aLt + c0, ldd, M16);
+            if (!kZ) strip_mma16<false, true>(acc, nt, U16 + r0 * ldp, ldp, Wt + c0, ldw, M16);
+            strip_rmw(acc, nt, r0, c0, true, [&](int ll, int d) -> float* {
+                return (l0 + ll < M && d < D) ? G.dq + (eh * M * B + (l0 + ll) * B + j) * D + d : nullptr;
+            });
+        });
+        __syncthreads();
+    }
+}
+
+// LDS of the 16-bit R stage: Kt[B16][ldd], Vt[B16][ldv], kok[B16], X[TJ][ldd], Ga[TJ][ldd]
+// (sm * gaL, rounded), Gy[TJ][ldv], c[TJ], gcl[TJ], S, R, Gg [TJ][ldb] f32, R16, D16 [TJ][ldp]
+struct RLayout16 {
+    int ldd, ldv, ldb, ldp;
+    unsigned Kt, Vt, kok, X, Ga, Gy, c, gcl, S, R, Gg, R16, D16, total;
+};
+__host__ __device__ inline RLayout16 r_layout16(int B, int D, int Dv, bool with_v, int TJ) {
+    const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
+    RLayout16 L;
+    L.ldd = ld16(D16);
+    L.ldv = ld16(V16);
+    L.ldb = ld_of(B16);
+    L.ldp = ld16(B16);
+    unsigned off = 0;
+    auto take = [&](size_t bytes) { const unsigned at = off; off += static_cast<unsigned>((bytes + 15) / 16 * 16); return at; };
+    L.Kt = take(2 * B16 * L.ldd);
+    L.Vt = take(with_v ? 2 * B16 * L.ldv : 0);
+    L.kok = take(4 * B16);
+    L.X = take(2 * TJ * L.ldd);
+    L.Ga = take(2 * TJ * L.ldd);
+    L.Gy = take(with_v ? 2 * TJ * L.ldv : 0);
+    L.c = take(4 * TJ);
+    L.gcl = take(4 * TJ);
+    L.S = take(4 * TJ * L.ldb);
+    L.R = take(4 * TJ * L.ldb);
+    L.Gg = take(4 * TJ * L.ldb);
+    L.R16 = take(2 * TJ * L.ldp);
+    L.D16 = take(2 * TJ * L.ldp);
+    L.total = off;
+    return L;
+}
+
+template <class TQ, int NTH>
+__global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int TJ, int first, int with_v) {
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+    const int B = P.B, M = P.M, D = P.D, Dv = P.Dv;
+    const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
+    const RLayout16 L = r_layout16(B, D, Dv, with_v != 0, TJ);
+    const int ldd = L.ldd, ldv = L.ldv, ldb = L.ldb, ldp = L.ldp;
+    int w = blockIdx.x;
+    const int k = w % M; w /= M;
+    const int h = w % P.H, e = w / P.H;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const TQ* aR = reinterpret_cast<const TQ*>(P.aR) + (eh * M + k) * B * D;
+    const float* cR = P.cR + (eh * M + k) * B;
+    const float sm = P.sm_scale;
+    TQ* Kt = reinterpret_cast<TQ*>(lds_raw + L.Kt);
+    TQ* Vt = reinterpret_cast<TQ*>(lds_raw + L.Vt);
+    float* kok = reinterpret_cast<float*>(lds_raw + L.kok);
+    TQ* X = reinterpret_cast<TQ*>(lds_raw + L.X);
+    TQ* Ga = reinterpret_cast<TQ*>(lds_raw + L.Ga);
+    TQ* Gy = reinterpret_cast<TQ*>(lds_raw + L.Gy);
+    float* c = reinterpret_cast<float*>(lds_raw + L.c);
+    float* gcl = reinterpret_cast<float*>(lds_raw + L.gcl);
+    float* S = reinterpret_cast<float*>(lds_raw + L.S);
+    float* R = reinterpret_cast<float*>(lds_raw + L.R);
+    float* Gg = reinterpret_cast<float*>(lds_raw + L.Gg);
+    TQ* R16 = reinterpret_cast<TQ*>(lds_raw + L.R16);
+    TQ* Dd = reinterpret_cast<TQ*>(lds_raw + L.D16);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    stage_rows<NTH, TQ, TQ>(Kt, ldd, B16, D16, D, 1.f,
+                            [&](int i) { return i < B ? tok_row<TQ>(P.k, P.ks, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
+    if (with_v)
+        stage_rows<NTH, TQ, TQ>(Vt, ldv, B16, V16, Dv, 1.f,
+                                [&](int i) { return i < B ? tok_row<TQ>(P.v, P.vs, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
+    for (int i = threadIdx.x; i < B16; i += NTH) kok[i] = (i < B && token_ok(P, e, k * B + i - P.pad_off)) ? 1.f : 0.f;
+
+    for (int j0 = 0; j0 < B; j0 += TJ) {
+        stage_rows<NTH, TQ, TQ>(X, ldd, TJ, D16, D, 1.f, [&](int jj) -> const TQ* {
+            if (j0 + jj >= B) return nullptr;
+            return first ? tok_row<TQ>(P.q, P.qs, e, h, k * B + j0 + jj - P.pad_off, P.N) : aR + (j0 + jj) * D;
+        });
+        stage_rows<NTH, float, TQ>(Ga, ldd, TJ, D16, D, sm,
+                                   [&](int jj) { return j0 + jj < B ? G.gaL + ((eh * B + j0 + jj) * M + k) * D : nullptr; });
+        if (with_v)
+            stage_rows<NTH, float, TQ>(Gy, ldv, TJ, V16, Dv, 1.f, [&](int jj) {
+                return j0 + jj < B ? G.gY + ((eh * B + j0 + jj) * M + k) * static_cast<long long>(Dv) : nullptr;
+            });
+        for (int jj = threadIdx.x; jj < TJ; jj += NTH) {
+            const bool in = j0 + jj < B;
+            c[jj] = 1.0f / (((first || !in) ? 1.0f : cR[j0 + jj]) + P.eps);   // c holds 1 / (cR + eps)
+            gcl[jj] = in ? G.gcL[(eh * B + j0 + jj) * M + k] : 0.f;
+        }
+        __syncthreads();
+
+        // S = sm round(X K^T) / (cR + eps), -inf for masked / padded keys
+        for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma16<false, false>(acc, nt, X + r0 * ldd, ldd, Kt + c0 * ldd, ldd, D16);
+            strip_each(acc, nt, r0, c0,
+                       [&](int jj, int i, float x) { S[jj * ldb + i] = kok[i] != 0.f ? sm * round_to<TQ>(x) * c[jj] : -INFINITY; });
+        });
+        __syncthreads();
+        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // probabilities (ma_torch.py:14-18); Gg <- 1 where the clamp did not act
+            float mx = -INFINITY;
+            for (int i = lane; i < B16; i += 64) mx = fmaxf(mx, S[jj * ldb + i]);
+            mx = fmaxf(wmax(mx), P.eps);
+            float sum = 0.f;
+            for (int i = lane; i < B16; i += 64) {
+                const float p = __expf(S[jj * ldb + i] - mx);
+                R[jj * ldb + i] = p;
+                sum += p;
+            }
+            const float inv = 1.0f / (wsum(sum) + P.eps);
+            for (int i = lane; i < B16; i += 64) {
+                const float r = R[jj * ldb + i] * inv;
+                Gg[jj * ldb + i] = (i < B && r >= kTiny) ? 1.f : 0.f;
+                R[jj * ldb + i] = i < B ? fmaxf(r, kTiny) : 0.f;
+            }
+        }
+        __syncthreads();
+        // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act
+        for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma16<false, false>(acc, nt, Ga + r0 * ldd, ldd, Kt + c0 * ldd, ldd, D16);
+            if (with_v) strip_mma16<false, false>(acc, nt, Gy + r0 * ldv, ldv, Vt + c0 * ldv, ldv, V16);
+            strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) {
+                float* g = Gg + jj * ldb + i;
+                *g = *g != 0.f ? fmaf(gcl[jj], __logf(R[jj * ldb + i]) + 1.0f, x) : 0.f;
+            });
+        });
+        __syncthreads();
+        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // dS, gcR; D16 <- dDot = dS sm / (cR + eps); R16 <- round(r)
+            float dot = 0.f;
+            for (int i = lane; i < B16; i += 64) dot = fmaf(Gg[jj * ldb + i], R[jj * ldb + i], dot);
+            dot = wsum(dot);
+            float gc = 0.f;
+            for (int i = lane; i < B16; i += 64) {
+                const float s = S[jj * ldb + i], r = R[jj * ldb + i];
+                const float ds = s == -INFINITY ? 0.f : r * (Gg[jj * ldb + i] - dot);
+                if (s != -INFINITY) gc = fmaf(-ds, s * c[jj], gc);
+                Dd[jj * ldp + i] = from_f<TQ>(ds * sm * c[jj]);
+                R16[jj * ldp + i] = from_f<TQ>(r);
+            }
+            gc = wsum(gc);
+            if (!first && lane == 0 && j0 + jj < B) G.gcR[(eh * M + k) * B + j0 + jj] = gc;
+        }
+        __syncthreads();
+        // gaR = dDot K (first step: aR is q, the rows of block k of dq)
+        for_strips<NTH>(TJ, D16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma16<false, true>(acc, nt, Dd + r0 * ldp, ldp, Kt + c0, ldd, B16);
+            strip_rmw(acc, nt, r0, c0, first != 0, [&](int jj, int d) -> float* {
+                if (j0 + jj >= B || d >= D) return nullptr;
+                return (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0 + jj) * D + d;
+            });
+        });
+        // dK += round(r)^T (sm gaL) + dDot^T X
+        for_strips<NTH>(B16, D16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma16<true, true>(acc, nt, R16 + r0, ldp, Ga + c0, ldd, TJ);
+            strip_mma16<true, true>(acc, nt, Dd + r0, ldp, X + c0, ldd, TJ);
+            strip_rmw(acc, nt, r0, c0, true,
+                      [&](int i, int d) -> float* { return (i < B && d < D) ? G.dk + ((eh * M + k) * B + i) * D + d : nullptr; });
+        });
+        if (with_v)   // dV += round(r)^T gY
+            for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
+                f32x4 acc[4];
+                zero_acc(acc);
+                strip_mma16<true, true>(acc, nt, R16 + r0, ldp, Gy + c0, ldv, TJ);
+                strip_rmw(acc, nt, r0, c0, true, [&](int i, int d) -> float* {
+                    return (i < B && d < Dv) ? G.dv + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d : nullptr;
+                });
+            });
+        __syncthreads();
+    }
 }
 
 // threads per workgroup for a stage whose probability matrix has `tiles` 16 x 16 tiles
@@ -552,9 +944,14 @@ int dispatch16(int dt, F&& f) {
 int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z, hipStream_t s) {
     return dispatch16(dt_qk, [&](auto tq) {
         using TQ = decltype(tq);
-        const int TL = pick_tile(P.M, [&](int t) { return lz_lds_bytes<TQ>(P, z, t); });
+        constexpr bool k32 = sizeof(TQ) == 4;
+        const int W = z ? P.Dv : P.D;
+        auto bytes = [&](int t) -> size_t {
+            return k32 ? lz_layout<TQ>(P.M, P.D, W, z, t).total : lz_layout16(P.M, P.D, W, z, t).total;
+        };
+        const int TL = pick_tile(P.M, bytes);
         if (TL == 0) return static_cast<int>(MA_ERR_UNSUPPORTED);
-        const size_t lds = lz_lds_bytes<TQ>(P, z, TL);
+        const size_t lds = bytes(TL);
         const int nth = threads_for((TL / 16) * (up(P.M, 16) / 16));
         auto launch = [&](auto kernel) {
             const int attr = mfma::set_lds_limit(kernel, kLdsBudget);
@@ -562,18 +959,28 @@ int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z,
             hipLaunchKernelGGL(kernel, dim3(P.E * P.H * P.B), dim3(nth), lds, s, P, G, TL);
             return static_cast<int>(hipGetLastError());
         };
-        if (nth == 64) return z ? launch(lz_bwd_mfma<TQ, true, 64>) : launch(lz_bwd_mfma<TQ, false, 64>);
-        if (nth == 256) return z ? launch(lz_bwd_mfma<TQ, true, 256>) : launch(lz_bwd_mfma<TQ, false, 256>);
-        return z ? launch(lz_bwd_mfma<TQ, true, 1024>) : launch(lz_bwd_mfma<TQ, false, 1024>);
+        if constexpr (k32) {
+            if (nth == 64) return z ? launch(lz_bwd_mfma<TQ, true, 64>) : launch(lz_bwd_mfma<TQ, false, 64>);
+            if (nth == 256) return z ? launch(lz_bwd_mfma<TQ, true, 256>) : launch(lz_bwd_mfma<TQ, false, 256>);
+            return z ? launch(lz_bwd_mfma<TQ, true, 1024>) : launch(lz_bwd_mfma<TQ, false, 1024>);
+        } else {
+            if (nth == 64) return z ? launch(lz_bwd_mfma16<TQ, true, 64>) : launch(lz_bwd_mfma16<TQ, false, 64>);
+            if (nth == 256) return z ? launch(lz_bwd_mfma16<TQ, true, 256>) : launch(lz_bwd_mfma16<TQ, false, 256>);
+            return z ? launch(lz_bwd_mfma16<TQ, true, 1024>) : launch(lz_bwd_mfma16<TQ, false, 1024>);
+        }
     });
 }
 
 int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool first, bool with_v, hipStream_t s) {
     return dispatch16(dt_qk, [&](auto tq) {
         using TQ = decltype(tq);
-        const int TJ = pick_tile(P.B, [&](int t) { return r_lds_bytes<TQ>(P, with_v, t); });
+        constexpr bool k32 = sizeof(TQ) == 4;
+        auto bytes = [&](int t) -> size_t {
+            return k32 ? r_layout<TQ>(P.B, P.D, P.Dv, with_v, t).total : r_layout16(P.B, P.D, P.Dv, with_v, t).total;
+        };
+        const int TJ = pick_tile(P.B, bytes);
         if (TJ == 0) return static_cast<int>(MA_ERR_UNSUPPORTED);
-        const size_t lds = r_lds_bytes<TQ>(P, with_v, TJ);
+        const size_t lds = bytes(TJ);
         const int nth = threads_for((TJ / 16) * (up(P.B, 16) / 16));
         auto launch = [&](auto kernel) {
             const int attr = mfma::set_lds_limit(kernel, kLdsBudget);
@@ -581,9 +988,15 @@ int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool fir
             hipLaunchKernelGGL(kernel, dim3(P.E * P.H * P.M), dim3(nth), lds, s, P, G, TJ, first ? 1 : 0, with_v ? 1 : 0);
             return static_cast<int>(hipGetLastError());
         };
-        if (nth == 64) return launch(r_bwd_mfma<TQ, 64>);
-        if (nth == 256) return launch(r_bwd_mfma<TQ, 256>);
-        return launch(r_bwd_mfma<TQ, 1024>);
+        if constexpr (k32) {
+            if (nth == 64) return launch(r_bwd_mfma<TQ, 64>);
+            if (nth == 256) return launch(r_bwd_mfma<TQ, 256>);
+            return launch(r_bwd_mfma<TQ, 1024>);
+        } else {
+            if (nth == 64) return launch(r_bwd_mfma16<TQ, 64>);
+            if (nth == 256) return launch(r_bwd_mfma16<TQ, 256>);
+            return launch(r_bwd_mfma16<TQ, 1024>);
+        }
     });
 }
 
