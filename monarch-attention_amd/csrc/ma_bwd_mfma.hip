@@ -598,11 +598,11 @@ __device__ __forceinline__ void strip_mma16(f32x4 (&acc)[4], int nt, const T* A,
 }
 
 // LDS of the 16-bit Z / L stage: aL[M16][ldd], W[M16][ldw] (Z: Y_j; L: gaR_j rounded), cl[M16],
-// cw[M16], Qt[TL][ldd], dO[TL][ldw] (Z), qok[TL], U[TL][ldm] f32, Gg[TL][ldm] f32, U16[TL][ldp],
-// G16[TL][ldp]
+// cw[M16], Qt[TL][ldd], dO[TL][ldw] (Z), qok[TL], U[TL][ldm] f32, Gg[TL][ldm] f32, G16[TL][ldp].
+// The rounded probabilities U16 are written over U row by row (row pitch 2 ldm elements).
 struct LzLayout16 {
     int ldd, ldw, ldm, ldp;
-    unsigned aLt, Wt, cl, cw, Qt, dO, qok, U, Gg, U16, G16, total;
+    unsigned aLt, Wt, cl, cw, Qt, dO, qok, U, Gg, G16, total;
 };
 __host__ __device__ inline LzLayout16 lz_layout16(int M, int D, int W, bool z, int TL) {
     const int M16 = up(M, 16), D16 = up(D, 16), W16 = up(W, 16);
@@ -622,7 +622,6 @@ __host__ __device__ inline LzLayout16 lz_layout16(int M, int D, int W, bool z, i
     L.qok = take(4 * TL);
     L.U = take(4 * TL * L.ldm);
     L.Gg = take(4 * TL * L.ldm);
-    L.U16 = take(2 * TL * L.ldp);
     L.G16 = take(2 * TL * L.ldp);
     L.total = off;
     return L;
@@ -649,7 +648,9 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
     float* qok = reinterpret_cast<float*>(lds_raw + L.qok);
     float* U = reinterpret_cast<float*>(lds_raw + L.U);
     float* Gg = reinterpret_cast<float*>(lds_raw + L.Gg);
-    TQ* U16 = reinterpret_cast<TQ*>(lds_raw + L.U16);
+    typedef TQ __attribute__((may_alias)) TQa;   // 16-bit values stored over fp32 ones that were just read
+    TQa* U16 = reinterpret_cast<TQa*>(lds_raw + L.U);
+    const int ldu = 2 * ldm;
     TQ* G16 = reinterpret_cast<TQ*>(lds_raw + L.G16);
 
     const TQ* aL = reinterpret_cast<const TQ*>(P.aL) + jm * D;
@@ -711,7 +712,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
                     const float du = p * (Gg[ll * ldm + k] - dot);
                     Gg[ll * ldm + k] = du;
                     G16[ll * ldp + k] = from_f<TQ>(du);
-                    U16[ll * ldp + k] = from_f<TQ>(keep * p);
+                    U16[ll * ldu + k] = from_f<TQ>(keep * p);   // lands on fp32 entries this wave has read already
                 }
             }
         }
@@ -720,7 +721,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             for_strips<NTH>(M16, W16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
-                strip_mma16<true, true>(acc, nt, U16 + r0, ldp, dO + c0, ldw, TL);
+                strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(U16) + r0, ldu, dO + c0, ldw, TL);
                 strip_rmw(acc, nt, r0, c0, l0 != 0,
                           [&](int k, int d) -> float* { return (k < M && d < W) ? G.gY + (jm + k) * W + d : nullptr; });
             });
@@ -744,7 +745,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma16<false, true>(acc, nt, G16 + r0 * ldp, ldp, aLt + c0, ldd, M16);
-            if (!kZ) strip_mma16<false, true>(acc, nt, U16 + r0 * ldp, ldp, Wt + c0, ldw, M16);
+            if (!kZ) strip_mma16<false, true>(acc, nt, reinterpret_cast<const TQ*>(U16) + r0 * ldu, ldu, Wt + c0, ldw, M16);
             strip_rmw(acc, nt, r0, c0, true, [&](int ll, int d) -> float* {
                 return (l0 + ll < M && d < D) ? G.dq + (eh * M * B + (l0 + ll) * B + j) * D + d : nullptr;
             });
@@ -754,10 +755,11 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
 }
 
 // LDS of the 16-bit R stage: Kt[B16][ldd], Vt[B16][ldv], kok[B16], X[TJ][ldd], Ga[TJ][ldd]
-// (sm * gaL, rounded), Gy[TJ][ldv], c[TJ], gcl[TJ], S, R, Gg [TJ][ldb] f32, R16, D16 [TJ][ldp]
+// (sm * gaL, rounded), Gy[TJ][ldv], c[TJ], gcl[TJ], S, R, Gg [TJ][ldb] f32.  The rounded
+// probabilities and the rounded dDot are written over R and Gg row by row (row pitch 2 ldb elements).
 struct RLayout16 {
-    int ldd, ldv, ldb, ldp;
-    unsigned Kt, Vt, kok, X, Ga, Gy, c, gcl, S, R, Gg, R16, D16, total;
+    int ldd, ldv, ldb;
+    unsigned Kt, Vt, kok, X, Ga, Gy, c, gcl, S, R, Gg, total;
 };
 __host__ __device__ inline RLayout16 r_layout16(int B, int D, int Dv, bool with_v, int TJ) {
     const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
@@ -765,7 +767,6 @@ __host__ __device__ inline RLayout16 r_layout16(int B, int D, int Dv, bool with_
     L.ldd = ld16(D16);
     L.ldv = ld16(V16);
     L.ldb = ld_of(B16);
-    L.ldp = ld16(B16);
     unsigned off = 0;
     auto take = [&](size_t bytes) { const unsigned at = off; off += static_cast<unsigned>((bytes + 15) / 16 * 16); return at; };
     L.Kt = take(2 * B16 * L.ldd);
@@ -779,8 +780,6 @@ __host__ __device__ inline RLayout16 r_layout16(int B, int D, int Dv, bool with_
     L.S = take(4 * TJ * L.ldb);
     L.R = take(4 * TJ * L.ldb);
     L.Gg = take(4 * TJ * L.ldb);
-    L.R16 = take(2 * TJ * L.ldp);
-    L.D16 = take(2 * TJ * L.ldp);
     L.total = off;
     return L;
 }
@@ -791,7 +790,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
     const int B = P.B, M = P.M, D = P.D, Dv = P.Dv;
     const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
     const RLayout16 L = r_layout16(B, D, Dv, with_v != 0, TJ);
-    const int ldd = L.ldd, ldv = L.ldv, ldb = L.ldb, ldp = L.ldp;
+    const int ldd = L.ldd, ldv = L.ldv, ldb = L.ldb, ldp = 2 * L.ldb;
     int w = blockIdx.x;
     const int k = w % M; w /= M;
     const int h = w % P.H, e = w / P.H;
@@ -810,8 +809,9 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
     float* S = reinterpret_cast<float*>(lds_raw + L.S);
     float* R = reinterpret_cast<float*>(lds_raw + L.R);
     float* Gg = reinterpret_cast<float*>(lds_raw + L.Gg);
-    TQ* R16 = reinterpret_cast<TQ*>(lds_raw + L.R16);
-    TQ* Dd = reinterpret_cast<TQ*>(lds_raw + L.D16);
+    typedef TQ __attribute__((may_alias)) TQa;   // 16-bit values stored over fp32 ones that were just read
+    TQa* R16 = reinterpret_cast<TQa*>(lds_raw + L.R);
+    TQa* Dd = reinterpret_cast<TQa*>(lds_raw + L.Gg);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
     stage_rows<NTH, TQ, TQ>(Kt, ldd, B16, D16, D, 1.f,
@@ -887,7 +887,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
                 const float s = S[jj * ldb + i], r = R[jj * ldb + i];
                 const float ds = s == -INFINITY ? 0.f : r * (Gg[jj * ldb + i] - dot);
                 if (s != -INFINITY) gc = fmaf(-ds, s * c[jj], gc);
-                Dd[jj * ldp + i] = from_f<TQ>(ds * sm * c[jj]);
+                Dd[jj * ldp + i] = from_f<TQ>(ds * sm * c[jj]);   // both land on fp32 entries this wave has read already
                 R16[jj * ldp + i] = from_f<TQ>(r);
             }
             gc = wsum(gc);
@@ -898,7 +898,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
         for_strips<NTH>(TJ, D16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma16<false, true>(acc, nt, Dd + r0 * ldp, ldp, Kt + c0, ldd, B16);
+            strip_mma16<false, true>(acc, nt, reinterpret_cast<const TQ*>(Dd) + r0 * ldp, ldp, Kt + c0, ldd, B16);
             strip_rmw(acc, nt, r0, c0, first != 0, [&](int jj, int d) -> float* {
                 if (j0 + jj >= B || d >= D) return nullptr;
                 return (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0 + jj) * D + d;
@@ -908,8 +908,8 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
         for_strips<NTH>(B16, D16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
             zero_acc(acc);
-            strip_mma16<true, true>(acc, nt, R16 + r0, ldp, Ga + c0, ldd, TJ);
-            strip_mma16<true, true>(acc, nt, Dd + r0, ldp, X + c0, ldd, TJ);
+            strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(R16) + r0, ldp, Ga + c0, ldd, TJ);
+            strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(Dd) + r0, ldp, X + c0, ldd, TJ);
             strip_rmw(acc, nt, r0, c0, true,
                       [&](int i, int d) -> float* { return (i < B && d < D) ? G.dk + ((eh * M + k) * B + i) * D + d : nullptr; });
         });
@@ -917,7 +917,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
-                strip_mma16<true, true>(acc, nt, R16 + r0, ldp, Gy + c0, ldv, TJ);
+                strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(R16) + r0, ldp, Gy + c0, ldv, TJ);
                 strip_rmw(acc, nt, r0, c0, true, [&](int i, int d) -> float* {
                     return (i < B && d < Dv) ? G.dv + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d : nullptr;
                 });
