@@ -314,20 +314,29 @@ __global__ void fill_zero_kernel(float* p, long long n) {
         p[i] = 0.f;
 }
 
-// real rows of a padded fp32 gradient (E,H,Np,W) -> the caller's tensor (dtype T, its strides)
-template <class T>
+// real rows of a padded fp32 gradient (E,H,Np,W) -> the caller's tensor (dtype T, its strides).
+// VEC = 4: four consecutive columns per thread (W % 4 == 0, rows of dst aligned to four elements).
+template <class T, int VEC>
 __global__ void grad_out_kernel(const float* src, char* dst, long long s0, long long s1, long long s2, int E, int H, int N, int Np,
                                 int W, int pad_off) {
-    const long long total = static_cast<long long>(E) * H * N * W;
+    const int WV = W / VEC;
+    const long long total = static_cast<long long>(E) * H * N * WV;
     for (long long i = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x; i < total;
          i += static_cast<long long>(gridDim.x) * blockDim.x) {
-        const int d = static_cast<int>(i % W);
-        long long w = i / W;
+        const int d = static_cast<int>(i % WV) * VEC;
+        long long w = i / WV;
         const int t = static_cast<int>(w % N); w /= N;
         const int h = static_cast<int>(w % H);
         const int e = static_cast<int>(w / H);
-        const float x = src[((static_cast<long long>(e) * H + h) * Np + (t + pad_off)) * W + d];
-        reinterpret_cast<T*>(dst)[e * s0 + h * s1 + t * s2 + d] = from_f<T>(x);
+        const float* x = src + ((static_cast<long long>(e) * H + h) * Np + (t + pad_off)) * W + d;
+        T* y = reinterpret_cast<T*>(dst) + e * s0 + h * s1 + t * s2 + d;
+        if constexpr (VEC == 4) {
+            struct alignas(4 * sizeof(T)) Quad { T v[4]; };
+            const float4 v = *reinterpret_cast<const float4*>(x);
+            *reinterpret_cast<Quad*>(y) = Quad{{from_f<T>(v.x), from_f<T>(v.y), from_f<T>(v.z), from_f<T>(v.w)}};
+        } else {
+            *y = from_f<T>(*x);
+        }
     }
 }
 
@@ -395,11 +404,17 @@ int launch_bwd_r(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, boo
 }
 
 int launch_bwd_out(const float* src, void* dst, const long long* st, int dt, const Problem& P, int W, hipStream_t s) {
-    const long long total = static_cast<long long>(P.E) * P.H * P.N * W;
     return dispatch_qk(dt, [&](auto t) {
         using T = decltype(t);
-        hipLaunchKernelGGL((grad_out_kernel<T>), dim3(blocks_for(total)), dim3(256), 0, s, src, static_cast<char*>(dst), st[0], st[1],
-                           st[2], P.E, P.H, P.N, P.M * P.B, W, P.pad_off);
+        const bool vec = W % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % (4 * sizeof(T)) == 0 && st[0] % 4 == 0 && st[1] % 4 == 0 &&
+                         st[2] % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0;
+        const long long total = static_cast<long long>(P.E) * P.H * P.N * (vec ? W / 4 : W);
+        if (vec)
+            hipLaunchKernelGGL((grad_out_kernel<T, 4>), dim3(blocks_for(total)), dim3(256), 0, s, src, static_cast<char*>(dst), st[0],
+                               st[1], st[2], P.E, P.H, P.N, P.M * P.B, W, P.pad_off);
+        else
+            hipLaunchKernelGGL((grad_out_kernel<T, 1>), dim3(blocks_for(total)), dim3(256), 0, s, src, static_cast<char*>(dst), st[0],
+                               st[1], st[2], P.E, P.H, P.N, P.M * P.B, W, P.pad_off);
         return static_cast<int>(hipGetLastError());
     });
 }
