@@ -186,3 +186,54 @@ def test_auto_variant_policy():
     assert auto(1, 16, 4096, 64, 64, Dv=128) == "generic"
     assert auto(1, 16, 4096, 60, 64) == "generic"       # D % 8 != 0
     assert auto(1, 16, 4096, 64, 256) == "generic"      # B > 128
+
+
+def good_bwd_params(**kw):
+    b = L.BwdParams()
+    b.fwd = good_params(**kw)
+    for name, inner in (("dout_stride", 16), ("dq_stride", 16), ("dk_stride", 16), ("dv_stride", 16)):
+        setattr(b, name, (C.c_int64 * 3)(3 * 50 * inner, 50 * inner, inner))
+    return b
+
+
+def test_backward_workspace_and_argument_checks_precede_any_launch():
+    """ma_bwd validates before it launches: everything here runs without a GPU."""
+    lib = L.load()
+    b = good_bwd_params()
+    need = lib.ma_bwd_workspace_bytes(b)
+    rows, T, D = 2 * 3 * 7 * 8, 2, 16
+    # every step's state (T aL + T-1 aR slots of 16-bit rows), fp32 state gradients and fp32 dq, dk, dv
+    assert need >= (2 * T - 1) * rows * D * 2 + 3 * rows * D * 4 + 3 * rows * D * 4
+    assert need % 256 == 0
+    assert lib.ma_bwd_workspace_bytes(good_bwd_params(T=3)) > need
+    assert lib.ma_bwd(None, None) == L.MA_ERR_NULL
+    assert lib.ma_bwd(b, None) == L.MA_ERR_NULL                        # q / k / v / dout / dq / dk / dv NULL
+    b.fwd.q = b.fwd.k = b.fwd.v = b.dout = b.dq = b.dk = b.dv = 0x10000
+    assert lib.ma_bwd(b, None) == L.MA_ERR_WORKSPACE                   # fwd.out is not needed; no workspace
+    b.fwd.workspace, b.fwd.workspace_bytes = 0x100000, need - 1
+    assert lib.ma_bwd(b, None) == L.MA_ERR_WORKSPACE                   # too small
+    b.fwd.workspace, b.fwd.workspace_bytes = 0x100010, need
+    assert lib.ma_bwd(b, None) == L.MA_ERR_WORKSPACE                   # misaligned
+    b.fwd.workspace = 0x100000
+    b.dq = 0x10001                                                     # fp16 pointer must be 2-byte aligned
+    assert lib.ma_bwd(b, None) == L.MA_ERR_STRIDE
+    b.dq = 0x10000
+    for name in ("fused", "resident", "chained"):                      # the T steps run as separate launches
+        b.fwd.variant = L.VARIANTS[name]
+        assert lib.ma_bwd(b, None) == L.MA_ERR_UNSUPPORTED
+        assert lib.ma_bwd_workspace_bytes(b) == 0
+    b.fwd.variant = L.VARIANTS["auto"]
+    b.dk_stride = (C.c_int64 * 3)(0, 50 * 16, 16)                      # gradient slices of batch entries coincide
+    assert lib.ma_bwd(b, None) == L.MA_ERR_STRIDE
+    b.dk_stride = (C.c_int64 * 3)(3 * 50 * 16, 50 * 16, 8)             # rows of dk overlap
+    assert lib.ma_bwd(b, None) == L.MA_ERR_STRIDE
+    bad = good_bwd_params(B=5000)                                      # beyond the backward kernels' block size
+    bad.fwd.N = 20000
+    bad.fwd.q = bad.fwd.k = bad.fwd.v = bad.dout = bad.dq = bad.dk = bad.dv = 0x10000
+    for name in ("q_stride", "k_stride", "v_stride", "out_stride"):
+        setattr(bad.fwd, name, (C.c_int64 * 3)(3 * 20000 * 16, 20000 * 16, 16))
+    for name in ("dout_stride", "dq_stride", "dk_stride", "dv_stride"):
+        setattr(bad, name, (C.c_int64 * 3)(3 * 20000 * 16, 20000 * 16, 16))
+    need = lib.ma_bwd_workspace_bytes(bad)
+    bad.fwd.workspace, bad.fwd.workspace_bytes = 0x100000, need
+    assert need > 0 and lib.ma_bwd(bad, None) == L.MA_ERR_UNSUPPORTED
