@@ -281,8 +281,6 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             strip_mma(acc, nt, Qt + r0 * ldd, ldd, 1, aLt + c0 * ldd, 1, ldd, D16);
             strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) { U[ll * ldm + k] = k < M ? round_to<TQ>(x) - cl[k] : -INFINITY; });
         });
-        __syncthreads();
-        softmax_rows_lds<NTH>(U, ldm, TL, M16);
         // Z: gLz = dO Y^T;  L: gLm = mask_q (Qt gaR^T + gcR)
         for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
@@ -295,6 +293,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             });
         });
         __syncthreads();
+        softmax_rows_lds<NTH>(U, ldm, TL, M16);   // a wave has the same rows here and in the pass below
         {   // dU = p (g - sum g p); afterwards U holds the rounded (L: query-masked) probabilities
             const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
             for (int ll = wave; ll < TL; ll += NTH / 64) {
@@ -442,8 +441,17 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             strip_each(acc, nt, r0, c0,
                        [&](int jj, int i, float x) { S[jj * ldb + i] = kok[i] != 0.f ? sm * round_to<TQ>(x) * c[jj] : -INFINITY; });
         });
+        // sm gaL K^T + gY V^T, the part of g that does not need the probabilities
+        for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma(acc, nt, Ga + r0 * lga, lga, 1, Kt + c0 * ldd, 1, ldd, D16);
+            if (with_v) strip_mma(acc, nt, Gy + r0 * lgy, lgy, 1, Vt + c0 * ldv, 1, ldv, V16);
+            strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) { Gg[jj * ldb + i] = x; });
+        });
         __syncthreads();
-        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // probabilities (ma_torch.py:14-18); Gg <- 1 where the clamp did not act
+        for (int jj = wave; jj < TJ; jj += NTH / 64) {
+            // probabilities (ma_torch.py:14-18)
             float mx = -INFINITY;
             for (int i = lane; i < B16; i += 64) mx = fmaxf(mx, S[jj * ldb + i]);
             mx = fmaxf(wmax(mx), P.eps);
@@ -454,29 +462,18 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
                 sum += p;
             }
             const float inv = 1.0f / (wsum(sum) + P.eps);
+            // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act, else 0
+            float dot = 0.f;
             for (int i = lane; i < B16; i += 64) {
                 const float r = R[jj * ldb + i] * inv;
-                Gg[jj * ldb + i] = (i < B && r >= kTiny) ? 1.f : 0.f;
-                R[jj * ldb + i] = i < B ? fmaxf(r, kTiny) : 0.f;
+                const float rc = i < B ? fmaxf(r, kTiny) : 0.f;
+                const float g = (i < B && r >= kTiny) ? fmaf(gcl[jj], __logf(rc) + 1.0f, Gg[jj * ldb + i]) : 0.f;
+                R[jj * ldb + i] = rc;
+                Gg[jj * ldb + i] = g;
+                dot = fmaf(g, rc, dot);
             }
-        }
-        __syncthreads();
-        // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act
-        for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
-            f32x4 acc[4];
-            zero_acc(acc);
-            strip_mma(acc, nt, Ga + r0 * lga, lga, 1, Kt + c0 * ldd, 1, ldd, D16);
-            if (with_v) strip_mma(acc, nt, Gy + r0 * lgy, lgy, 1, Vt + c0 * ldv, 1, ldv, V16);
-            strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) {
-                float* g = Gg + jj * ldb + i;
-                *g = *g != 0.f ? fmaf(gcl[jj], __logf(R[jj * ldb + i]) + 1.0f, x) : 0.f;
-            });
-        });
-        __syncthreads();
-        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // dS, gcR; Gg <- dDot = dS sm / (cR + eps); R <- round(r)
-            float dot = 0.f;
-            for (int i = lane; i < B16; i += 64) dot = fmaf(Gg[jj * ldb + i], R[jj * ldb + i], dot);
             dot = wsum(dot);
+            // dS, gcR; Gg <- dDot = dS sm / (cR + eps); R <- round(r)
             float gc = 0.f;
             for (int i = lane; i < B16; i += 64) {
                 const float s = S[jj * ldb + i], r = R[jj * ldb + i];
@@ -686,8 +683,6 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             strip_mma16<false, false>(acc, nt, Qt + r0 * ldd, ldd, aLt + c0 * ldd, ldd, D16);
             strip_each(acc, nt, r0, c0, [&](int ll, int k, float x) { U[ll * ldm + k] = k < M ? round_to<TQ>(x) - cl[k] : -INFINITY; });
         });
-        __syncthreads();
-        softmax_rows_lds<NTH>(U, ldm, TL, M16);
         // Z: gLz = dO Y^T;  L: gLm = mask_q (Qt gaR^T + gcR)
         for_strips<NTH>(TL, M16, [&](int r0, int c0, int nt) {
             f32x4 acc[4];
@@ -700,6 +695,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             });
         });
         __syncthreads();
+        softmax_rows_lds<NTH>(U, ldm, TL, M16);   // a wave has the same rows here and in the pass below
         {   // dU = p (g - sum g p); U16 <- rounded (L: query-masked) probabilities, G16 <- rounded dU
             const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
             for (int ll = wave; ll < TL; ll += NTH / 64) {
@@ -847,8 +843,17 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             strip_each(acc, nt, r0, c0,
                        [&](int jj, int i, float x) { S[jj * ldb + i] = kok[i] != 0.f ? sm * round_to<TQ>(x) * c[jj] : -INFINITY; });
         });
+        // sm gaL K^T + gY V^T, the part of g that does not need the probabilities
+        for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
+            f32x4 acc[4];
+            zero_acc(acc);
+            strip_mma16<false, false>(acc, nt, Ga + r0 * ldd, ldd, Kt + c0 * ldd, ldd, D16);
+            if (with_v) strip_mma16<false, false>(acc, nt, Gy + r0 * ldv, ldv, Vt + c0 * ldv, ldv, V16);
+            strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) { Gg[jj * ldb + i] = x; });
+        });
         __syncthreads();
-        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // probabilities (ma_torch.py:14-18); Gg <- 1 where the clamp did not act
+        for (int jj = wave; jj < TJ; jj += NTH / 64) {
+            // probabilities (ma_torch.py:14-18)
             float mx = -INFINITY;
             for (int i = lane; i < B16; i += 64) mx = fmaxf(mx, S[jj * ldb + i]);
             mx = fmaxf(wmax(mx), P.eps);
@@ -859,29 +864,18 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
                 sum += p;
             }
             const float inv = 1.0f / (wsum(sum) + P.eps);
+            // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act, else 0
+            float dot = 0.f;
             for (int i = lane; i < B16; i += 64) {
                 const float r = R[jj * ldb + i] * inv;
-                Gg[jj * ldb + i] = (i < B && r >= kTiny) ? 1.f : 0.f;
-                R[jj * ldb + i] = i < B ? fmaxf(r, kTiny) : 0.f;
+                const float rc = i < B ? fmaxf(r, kTiny) : 0.f;
+                const float g = (i < B && r >= kTiny) ? fmaf(gcl[jj], __logf(rc) + 1.0f, Gg[jj * ldb + i]) : 0.f;
+                R[jj * ldb + i] = rc;
+                Gg[jj * ldb + i] = g;
+                dot = fmaf(g, rc, dot);
             }
-        }
-        __syncthreads();
-        // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act
-        for_strips<NTH>(TJ, B16, [&](int r0, int c0, int nt) {
-            f32x4 acc[4];
-            zero_acc(acc);
-            strip_mma16<false, false>(acc, nt, Ga + r0 * ldd, ldd, Kt + c0 * ldd, ldd, D16);
-            if (with_v) strip_mma16<false, false>(acc, nt, Gy + r0 * ldv, ldv, Vt + c0 * ldv, ldv, V16);
-            strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) {
-                float* g = Gg + jj * ldb + i;
-                *g = *g != 0.f ? fmaf(gcl[jj], __logf(R[jj * ldb + i]) + 1.0f, x) : 0.f;
-            });
-        });
-        __syncthreads();
-        for (int jj = wave; jj < TJ; jj += NTH / 64) {   // dS, gcR; D16 <- dDot = dS sm / (cR + eps); R16 <- round(r)
-            float dot = 0.f;
-            for (int i = lane; i < B16; i += 64) dot = fmaf(Gg[jj * ldb + i], R[jj * ldb + i], dot);
             dot = wsum(dot);
+            // dS, gcR; D16 <- dDot = dS sm / (cR + eps); R16 <- round(r)
             float gc = 0.f;
             for (int i = lane; i < B16; i += 64) {
                 const float s = S[jj * ldb + i], r = R[jj * ldb + i];
