@@ -58,6 +58,10 @@ CASES = [  # E, H, N, D, Dv, B, T, pre, dt, masked
     (1, 2, 300, 40, 40, 32, 3, False, "bf16", True), (1, 1, 5, 4, 4, 8, 2, False, "f32", False),
     (1, 4, 256, 64, 64, 16, 2, False, "f32", False), (1, 2, 130, 16, 16, 1, 1, False, "f32", False),
     (1, 2, 48, 16, 16, 64, 2, True, "f32", True), (1, 1, 700, 8, 8, 2, 2, False, "f32", False),
+    # problems walked in several row tiles: 128 key blocks (L / Z stages), 128-row blocks with d = 128 (R stage;
+    # in fp32 that one is beyond the matrix-core kernels' LDS and takes the FMA kernels)
+    (1, 2, 1024, 64, 64, 8, 2, False, "bf16", True), (1, 2, 1024, 64, 64, 8, 2, False, "f32", False),
+    (1, 2, 256, 128, 128, 128, 2, False, "f16", False), (1, 1, 256, 128, 128, 128, 2, True, "f32", True),
 ]
 
 
