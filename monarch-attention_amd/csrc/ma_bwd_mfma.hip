@@ -36,6 +36,50 @@ __host__ __device__ constexpr int up(int x, int m) { return (x + m - 1) / m * m;
 __device__ __forceinline__ float wmax(float x) { return mfma::quad_rows_max(mfma::row16_max(x)); }
 __device__ __forceinline__ float wsum(float x) { return mfma::quad_rows_sum(mfma::row16_sum(x)); }
 
+// all-reduce over aligned groups of G lanes (G = 4 .. 64, a power of two).  The row passes give a
+// matrix row to G lanes, so that a wave works on 64 / G rows at once: short rows (small blocks)
+// would otherwise leave most lanes idle and walk the rows one after the other.
+template <int G>
+__device__ __forceinline__ float seg_max(float x) {
+    x = fmaxf(x, mfma::dpp<0xB1>(x));
+    x = fmaxf(x, mfma::dpp<0x4E>(x));
+    if (G >= 8) x = fmaxf(x, mfma::dpp<0x141>(x));
+    if (G >= 16) x = fmaxf(x, mfma::dpp<0x140>(x));
+    if (G >= 32) {
+        float a = x, b = x;
+        mfma::swap_rows16(a, b);
+        x = fmaxf(a, b);
+    }
+    if (G >= 64) {
+        float a = x, b = x;
+        mfma::swap_halves32(a, b);
+        x = fmaxf(a, b);
+    }
+    return x;
+}
+template <int G>
+__device__ __forceinline__ float seg_sum(float x) {
+    x += mfma::dpp<0xB1>(x);
+    x += mfma::dpp<0x4E>(x);
+    if (G >= 8) x += mfma::dpp<0x141>(x);
+    if (G >= 16) x += mfma::dpp<0x140>(x);
+    if (G >= 32) {
+        float a = x, b = x;
+        mfma::swap_rows16(a, b);
+        x = a + b;
+    }
+    if (G >= 64) {
+        float a = x, b = x;
+        mfma::swap_halves32(a, b);
+        x = a + b;
+    }
+    return x;
+}
+// lanes per row for rows of n (a multiple of 16) entries: four entries per lane for short rows, the
+// whole wave for rows of more than 32 entries (measured: there the one-row-per-wave walk, with its
+// conflict-free LDS accesses, is the faster one)
+inline int group_lanes(int n) { return n <= 16 ? 4 : n <= 32 ? 8 : 64; }
+
 // acc[t] += sum_k A(r,k) B(k, 16 t + c) for one 16-row strip of up to four 16-column tiles.
 // A(r,k) = A[r*ars + k*acs], B(k,c) = B[k*brs + c*bcs]; K is a multiple of 16.  Lane (r = lane % 16,
 // q = lane / 16) feeds A(r, k0+q) and B(k0+q, r); acc[t][v] is C(4q+v, 16t+r).  The operands of four
@@ -624,7 +668,7 @@ __host__ __device__ inline LzLayout16 lz_layout16(int M, int D, int W, bool z, i
     return L;
 }
 
-template <class TQ, bool kZ, int NTH>
+template <class TQ, bool kZ, int NTH, int GL>
 __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, int TL) {
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];
     const int M = P.M, D = P.D, B = P.B, W = kZ ? P.Dv : P.D;
@@ -695,20 +739,34 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             });
         });
         __syncthreads();
-        softmax_rows_lds<NTH>(U, ldm, TL, M16);   // a wave has the same rows here and in the pass below
-        {   // dU = p (g - sum g p); U16 <- rounded (L: query-masked) probabilities, G16 <- rounded dU
-            const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-            for (int ll = wave; ll < TL; ll += NTH / 64) {
+        // per row: softmax, dU = p (g - sum g p); U16 <- rounded (L: query-masked) probabilities, G16 <- rounded dU
+        {
+            constexpr int RPP = 64 / GL;
+            const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane / GL, cg = lane % GL;
+            for (int l1 = wave * RPP; l1 < TL; l1 += (NTH / 64) * RPP) {
+                const int ll = l1 + sub;
+                float* Ul = U + ll * ldm;
+                float* Gl = Gg + ll * ldm;
+                float mx = -INFINITY;
+                for (int k = cg; k < M16; k += GL) mx = fmaxf(mx, Ul[k]);
+                mx = seg_max<GL>(mx);
+                float sum = 0.f;
+                for (int k = cg; k < M16; k += GL) {
+                    const float p = __expf(Ul[k] - mx);
+                    Ul[k] = p;
+                    sum += p;
+                }
+                const float inv = 1.0f / seg_sum<GL>(sum);
                 float dot = 0.f;
-                for (int k = lane; k < M16; k += 64) dot = fmaf(Gg[ll * ldm + k], U[ll * ldm + k], dot);
-                dot = wsum(dot);
+                for (int k = cg; k < M16; k += GL) dot = fmaf(Gl[k], Ul[k] * inv, dot);
+                dot = seg_sum<GL>(dot);
                 const float keep = kZ ? 1.f : qok[ll];
-                for (int k = lane; k < M16; k += 64) {
-                    const float p = U[ll * ldm + k];
-                    const float du = p * (Gg[ll * ldm + k] - dot);
-                    Gg[ll * ldm + k] = du;
+                for (int k = cg; k < M16; k += GL) {
+                    const float p = Ul[k] * inv;
+                    const float du = p * (Gl[k] - dot);
+                    Gl[k] = du;
                     G16[ll * ldp + k] = from_f<TQ>(du);
-                    U16[ll * ldu + k] = from_f<TQ>(keep * p);   // lands on fp32 entries this wave has read already
+                    U16[ll * ldu + k] = from_f<TQ>(keep * p);   // lands on fp32 entries these lanes have read already
                 }
             }
         }
@@ -780,7 +838,7 @@ __host__ __device__ inline RLayout16 r_layout16(int B, int D, int Dv, bool with_
     return L;
 }
 
-template <class TQ, int NTH>
+template <class TQ, int NTH, int GL>
 __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int TJ, int first, int with_v) {
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];
     const int B = P.B, M = P.M, D = P.D, Dv = P.Dv;
@@ -852,40 +910,48 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             strip_each(acc, nt, r0, c0, [&](int jj, int i, float x) { Gg[jj * ldb + i] = x; });
         });
         __syncthreads();
-        for (int jj = wave; jj < TJ; jj += NTH / 64) {
-            // probabilities (ma_torch.py:14-18)
-            float mx = -INFINITY;
-            for (int i = lane; i < B16; i += 64) mx = fmaxf(mx, S[jj * ldb + i]);
-            mx = fmaxf(wmax(mx), P.eps);
-            float sum = 0.f;
-            for (int i = lane; i < B16; i += 64) {
-                const float p = __expf(S[jj * ldb + i] - mx);
-                R[jj * ldb + i] = p;
-                sum += p;
+        {
+            constexpr int RPP = 64 / GL;
+            const int sub = lane / GL, cg = lane % GL;
+            for (int j1 = wave * RPP; j1 < TJ; j1 += (NTH / 64) * RPP) {
+                const int jj = j1 + sub;
+                float* Sj = S + jj * ldb;
+                float* Rj = R + jj * ldb;
+                float* Gj = Gg + jj * ldb;
+                // probabilities (ma_torch.py:14-18)
+                float mx = -INFINITY;
+                for (int i = cg; i < B16; i += GL) mx = fmaxf(mx, Sj[i]);
+                mx = fmaxf(seg_max<GL>(mx), P.eps);
+                float sum = 0.f;
+                for (int i = cg; i < B16; i += GL) {
+                    const float p = __expf(Sj[i] - mx);
+                    Rj[i] = p;
+                    sum += p;
+                }
+                const float inv = 1.0f / (seg_sum<GL>(sum) + P.eps);
+                // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act, else 0
+                float dot = 0.f;
+                for (int i = cg; i < B16; i += GL) {
+                    const float r = Rj[i] * inv;
+                    const float rc = i < B ? fmaxf(r, kTiny) : 0.f;
+                    const float g = (i < B && r >= kTiny) ? fmaf(gcl[jj], __logf(rc) + 1.0f, Gj[i]) : 0.f;
+                    Rj[i] = rc;
+                    Gj[i] = g;
+                    dot = fmaf(g, rc, dot);
+                }
+                dot = seg_sum<GL>(dot);
+                // dS, gcR; D16 <- dDot = dS sm / (cR + eps); R16 <- round(r)
+                float gc = 0.f;
+                for (int i = cg; i < B16; i += GL) {
+                    const float sv = Sj[i], r = Rj[i];
+                    const float ds = sv == -INFINITY ? 0.f : r * (Gj[i] - dot);
+                    if (sv != -INFINITY) gc = fmaf(-ds, sv * c[jj], gc);
+                    Dd[jj * ldp + i] = from_f<TQ>(ds * sm * c[jj]);   // both land on fp32 entries these lanes have read already
+                    R16[jj * ldp + i] = from_f<TQ>(r);
+                }
+                gc = seg_sum<GL>(gc);
+                if (!first && cg == 0 && j0 + jj < B) G.gcR[(eh * M + k) * B + j0 + jj] = gc;
             }
-            const float inv = 1.0f / (wsum(sum) + P.eps);
-            // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act, else 0
-            float dot = 0.f;
-            for (int i = lane; i < B16; i += 64) {
-                const float r = R[jj * ldb + i] * inv;
-                const float rc = i < B ? fmaxf(r, kTiny) : 0.f;
-                const float g = (i < B && r >= kTiny) ? fmaf(gcl[jj], __logf(rc) + 1.0f, Gg[jj * ldb + i]) : 0.f;
-                R[jj * ldb + i] = rc;
-                Gg[jj * ldb + i] = g;
-                dot = fmaf(g, rc, dot);
-            }
-            dot = wsum(dot);
-            // dS, gcR; D16 <- dDot = dS sm / (cR + eps); R16 <- round(r)
-            float gc = 0.f;
-            for (int i = lane; i < B16; i += 64) {
-                const float s = S[jj * ldb + i], r = R[jj * ldb + i];
-                const float ds = s == -INFINITY ? 0.f : r * (Gg[jj * ldb + i] - dot);
-                if (s != -INFINITY) gc = fmaf(-ds, s * c[jj], gc);
-                Dd[jj * ldp + i] = from_f<TQ>(ds * sm * c[jj]);   // both land on fp32 entries this wave has read already
-                R16[jj * ldp + i] = from_f<TQ>(r);
-            }
-            gc = wsum(gc);
-            if (!first && lane == 0 && j0 + jj < B) G.gcR[(eh * M + k) * B + j0 + jj] = gc;
         }
         __syncthreads();
         // gaR = dDot K (first step: aR is q, the rows of block k of dq)
@@ -958,9 +1024,14 @@ int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z,
             if (nth == 256) return z ? launch(lz_bwd_mfma<TQ, true, 256>) : launch(lz_bwd_mfma<TQ, false, 256>);
             return z ? launch(lz_bwd_mfma<TQ, true, 1024>) : launch(lz_bwd_mfma<TQ, false, 1024>);
         } else {
-            if (nth == 64) return z ? launch(lz_bwd_mfma16<TQ, true, 64>) : launch(lz_bwd_mfma16<TQ, false, 64>);
-            if (nth == 256) return z ? launch(lz_bwd_mfma16<TQ, true, 256>) : launch(lz_bwd_mfma16<TQ, false, 256>);
-            return z ? launch(lz_bwd_mfma16<TQ, true, 1024>) : launch(lz_bwd_mfma16<TQ, false, 1024>);
+            // lanes per probability row: short rows go with the small workgroups
+            const int gl = group_lanes(up(P.M, 16));
+            if (nth == 64 && gl == 4) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 4>) : launch(lz_bwd_mfma16<TQ, false, 64, 4>);
+            if (nth == 64 && gl == 8) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 8>) : launch(lz_bwd_mfma16<TQ, false, 64, 8>);
+            if (nth == 64) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 64>) : launch(lz_bwd_mfma16<TQ, false, 64, 64>);
+            if (nth == 256 && gl == 8) return z ? launch(lz_bwd_mfma16<TQ, true, 256, 8>) : launch(lz_bwd_mfma16<TQ, false, 256, 8>);
+            if (nth == 256) return z ? launch(lz_bwd_mfma16<TQ, true, 256, 64>) : launch(lz_bwd_mfma16<TQ, false, 256, 64>);
+            return z ? launch(lz_bwd_mfma16<TQ, true, 1024, 64>) : launch(lz_bwd_mfma16<TQ, false, 1024, 64>);
         }
     });
 }
@@ -987,9 +1058,13 @@ int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool fir
             if (nth == 256) return launch(r_bwd_mfma<TQ, 256>);
             return launch(r_bwd_mfma<TQ, 1024>);
         } else {
-            if (nth == 64) return launch(r_bwd_mfma16<TQ, 64>);
-            if (nth == 256) return launch(r_bwd_mfma16<TQ, 256>);
-            return launch(r_bwd_mfma16<TQ, 1024>);
+            const int gl = group_lanes(up(P.B, 16));
+            if (nth == 64 && gl == 4) return launch(r_bwd_mfma16<TQ, 64, 4>);
+            if (nth == 64 && gl == 8) return launch(r_bwd_mfma16<TQ, 64, 8>);
+            if (nth == 64) return launch(r_bwd_mfma16<TQ, 64, 64>);
+            if (nth == 256 && gl == 8) return launch(r_bwd_mfma16<TQ, 256, 8>);
+            if (nth == 256) return launch(r_bwd_mfma16<TQ, 256, 64>);
+            return launch(r_bwd_mfma16<TQ, 1024, 64>);
         }
     });
 }
