@@ -215,6 +215,71 @@ __device__ __forceinline__ void stage_rows(TD* dst, int ld, int rows, int width,
     }
 }
 
+// Several tiles staged together: the loads of all of them are issued before any is written to LDS,
+// so a stage waits for one memory round trip instead of one per tile.  Same work split and same
+// zero-filling as stage_rows; the tiles may differ in rows, width and types.  Costs registers: used
+// by the single-wave workgroups of small blocks, whose stages are one chain of memory round trips.
+template <class T, class TD, class RowPtr>
+struct TileSpec {
+    struct alignas(4 * sizeof(T)) Quad { T v[4]; };
+    struct alignas(2 * sizeof(TD)) Pair { TD a, b; };
+    TD* dst;
+    int ld, rows, width, W;
+    float scale;
+    RowPtr row_ptr;
+    const T* p[2];
+    Quad x[2];
+
+    __device__ __forceinline__ void rows_begin(int i0, int step) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) p[u] = i0 + step * u < rows ? row_ptr(i0 + step * u) : nullptr;
+    }
+    __device__ __forceinline__ void load(int c) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            if (p[u] != nullptr && W % 4 == 0 && reinterpret_cast<uintptr_t>(p[u]) % sizeof(Quad) == 0 && 4 * c < W) {
+                x[u] = *reinterpret_cast<const Quad*>(p[u] + 4 * c);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x[u].v[e] = (p[u] != nullptr && 4 * c + e < W) ? p[u][4 * c + e] : from_f<T>(0.f);
+            }
+        }
+    }
+    __device__ __forceinline__ void store(int i0, int step, int c) const {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int i = i0 + step * u;
+            if (i >= rows || 4 * c >= width) continue;
+            TD* d = dst + i * ld + 4 * c;
+            if constexpr (sizeof(TD) == 4) {
+                *reinterpret_cast<f32x4*>(d) = f32x4{scale * to_f(x[u].v[0]), scale * to_f(x[u].v[1]), scale * to_f(x[u].v[2]),
+                                                     scale * to_f(x[u].v[3])};
+            } else {
+                *reinterpret_cast<Pair*>(d) = Pair{from_f<TD>(scale * to_f(x[u].v[0])), from_f<TD>(scale * to_f(x[u].v[1]))};
+                *reinterpret_cast<Pair*>(d + 2) = Pair{from_f<TD>(scale * to_f(x[u].v[2])), from_f<TD>(scale * to_f(x[u].v[3]))};
+            }
+        }
+    }
+};
+template <class T, class TD, class RowPtr>
+__device__ __forceinline__ TileSpec<T, TD, RowPtr> tile_of(TD* dst, int ld, int rows, int width, int W, float scale, RowPtr row_ptr) {
+    return TileSpec<T, TD, RowPtr>{dst, ld, rows, width, W, scale, row_ptr, {nullptr, nullptr}, {}};
+}
+template <int NTH, class... Ts>
+__device__ __forceinline__ void stage_tiles(Ts... t) {
+    constexpr int NW = NTH / 64;
+    const int lane = threadIdx.x & 63, sub = lane >> 4, c0 = lane & 15;
+    int rows = 0, width = 0;
+    ((rows = max(rows, t.rows), width = max(width, t.width)), ...);
+    for (int i0 = 4 * (threadIdx.x >> 6) + sub; i0 < rows; i0 += 8 * NW) {
+        (t.rows_begin(i0, 4 * NW), ...);
+        for (int c = c0; 4 * c < width; c += 16) {
+            (t.load(c), ...);
+            (t.store(i0, 4 * NW, c), ...);
+        }
+    }
+}
+
 // softmax over columns [0, cols) of every row of U[rows][ld], in place (entries may be -inf)
 template <int NTH>
 __device__ __forceinline__ void softmax_rows_lds(float* U, int ld, int rows, int cols) {
@@ -695,13 +760,15 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
     TQ* G16 = reinterpret_cast<TQ*>(lds_raw + L.G16);
 
     const TQ* aL = reinterpret_cast<const TQ*>(P.aL) + jm * D;
-    stage_rows<NTH, TQ, TQ>(aLt, ldd, M16, D16, D, 1.f, [&](int k) { return k < M ? aL + k * D : nullptr; });
-    if (kZ) {
-        const TQ* Y = reinterpret_cast<const TQ*>(P.Y) + jm * W;
-        stage_rows<NTH, TQ, TQ>(Wt, ldw, M16, W16, W, 1.f, [&](int k) { return k < M ? Y + k * static_cast<long long>(W) : nullptr; });
-    } else {
-        stage_rows<NTH, float, TQ>(Wt, ldw, M16, W16, W, 1.f,
-                                   [&](int k) { return k < M ? G.gaR + ((eh * M + k) * B + j) * D : nullptr; });
+    const TQ* Y = reinterpret_cast<const TQ*>(P.Y) + jm * W;
+    auto aL_row = [=](int k) { return k < M ? aL + k * D : nullptr; };
+    auto y_row = [=](int k) { return k < M ? Y + k * static_cast<long long>(W) : nullptr; };
+    auto gar_row = [=](int k) { return k < M ? G.gaR + ((eh * M + k) * B + j) * D : nullptr; };
+    constexpr bool kJoint = NTH == 64;   // single-wave workgroups stage all their tiles in one go
+    if (!kJoint) {
+        stage_rows<NTH, TQ, TQ>(aLt, ldd, M16, D16, D, 1.f, aL_row);
+        if (kZ) stage_rows<NTH, TQ, TQ>(Wt, ldw, M16, W16, W, 1.f, y_row);
+        else stage_rows<NTH, float, TQ>(Wt, ldw, M16, W16, W, 1.f, gar_row);
     }
     for (int k = threadIdx.x; k < M16; k += NTH) {
         cl[k] = k < M ? P.cL[jm + k] : 0.f;
@@ -709,13 +776,24 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
     }
 
     for (int l0 = 0; l0 < M; l0 += TL) {
-        stage_rows<NTH, TQ, TQ>(Qt, ldd, TL, D16, D, 1.f, [&](int ll) {
+        auto q_row = [=](int ll) {
             return l0 + ll < M ? tok_row<TQ>(P.q, P.qs, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
-        });
-        if (kZ)
-            stage_rows<NTH, TQ, TQ>(dO, ldw, TL, W16, W, 1.f, [&](int ll) {
-                return l0 + ll < M ? tok_row<TQ>(G.dout, G.dos, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
-            });
+        };
+        auto do_row = [=](int ll) {
+            return l0 + ll < M ? tok_row<TQ>(G.dout, G.dos, e, h, (l0 + ll) * B + j - P.pad_off, P.N) : nullptr;
+        };
+        if (kJoint) {   // the state tiles of the whole problem travel with the first tile of query blocks
+            const int state_rows = l0 == 0 ? M16 : 0;
+            if (kZ)
+                stage_tiles<NTH>(tile_of<TQ>(aLt, ldd, state_rows, D16, D, 1.f, aL_row), tile_of<TQ>(Wt, ldw, state_rows, W16, W, 1.f, y_row),
+                                 tile_of<TQ>(Qt, ldd, TL, D16, D, 1.f, q_row), tile_of<TQ>(dO, ldw, TL, W16, W, 1.f, do_row));
+            else
+                stage_tiles<NTH>(tile_of<TQ>(aLt, ldd, state_rows, D16, D, 1.f, aL_row),
+                                 tile_of<float>(Wt, ldw, state_rows, W16, W, 1.f, gar_row), tile_of<TQ>(Qt, ldd, TL, D16, D, 1.f, q_row));
+        } else {
+            stage_rows<NTH, TQ, TQ>(Qt, ldd, TL, D16, D, 1.f, q_row);
+            if (kZ) stage_rows<NTH, TQ, TQ>(dO, ldw, TL, W16, W, 1.f, do_row);
+        }
         for (int ll = threadIdx.x; ll < TL; ll += NTH)
             qok[ll] = (l0 + ll < M && token_ok(P, e, (l0 + ll) * B + j - P.pad_off)) ? 1.f : 0.f;
         __syncthreads();
@@ -868,24 +946,34 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
     TQa* Dd = reinterpret_cast<TQa*>(lds_raw + L.Gg);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-    stage_rows<NTH, TQ, TQ>(Kt, ldd, B16, D16, D, 1.f,
-                            [&](int i) { return i < B ? tok_row<TQ>(P.k, P.ks, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
-    if (with_v)
-        stage_rows<NTH, TQ, TQ>(Vt, ldv, B16, V16, Dv, 1.f,
-                                [&](int i) { return i < B ? tok_row<TQ>(P.v, P.vs, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
+    auto k_row = [=](int i) { return i < B ? tok_row<TQ>(P.k, P.ks, e, h, k * B + i - P.pad_off, P.N) : nullptr; };
+    auto v_row = [=](int i) { return i < B ? tok_row<TQ>(P.v, P.vs, e, h, k * B + i - P.pad_off, P.N) : nullptr; };
+    constexpr bool kJoint = NTH == 64;   // single-wave workgroups stage all their tiles in one go
+    if (!kJoint) {
+        stage_rows<NTH, TQ, TQ>(Kt, ldd, B16, D16, D, 1.f, k_row);
+        if (with_v) stage_rows<NTH, TQ, TQ>(Vt, ldv, B16, V16, Dv, 1.f, v_row);
+    }
     for (int i = threadIdx.x; i < B16; i += NTH) kok[i] = (i < B && token_ok(P, e, k * B + i - P.pad_off)) ? 1.f : 0.f;
 
     for (int j0 = 0; j0 < B; j0 += TJ) {
-        stage_rows<NTH, TQ, TQ>(X, ldd, TJ, D16, D, 1.f, [&](int jj) -> const TQ* {
+        auto x_row = [=](int jj) -> const TQ* {
             if (j0 + jj >= B) return nullptr;
             return first ? tok_row<TQ>(P.q, P.qs, e, h, k * B + j0 + jj - P.pad_off, P.N) : aR + (j0 + jj) * D;
-        });
-        stage_rows<NTH, float, TQ>(Ga, ldd, TJ, D16, D, sm,
-                                   [&](int jj) { return j0 + jj < B ? G.gaL + ((eh * B + j0 + jj) * M + k) * D : nullptr; });
-        if (with_v)
-            stage_rows<NTH, float, TQ>(Gy, ldv, TJ, V16, Dv, 1.f, [&](int jj) {
-                return j0 + jj < B ? G.gY + ((eh * B + j0 + jj) * M + k) * static_cast<long long>(Dv) : nullptr;
-            });
+        };
+        auto ga_row = [=](int jj) { return j0 + jj < B ? G.gaL + ((eh * B + j0 + jj) * M + k) * D : nullptr; };
+        auto gy_row = [=](int jj) {
+            return j0 + jj < B ? G.gY + ((eh * B + j0 + jj) * M + k) * static_cast<long long>(Dv) : nullptr;
+        };
+        if (kJoint) {   // the key / value tiles of the block travel with the first tile of query rows
+            const int kv_rows = j0 == 0 ? B16 : 0;
+            stage_tiles<NTH>(tile_of<TQ>(Kt, ldd, kv_rows, D16, D, 1.f, k_row),
+                             tile_of<TQ>(Vt, ldv, with_v ? kv_rows : 0, V16, Dv, 1.f, v_row), tile_of<TQ>(X, ldd, TJ, D16, D, 1.f, x_row),
+                             tile_of<float>(Ga, ldd, TJ, D16, D, sm, ga_row), tile_of<float>(Gy, ldv, with_v ? TJ : 0, V16, Dv, 1.f, gy_row));
+        } else {
+            stage_rows<NTH, TQ, TQ>(X, ldd, TJ, D16, D, 1.f, x_row);
+            stage_rows<NTH, float, TQ>(Ga, ldd, TJ, D16, D, sm, ga_row);
+            if (with_v) stage_rows<NTH, float, TQ>(Gy, ldv, TJ, V16, Dv, 1.f, gy_row);
+        }
         for (int jj = threadIdx.x; jj < TJ; jj += NTH) {
             const bool in = j0 + jj < B;
             c[jj] = 1.0f / (((first || !in) ? 1.0f : cR[j0 + jj]) + P.eps);   // c holds 1 / (cR + eps)
