@@ -447,7 +447,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             zero_acc(acc);
             strip_mma(acc, nt, Gg + r0 * ldm, ldm, 1, aLt + c0, ldd, 1, M16);
             if (!kZ) strip_mma(acc, nt, U + r0 * ldm, ldm, 1, Wt + c0, ldw, 1, M16);
-            strip_rmw(acc, nt, r0, c0, true, [&](int ll, int d) -> float* {
+            // the Z stage runs first and every dq row belongs to one tile of one workgroup: it is written, not added to
+            strip_rmw(acc, nt, r0, c0, !kZ, [&](int ll, int d) -> float* {
                 return (l0 + ll < M && d < D) ? G.dq + (eh * M * B + (l0 + ll) * B + j) * D + d : nullptr;
             });
         });
@@ -619,7 +620,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma(acc, nt, R + r0, 1, ldb, Gy + c0, lgy, 1, TJ);
-                strip_rmw(acc, nt, r0, c0, true, [&](int i, int d) -> float* {
+                strip_rmw(acc, nt, r0, c0, j0 != 0, [&](int i, int d) -> float* {   // dv has this one writer
                     return (i < B && d < Dv) ? G.dv + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d : nullptr;
                 });
             });
@@ -878,7 +879,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             zero_acc(acc);
             strip_mma16<false, true>(acc, nt, G16 + r0 * ldp, ldp, aLt + c0, ldd, M16);
             if (!kZ) strip_mma16<false, true>(acc, nt, reinterpret_cast<const TQ*>(U16) + r0 * ldu, ldu, Wt + c0, ldw, M16);
-            strip_rmw(acc, nt, r0, c0, true, [&](int ll, int d) -> float* {
+            // the Z stage runs first and every dq row belongs to one tile of one workgroup: it is written, not added to
+            strip_rmw(acc, nt, r0, c0, !kZ, [&](int ll, int d) -> float* {
                 return (l0 + ll < M && d < D) ? G.dq + (eh * M * B + (l0 + ll) * B + j) * D + d : nullptr;
             });
         });
@@ -1066,7 +1068,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(R16) + r0, ldp, Gy + c0, ldv, TJ);
-                strip_rmw(acc, nt, r0, c0, true, [&](int i, int d) -> float* {
+                strip_rmw(acc, nt, r0, c0, j0 != 0, [&](int i, int d) -> float* {   // dv has this one writer
                     return (i < B && d < Dv) ? G.dv + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d : nullptr;
                 });
             });
