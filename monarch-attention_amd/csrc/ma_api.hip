@@ -284,7 +284,8 @@ int prepare(const ma_fwd_params* p, Prepared* out) {
 // fp32 accumulators of the input gradients.
 struct BwdLayout {
     uint64_t aL, cL, aR, cR, Y, stats;      // aL / cL: T slots; aR / cR: T - 1 slots (steps 1..T-1)
-    uint64_t gaR, gcR, gaL, gcL, gY, dq, dk, dv;
+    uint64_t gaR, gcR, gaL, gcL, gY, dq, dk, dv, pk, pv;
+    int parts;                              // per-tile partial buffers of dk / dv (R stage split over workgroups)
     uint64_t slot_a, slot_c;                // bytes of one aL / aR slot and of one cL / cR slot
     uint64_t total;
 };
@@ -326,6 +327,14 @@ int bwd_prepare(const ma_bwd_params* b, ma_fwd_params* pp, BwdLayout* L) {
     L->dq = off; off += rows * pp->D * 4;
     L->dk = off; off += rows * pp->D * 4;
     L->dv = off; off = align_up(off + rows * pp->Dv * 4);
+    {
+        ma_ws_layout none;
+        std::memset(&none, 0, sizeof(none));
+        const Problem P = make_problem(pp, none);
+        L->parts = pp->variant == MA_VARIANT_GENERIC ? 0 : bwd_r_split_tiles(P, pp->dtype_qk, pp->dtype_v);
+    }
+    L->pk = off; off = align_up(off + static_cast<uint64_t>(L->parts) * rows * pp->D * 4);
+    L->pv = off; off = align_up(off + static_cast<uint64_t>(L->parts) * rows * pp->Dv * 4);
     L->total = off;
     return MA_OK;
 }
@@ -528,6 +537,9 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
     G.gY = reinterpret_cast<float*>(ws + L.gY);
     G.dq = reinterpret_cast<float*>(ws + L.dq); G.dk = reinterpret_cast<float*>(ws + L.dk); G.dv = reinterpret_cast<float*>(ws + L.dv);
     G.fma_only = fma_only ? 1 : 0;
+    G.pk = L.parts ? reinterpret_cast<float*>(ws + L.pk) : nullptr;
+    G.pv = L.parts ? reinterpret_cast<float*>(ws + L.pv) : nullptr;
+    G.jt_split = 0;
     G.dout = static_cast<const char*>(b->dout);
     for (int i = 0; i < 3; ++i) G.dos[i] = b->dout_stride[i];
     const long long rows = static_cast<long long>(P.E) * P.H * P.M * P.B;

@@ -498,9 +498,15 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
     const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
     const RLayout L = r_layout<TQ>(B, D, Dv, with_v != 0, TJ);
     const int ldd = L.ldd, ldv = L.ldv, lga = L.lga, lgy = L.lgy, ldb = L.ldb;
+    // G.jt_split > 0: the tiles of query rows of a block go to different workgroups (few, large blocks);
+    // their dk / dv parts then land in per-tile partial buffers that a reduction adds up in a fixed order
     int w = blockIdx.x;
+    const int jt = G.jt_split ? w % G.jt_split : 0;
+    if (G.jt_split) w /= G.jt_split;
     const int k = w % M; w /= M;
     const int h = w % P.H, e = w / P.H;
+    const int j_begin = G.jt_split ? jt * TJ : 0, j_end = G.jt_split ? min(B, j_begin + TJ) : B;
+    const long long part = static_cast<long long>(jt) * P.E * P.H * M * B;   // row offset into the partial buffers
     const long long eh = static_cast<long long>(e) * P.H + h;
     const TQ* aR = reinterpret_cast<const TQ*>(P.aR) + (eh * M + k) * B * D;
     const float* cR = P.cR + (eh * M + k) * B;
@@ -525,7 +531,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
                        [&](int i) { return i < B ? tok_row<TQ>(P.v, P.vs, e, h, k * B + i - P.pad_off, P.N) : nullptr; });
     for (int i = threadIdx.x; i < B16; i += NTH) kok[i] = (i < B && token_ok(P, e, k * B + i - P.pad_off)) ? 1.f : 0.f;
 
-    for (int j0 = 0; j0 < B; j0 += TJ) {
+    for (int j0 = j_begin; j0 < j_end; j0 += TJ) {
         stage_rows<NTH, TQ, TQ>(X, ldd, TJ, D16, D, 1.f, [&](int jj) -> const TQ* {
             if (j0 + jj >= B) return nullptr;
             return first ? tok_row<TQ>(P.q, P.qs, e, h, k * B + j0 + jj - P.pad_off, P.N) : aR + (j0 + jj) * D;
@@ -612,16 +618,19 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             zero_acc(acc);
             strip_mma(acc, nt, R + r0, 1, ldb, Ga + c0, lga, 1, TJ);
             strip_mma(acc, nt, Gg + r0, 1, ldb, X + c0, ldd, 1, TJ);
-            strip_rmw(acc, nt, r0, c0, true,
-                      [&](int i, int d) -> float* { return (i < B && d < D) ? G.dk + ((eh * M + k) * B + i) * D + d : nullptr; });
+            strip_rmw(acc, nt, r0, c0, !G.jt_split, [&](int i, int d) -> float* {
+                if (i >= B || d >= D) return nullptr;
+                return (G.jt_split ? G.pk + part * D : G.dk) + ((eh * M + k) * B + i) * D + d;
+            });
         });
         if (with_v)   // dV += round(r)^T gY
             for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma(acc, nt, R + r0, 1, ldb, Gy + c0, lgy, 1, TJ);
-                strip_rmw(acc, nt, r0, c0, j0 != 0, [&](int i, int d) -> float* {   // dv has this one writer
-                    return (i < B && d < Dv) ? G.dv + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d : nullptr;
+                strip_rmw(acc, nt, r0, c0, j0 != j_begin, [&](int i, int d) -> float* {   // dv has this one writer
+                    if (i >= B || d >= Dv) return nullptr;
+                    return (G.jt_split ? G.pv + part * Dv : G.dv) + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d;
                 });
             });
         __syncthreads();
@@ -925,9 +934,15 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
     const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
     const RLayout16 L = r_layout16(B, D, Dv, with_v != 0, TJ);
     const int ldd = L.ldd, ldv = L.ldv, ldb = L.ldb, ldp = 2 * L.ldb;
+    // G.jt_split > 0: the tiles of query rows of a block go to different workgroups (few, large blocks);
+    // their dk / dv parts then land in per-tile partial buffers that a reduction adds up in a fixed order
     int w = blockIdx.x;
+    const int jt = G.jt_split ? w % G.jt_split : 0;
+    if (G.jt_split) w /= G.jt_split;
     const int k = w % M; w /= M;
     const int h = w % P.H, e = w / P.H;
+    const int j_begin = G.jt_split ? jt * TJ : 0, j_end = G.jt_split ? min(B, j_begin + TJ) : B;
+    const long long part = static_cast<long long>(jt) * P.E * P.H * M * B;   // row offset into the partial buffers
     const long long eh = static_cast<long long>(e) * P.H + h;
     const TQ* aR = reinterpret_cast<const TQ*>(P.aR) + (eh * M + k) * B * D;
     const float* cR = P.cR + (eh * M + k) * B;
@@ -957,7 +972,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
     }
     for (int i = threadIdx.x; i < B16; i += NTH) kok[i] = (i < B && token_ok(P, e, k * B + i - P.pad_off)) ? 1.f : 0.f;
 
-    for (int j0 = 0; j0 < B; j0 += TJ) {
+    for (int j0 = j_begin; j0 < j_end; j0 += TJ) {
         auto x_row = [=](int jj) -> const TQ* {
             if (j0 + jj >= B) return nullptr;
             return first ? tok_row<TQ>(P.q, P.qs, e, h, k * B + j0 + jj - P.pad_off, P.N) : aR + (j0 + jj) * D;
@@ -967,7 +982,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             return j0 + jj < B ? G.gY + ((eh * B + j0 + jj) * M + k) * static_cast<long long>(Dv) : nullptr;
         };
         if (kJoint) {   // the key / value tiles of the block travel with the first tile of query rows
-            const int kv_rows = j0 == 0 ? B16 : 0;
+            const int kv_rows = j0 == j_begin ? B16 : 0;
             stage_tiles<NTH>(tile_of<TQ>(Kt, ldd, kv_rows, D16, D, 1.f, k_row),
                              tile_of<TQ>(Vt, ldv, with_v ? kv_rows : 0, V16, Dv, 1.f, v_row), tile_of<TQ>(X, ldd, TJ, D16, D, 1.f, x_row),
                              tile_of<float>(Ga, ldd, TJ, D16, D, sm, ga_row), tile_of<float>(Gy, ldv, with_v ? TJ : 0, V16, Dv, 1.f, gy_row));
@@ -1060,19 +1075,32 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             zero_acc(acc);
             strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(R16) + r0, ldp, Ga + c0, ldd, TJ);
             strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(Dd) + r0, ldp, X + c0, ldd, TJ);
-            strip_rmw(acc, nt, r0, c0, true,
-                      [&](int i, int d) -> float* { return (i < B && d < D) ? G.dk + ((eh * M + k) * B + i) * D + d : nullptr; });
+            strip_rmw(acc, nt, r0, c0, !G.jt_split, [&](int i, int d) -> float* {
+                if (i >= B || d >= D) return nullptr;
+                return (G.jt_split ? G.pk + part * D : G.dk) + ((eh * M + k) * B + i) * D + d;
+            });
         });
         if (with_v)   // dV += round(r)^T gY
             for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(R16) + r0, ldp, Gy + c0, ldv, TJ);
-                strip_rmw(acc, nt, r0, c0, j0 != 0, [&](int i, int d) -> float* {   // dv has this one writer
-                    return (i < B && d < Dv) ? G.dv + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d : nullptr;
+                strip_rmw(acc, nt, r0, c0, j0 != j_begin, [&](int i, int d) -> float* {   // dv has this one writer
+                    if (i >= B || d >= Dv) return nullptr;
+                    return (G.jt_split ? G.pv + part * Dv : G.dv) + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d;
                 });
             });
         __syncthreads();
+    }
+}
+
+// dst[i] += sum_t part[t][i], t ascending (n floats per part; four per thread)
+__global__ void add_parts_kernel(float* dst, const float* part, long long n, int parts, int assign) {
+    for (long long i = 4 * (blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x); i < n;
+         i += 4 * static_cast<long long>(gridDim.x) * blockDim.x) {
+        f32x4 acc = assign ? f32x4{0.f, 0.f, 0.f, 0.f} : *reinterpret_cast<const f32x4*>(dst + i);
+        for (int t = 0; t < parts; ++t) acc += *reinterpret_cast<const f32x4*>(part + t * n + i);
+        *reinterpret_cast<f32x4*>(dst + i) = acc;
     }
 }
 
@@ -1126,36 +1154,71 @@ int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z,
     });
 }
 
-int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool first, bool with_v, hipStream_t s) {
+// Tile of query rows of the R stage for a problem, 0 if it does not fit the LDS.
+static int r_tile(const Problem& P, int dt_qk, bool with_v) {
+    auto bytes = [&](int t) -> size_t {
+        return dt_qk == MA_F32 ? r_layout<float>(P.B, P.D, P.Dv, with_v, t).total : r_layout16(P.B, P.D, P.Dv, with_v, t).total;
+    };
+    return pick_tile(P.B, bytes);
+}
+
+// Number of per-tile partial buffers the R stage wants for dk / dv (0: none).  Splitting a block's
+// tiles of query rows over workgroups pays when the blocks alone cannot fill the chip.
+int bwd_r_split_tiles(const Problem& P, int dt_qk, int dt_v) {
+    if (dt_qk != dt_v) return 0;
+    const int TJ = r_tile(P, dt_qk, true);
+    if (TJ == 0) return 0;
+    const int tiles = (P.B + TJ - 1) / TJ;
+    const long long blocks = static_cast<long long>(P.E) * P.H * P.M;
+    const long long np = static_cast<long long>(P.M) * P.B;
+    return (tiles > 1 && blocks < 512 && (np * P.D) % 4 == 0 && (np * P.Dv) % 4 == 0) ? tiles : 0;
+}
+
+int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G0, int dt_qk, bool first, bool with_v, hipStream_t s) {
     return dispatch16(dt_qk, [&](auto tq) {
         using TQ = decltype(tq);
         constexpr bool k32 = sizeof(TQ) == 4;
         auto bytes = [&](int t) -> size_t {
             return k32 ? r_layout<TQ>(P.B, P.D, P.Dv, with_v, t).total : r_layout16(P.B, P.D, P.Dv, with_v, t).total;
         };
-        const int TJ = pick_tile(P.B, bytes);
+        int TJ = pick_tile(P.B, bytes);
         if (TJ == 0) return static_cast<int>(MA_ERR_UNSUPPORTED);
+        BwdBuffers G = G0;
+        // the partial buffers are sized for the tiling of the step that also forms dv (the smallest tile)
+        const int parts = G.pk != nullptr ? bwd_r_split_tiles(P, dt_qk, dt_qk) : 0;
+        G.jt_split = 0;
+        if (parts > 1) {
+            TJ = min(TJ, r_tile(P, dt_qk, true));
+            G.jt_split = (P.B + TJ - 1) / TJ;
+        }
         const size_t lds = bytes(TJ);
         const int nth = threads_for((TJ / 16) * (up(P.B, 16) / 16));
+        const long long grid = static_cast<long long>(P.E) * P.H * P.M * (G.jt_split ? G.jt_split : 1);
         auto launch = [&](auto kernel) {
             const int attr = mfma::set_lds_limit(kernel, kLdsBudget);
             if (attr) return attr;
-            hipLaunchKernelGGL(kernel, dim3(P.E * P.H * P.M), dim3(nth), lds, s, P, G, TJ, first ? 1 : 0, with_v ? 1 : 0);
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(nth), lds, s, P, G, TJ, first ? 1 : 0, with_v ? 1 : 0);
             return static_cast<int>(hipGetLastError());
         };
+        int st;
         if constexpr (k32) {
-            if (nth == 64) return launch(r_bwd_mfma<TQ, 64>);
-            if (nth == 256) return launch(r_bwd_mfma<TQ, 256>);
-            return launch(r_bwd_mfma<TQ, 1024>);
+            if (nth == 64) st = launch(r_bwd_mfma<TQ, 64>);
+            else if (nth == 256) st = launch(r_bwd_mfma<TQ, 256>);
+            else st = launch(r_bwd_mfma<TQ, 1024>);
         } else {
             const int gl = group_lanes(up(P.B, 16));
-            if (nth == 64 && gl == 4) return launch(r_bwd_mfma16<TQ, 64, 4>);
-            if (nth == 64 && gl == 8) return launch(r_bwd_mfma16<TQ, 64, 8>);
-            if (nth == 64) return launch(r_bwd_mfma16<TQ, 64, 64>);
-            if (nth == 256 && gl == 8) return launch(r_bwd_mfma16<TQ, 256, 8>);
-            if (nth == 256) return launch(r_bwd_mfma16<TQ, 256, 64>);
-            return launch(r_bwd_mfma16<TQ, 1024, 64>);
+            if (nth == 64 && gl == 4) st = launch(r_bwd_mfma16<TQ, 64, 4>);
+            else if (nth == 64 && gl == 8) st = launch(r_bwd_mfma16<TQ, 64, 8>);
+            else if (nth == 64) st = launch(r_bwd_mfma16<TQ, 64, 64>);
+            else if (nth == 256 && gl == 8) st = launch(r_bwd_mfma16<TQ, 256, 8>);
+            else if (nth == 256) st = launch(r_bwd_mfma16<TQ, 256, 64>);
+            else st = launch(r_bwd_mfma16<TQ, 1024, 64>);
         }
+        if (st || !G.jt_split) return st;
+        const long long rows = static_cast<long long>(P.E) * P.H * P.M * P.B;
+        hipLaunchKernelGGL(add_parts_kernel, dim3(1024), dim3(256), 0, s, G.dk, G.pk, rows * P.D, G.jt_split, 0);
+        if (with_v) hipLaunchKernelGGL(add_parts_kernel, dim3(1024), dim3(256), 0, s, G.dv, G.pv, rows * P.Dv, G.jt_split, 0);
+        return static_cast<int>(hipGetLastError());
     });
 }
 

@@ -69,7 +69,12 @@ struct BwdBuffers {
     const char* dout;
     long long dos[3];
     int fma_only;  // take the FMA kernels even where the matrix-core ones apply
+    float* pk;     // (parts,E,H,Np,D) / (parts,E,H,Np,Dv): per-tile parts of dk / dv of an R stage whose
+    float* pv;     //   tiles of query rows run in different workgroups; nullptr: never split
+    int jt_split;  // set by the launcher: workgroups per block (0 = one workgroup walks all tiles)
 };
+// partial buffers the R stage wants for this problem (0: it does not split blocks over workgroups)
+int bwd_r_split_tiles(const Problem& P, int dt_qk, int dt_v);
 bool bwd_fits(const Problem& P);
 // matrix-core backward stages: MA_ERR_UNSUPPORTED when the problem's tiles do not fit the LDS
 int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z, hipStream_t s);

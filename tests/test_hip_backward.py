@@ -62,6 +62,8 @@ CASES = [  # E, H, N, D, Dv, B, T, pre, dt, masked
     # in fp32 that one is beyond the matrix-core kernels' LDS and takes the FMA kernels)
     (1, 2, 1024, 64, 64, 8, 2, False, "bf16", True), (1, 2, 1024, 64, 64, 8, 2, False, "f32", False),
     (1, 2, 256, 128, 128, 128, 2, False, "f16", False), (1, 1, 256, 128, 128, 128, 2, True, "f32", True),
+    # few large blocks: the R stage gives a block's tiles of query rows to different workgroups (partial dk / dv)
+    (1, 2, 300, 48, 48, 128, 2, False, "f32", True), (1, 3, 260, 64, 64, 128, 3, True, "bf16", False),
 ]
 
 
