@@ -72,6 +72,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sdpa", action="store_true", help="skip the dense SDPA comparison")
     ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep")
+    ap.add_argument("--matrix", action="store_true",
+                    help="time ma_matrix (the dense (E,H,N,N) attention matrix of get_matrix) instead of the forward metric")
     ap.add_argument("--backward", action="store_true",
                     help="time ma_bwd (gradients of q, k, v; runs the T steps again) instead of the forward metric")
     args = ap.parse_args()
@@ -136,6 +138,26 @@ def main():
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
         return wall_ms, e0.elapsed_time(e1) / steps, ps, ws
+
+    if args.matrix:
+        from ma.ma_hip import monarch_matrix_hip
+        q, k, _, _ = sets[0]
+        variant = args.variant if args.variant in ("auto", "generic", "staged") else "auto"
+        for _ in range(3):
+            monarch_matrix_hip(q, k, None, T, B, False, variant=variant)
+        torch.cuda.synchronize()
+        steps = max(args.steps // 20, 5)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            monarch_matrix_hip(q, k, None, T, B, False, variant=variant)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        out_bytes = 4 * E * H * N * N
+        print(json.dumps({"metric": "ma_matrix_ms", "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": steps,
+                          "higher_is_better": False, "dtype": dt, "data": "synthetic",
+                          "config": {"workload": f"{args.config}: E{E} H{H} N{N} D{D} block {B} T={T}", "variant": variant},
+                          "output_bytes": out_bytes, "output_GBps": round(out_bytes / ms / 1e6, 1)}))
+        return
 
     if args.backward:
         from ma.ma_hip import monarch_attention_hip_backward

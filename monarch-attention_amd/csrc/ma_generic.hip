@@ -263,14 +263,33 @@ __global__ __launch_bounds__(kThreads) void matrix_kernel(Problem P, float* A, i
     }
     __syncthreads();
 
-    for (int ll = 0; ll < rows; ++ll) {
-        const int tq = (l0 + ll) * B + j - P.pad_off;
-        if (tq < 0 || tq >= P.N) continue;  // padded query rows are dropped
-        float* out = A + (eh * P.N + tq) * P.N;
-        const float* Ul = U + ll * M;
+    // A thread keeps its columns (four consecutive ones where rows of A allow 16-byte stores) and walks
+    // the query rows: one LDS read and one store per row and chunk.
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const bool vec = B % 4 == 0 && P.N % 4 == 0 && P.pad_off % 4 == 0;   // chunks stay inside a block and rows of A are aligned
+    if (vec) {
+        for (int idx = 4 * threadIdx.x; idx < M * B; idx += 4 * kThreads) {
+            const int tk = idx - P.pad_off;
+            if (tk < 0 || tk >= P.N) continue;
+            const f4 r4 = *reinterpret_cast<const f4*>(R + idx);
+            const int k = idx / B;
+            for (int ll = 0; ll < rows; ++ll) {
+                const int tq = (l0 + ll) * B + j - P.pad_off;
+                if (tq < 0 || tq >= P.N) continue;  // padded query rows are dropped
+                *reinterpret_cast<f4*>(A + (eh * P.N + tq) * P.N + tk) = U[ll * M + k] * r4;
+            }
+        }
+    } else {
         for (int idx = threadIdx.x; idx < M * B; idx += kThreads) {
             const int tk = idx - P.pad_off;
-            if (tk >= 0 && tk < P.N) out[tk] = Ul[idx / B] * R[idx];
+            if (tk < 0 || tk >= P.N) continue;
+            const float r = R[idx];
+            const int k = idx / B;
+            for (int ll = 0; ll < rows; ++ll) {
+                const int tq = (l0 + ll) * B + j - P.pad_off;
+                if (tq < 0 || tq >= P.N) continue;
+                A[(eh * P.N + tq) * P.N + tk] = U[ll * M + k] * r;
+            }
         }
     }
 }
