@@ -146,3 +146,19 @@ def test_backward_rejects_what_it_cannot_run():
             monarch_attention_hip_backward(q, k, v, None, w, 2, 16, False, variant=variant)
     with pytest.raises(ValueError):
         monarch_attention_hip_backward(q, k, v, None, w[:, :, :32], 2, 16, False)
+
+
+def test_backward_through_broadcast_keys_and_values():
+    """k and v shared by all heads (expanded views, stride 0): the forward reads them in place, the
+    gradient of the shared tensor is the sum over the heads."""
+    E, H, N, D, B, T = 2, 3, 64, 32, 16, 2
+    q, k1, v1 = seeded_qkv(E, H, N, D, torch.float32)
+    k1, v1 = k1[:1, :1].contiguous(), v1[:1, :1].contiguous()
+    w = torch.randn(E, H, N, D, generator=torch.Generator().manual_seed(3))
+    cpu = [t.clone().requires_grad_() for t in (q, k1, v1)]
+    out = monarch_attention_oracle(cpu[0], cpu[1].expand(E, H, N, D), cpu[2].expand(E, H, N, D), None, T, B, False)
+    (out * w).sum().backward()
+    dev = [t.to(DEV).requires_grad_() for t in (q, k1, v1)]
+    out = monarch_attention_hip(dev[0], dev[1].expand(E, H, N, D), dev[2].expand(E, H, N, D), None, T, B, False)
+    (out * w.to(DEV)).sum().backward()
+    assert_grads([t.grad for t in dev], [t.grad for t in cpu], "f32")
