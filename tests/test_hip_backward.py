@@ -162,3 +162,16 @@ def test_backward_through_broadcast_keys_and_values():
     out = monarch_attention_hip(dev[0], dev[1].expand(E, H, N, D), dev[2].expand(E, H, N, D), None, T, B, False)
     (out * w.to(DEV)).sum().backward()
     assert_grads([t.grad for t in dev], [t.grad for t in cpu], "f32")
+
+
+def test_backward_with_an_fp32_value_tensor_and_16_bit_queries():
+    """fp16 q / k with an fp32 v of another width (the dtype mix of get_matrix): the FMA backward kernels."""
+    E, H, N, D, Dv, B, T = 1, 2, 45, 16, 24, 8, 2
+    q, k, v = seeded_qkv(E, H, N, D, torch.float16, Dv=Dv)
+    v = v.float()
+    mask = block_safe_mask(E, N, B, seed=9)
+    w = torch.randn(E, H, N, Dv, generator=torch.Generator().manual_seed(4))
+    ref = oracle_grads(q, k, v, mask, w, T, B, True)
+    got = monarch_attention_hip_backward(*to_dev(q, k, v, mask, w), T, B, True)
+    assert got[0].dtype == torch.float16 and got[2].dtype == torch.float32
+    assert_grads(got, ref, "f16")
