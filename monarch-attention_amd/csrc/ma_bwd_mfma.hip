@@ -126,26 +126,45 @@ __device__ __forceinline__ void strip_each(const f32x4 (&acc)[4], int nt, int r0
         }
 }
 
-// *addr(row, col) = (accumulate ? *addr : 0) + value for every element of the strip whose addr is
-// not null.  All old values are loaded before the first store: the loads are in flight together
-// instead of one memory round trip per element.
-template <class F>
-__device__ __forceinline__ void strip_rmw(const f32x4 (&acc)[4], int nt, int r0, int c0, bool accumulate, F&& addr) {
+// base[row * row_stride + col] = (accumulate ? old : 0) + value for every element of the strip with
+// row < rows_valid and col < cols_valid.  All old values are loaded before the first store (the loads
+// are in flight together instead of one memory round trip per element), and only the strip's NT
+// tiles cost address arithmetic.
+template <int NT>
+__device__ __forceinline__ void strip_rmw_n(const f32x4 (&acc)[4], int r0, int c0, bool accumulate, float* base, long long row_stride,
+                                            int rows_valid, int cols_valid) {
     const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
-    float* p[16];
-    float old[16];
+    float* rowp[4];
+    bool rok[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int v = 0; v < 4; ++v) {
+        const int row = r0 + 4 * q + v;
+        rok[v] = row < rows_valid;
+        rowp[v] = base + row * row_stride + (c0 + r);
+    }
+    float old[NT][4];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            p[4 * t + v] = t < nt ? addr(r0 + 4 * q + v, c0 + 16 * t + r) : nullptr;
-            old[4 * t + v] = (accumulate && p[4 * t + v] != nullptr) ? *p[4 * t + v] : 0.f;
-        }
+    for (int t = 0; t < NT; ++t) {
+        const bool cok = c0 + 16 * t + r < cols_valid;
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+        for (int v = 0; v < 4; ++v) old[t][v] = (accumulate && rok[v] && cok) ? rowp[v][16 * t] : 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const bool cok = c0 + 16 * t + r < cols_valid;
 #pragma unroll
         for (int v = 0; v < 4; ++v)
-            if (p[4 * t + v] != nullptr) *p[4 * t + v] = old[4 * t + v] + acc[t][v];
+            if (rok[v] && cok) rowp[v][16 * t] = old[t][v] + acc[t][v];
+    }
+}
+__device__ __forceinline__ void strip_rmw(const f32x4 (&acc)[4], int nt, int r0, int c0, bool accumulate, float* base,
+                                          long long row_stride, int rows_valid, int cols_valid) {
+    switch (nt) {   // nt is the same for every lane of the wave
+        case 1: return strip_rmw_n<1>(acc, r0, c0, accumulate, base, row_stride, rows_valid, cols_valid);
+        case 2: return strip_rmw_n<2>(acc, r0, c0, accumulate, base, row_stride, rows_valid, cols_valid);
+        case 3: return strip_rmw_n<3>(acc, r0, c0, accumulate, base, row_stride, rows_valid, cols_valid);
+        default: return strip_rmw_n<4>(acc, r0, c0, accumulate, base, row_stride, rows_valid, cols_valid);
+    }
 }
 
 // Strips of a rows x cols output (both multiples of 16) dealt to the waves; body(r0, c0, nt).
@@ -423,8 +442,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma(acc, nt, U + r0, 1, ldm, dO + c0, ldo, 1, TL);
-                strip_rmw(acc, nt, r0, c0, l0 != 0,
-                          [&](int k, int d) -> float* { return (k < M && d < W) ? G.gY + (jm + k) * W + d : nullptr; });
+                strip_rmw(acc, nt, r0, c0, l0 != 0, G.gY + jm * W, W, M, W);
             });
         }
         // gaL (+)= dU^T Qt
@@ -432,8 +450,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma(acc, nt, Gg + r0, 1, ldm, Qt + c0, ldd, 1, TL);
-            strip_rmw(acc, nt, r0, c0, l0 != 0,
-                      [&](int k, int d) -> float* { return (k < M && d < D) ? G.gaL + (jm + k) * D + d : nullptr; });
+            strip_rmw(acc, nt, r0, c0, l0 != 0, G.gaL + jm * D, D, M, D);
         });
         for (int k = threadIdx.x; k < M; k += NTH) {   // gcL (+)= -sum_l dU
             float acc = l0 ? G.gcL[jm + k] : 0.f;
@@ -448,9 +465,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma(Problem P, BwdBuffers G, int 
             strip_mma(acc, nt, Gg + r0 * ldm, ldm, 1, aLt + c0, ldd, 1, M16);
             if (!kZ) strip_mma(acc, nt, U + r0 * ldm, ldm, 1, Wt + c0, ldw, 1, M16);
             // the Z stage runs first and every dq row belongs to one tile of one workgroup: it is written, not added to
-            strip_rmw(acc, nt, r0, c0, !kZ, [&](int ll, int d) -> float* {
-                return (l0 + ll < M && d < D) ? G.dq + (eh * M * B + (l0 + ll) * B + j) * D + d : nullptr;
-            });
+            strip_rmw(acc, nt, r0, c0, !kZ, G.dq + (eh * M * B + static_cast<long long>(l0) * B + j) * D, static_cast<long long>(B) * D,
+                      M - l0, D);
         });
         __syncthreads();
     }
@@ -607,10 +623,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma(acc, nt, Gg + r0 * ldb, ldb, 1, Kt + c0, ldd, 1, B16);
-            strip_rmw(acc, nt, r0, c0, first != 0, [&](int jj, int d) -> float* {
-                if (j0 + jj >= B || d >= D) return nullptr;
-                return (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0 + jj) * D + d;
-            });
+            strip_rmw(acc, nt, r0, c0, first != 0, (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0) * D, D, B - j0, D);
         });
         // dK += round(r)^T (sm gaL) + dDot^T X
         for_strips<NTH>(B16, D16, [&](int r0, int c0, int nt) {
@@ -618,20 +631,15 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma(Problem P, BwdBuffers G, int T
             zero_acc(acc);
             strip_mma(acc, nt, R + r0, 1, ldb, Ga + c0, lga, 1, TJ);
             strip_mma(acc, nt, Gg + r0, 1, ldb, X + c0, ldd, 1, TJ);
-            strip_rmw(acc, nt, r0, c0, !G.jt_split, [&](int i, int d) -> float* {
-                if (i >= B || d >= D) return nullptr;
-                return (G.jt_split ? G.pk + part * D : G.dk) + ((eh * M + k) * B + i) * D + d;
-            });
+            strip_rmw(acc, nt, r0, c0, !G.jt_split, (G.jt_split ? G.pk + part * D : G.dk) + (eh * M + k) * B * D, D, B, D);
         });
         if (with_v)   // dV += round(r)^T gY
             for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma(acc, nt, R + r0, 1, ldb, Gy + c0, lgy, 1, TJ);
-                strip_rmw(acc, nt, r0, c0, j0 != j_begin, [&](int i, int d) -> float* {   // dv has this one writer
-                    if (i >= B || d >= Dv) return nullptr;
-                    return (G.jt_split ? G.pv + part * Dv : G.dv) + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d;
-                });
+                strip_rmw(acc, nt, r0, c0, j0 != j_begin,   // dv has this one writer
+                          (G.jt_split ? G.pv + part * Dv : G.dv) + (eh * M + k) * B * static_cast<long long>(Dv), Dv, B, Dv);
             });
         __syncthreads();
     }
@@ -864,8 +872,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(U16) + r0, ldu, dO + c0, ldw, TL);
-                strip_rmw(acc, nt, r0, c0, l0 != 0,
-                          [&](int k, int d) -> float* { return (k < M && d < W) ? G.gY + (jm + k) * W + d : nullptr; });
+                strip_rmw(acc, nt, r0, c0, l0 != 0, G.gY + jm * W, W, M, W);
             });
         }
         // gaL (+)= dU^T Qt
@@ -873,8 +880,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma16<true, true>(acc, nt, G16 + r0, ldp, Qt + c0, ldd, TL);
-            strip_rmw(acc, nt, r0, c0, l0 != 0,
-                      [&](int k, int d) -> float* { return (k < M && d < D) ? G.gaL + (jm + k) * D + d : nullptr; });
+            strip_rmw(acc, nt, r0, c0, l0 != 0, G.gaL + jm * D, D, M, D);
         });
         for (int k = threadIdx.x; k < M; k += NTH) {   // gcL (+)= -sum_l dU
             float acc = l0 ? G.gcL[jm + k] : 0.f;
@@ -889,9 +895,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             strip_mma16<false, true>(acc, nt, G16 + r0 * ldp, ldp, aLt + c0, ldd, M16);
             if (!kZ) strip_mma16<false, true>(acc, nt, reinterpret_cast<const TQ*>(U16) + r0 * ldu, ldu, Wt + c0, ldw, M16);
             // the Z stage runs first and every dq row belongs to one tile of one workgroup: it is written, not added to
-            strip_rmw(acc, nt, r0, c0, !kZ, [&](int ll, int d) -> float* {
-                return (l0 + ll < M && d < D) ? G.dq + (eh * M * B + (l0 + ll) * B + j) * D + d : nullptr;
-            });
+            strip_rmw(acc, nt, r0, c0, !kZ, G.dq + (eh * M * B + static_cast<long long>(l0) * B + j) * D, static_cast<long long>(B) * D,
+                      M - l0, D);
         });
         __syncthreads();
     }
@@ -1064,10 +1069,7 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma16<false, true>(acc, nt, reinterpret_cast<const TQ*>(Dd) + r0 * ldp, ldp, Kt + c0, ldd, B16);
-            strip_rmw(acc, nt, r0, c0, first != 0, [&](int jj, int d) -> float* {
-                if (j0 + jj >= B || d >= D) return nullptr;
-                return (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0 + jj) * D + d;
-            });
+            strip_rmw(acc, nt, r0, c0, first != 0, (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0) * D, D, B - j0, D);
         });
         // dK += round(r)^T (sm gaL) + dDot^T X
         for_strips<NTH>(B16, D16, [&](int r0, int c0, int nt) {
@@ -1075,20 +1077,15 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             zero_acc(acc);
             strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(R16) + r0, ldp, Ga + c0, ldd, TJ);
             strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(Dd) + r0, ldp, X + c0, ldd, TJ);
-            strip_rmw(acc, nt, r0, c0, !G.jt_split, [&](int i, int d) -> float* {
-                if (i >= B || d >= D) return nullptr;
-                return (G.jt_split ? G.pk + part * D : G.dk) + ((eh * M + k) * B + i) * D + d;
-            });
+            strip_rmw(acc, nt, r0, c0, !G.jt_split, (G.jt_split ? G.pk + part * D : G.dk) + (eh * M + k) * B * D, D, B, D);
         });
         if (with_v)   // dV += round(r)^T gY
             for_strips<NTH>(B16, V16, [&](int r0, int c0, int nt) {
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(R16) + r0, ldp, Gy + c0, ldv, TJ);
-                strip_rmw(acc, nt, r0, c0, j0 != j_begin, [&](int i, int d) -> float* {   // dv has this one writer
-                    if (i >= B || d >= Dv) return nullptr;
-                    return (G.jt_split ? G.pv + part * Dv : G.dv) + ((eh * M + k) * B + i) * static_cast<long long>(Dv) + d;
-                });
+                strip_rmw(acc, nt, r0, c0, j0 != j_begin,   // dv has this one writer
+                          (G.jt_split ? G.pv + part * Dv : G.dv) + (eh * M + k) * B * static_cast<long long>(Dv), Dv, B, Dv);
             });
         __syncthreads();
     }
