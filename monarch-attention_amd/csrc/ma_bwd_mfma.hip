@@ -79,6 +79,23 @@ __device__ __forceinline__ float seg_sum(float x) {
 // whole wave for rows of more than 32 entries (measured: there the one-row-per-wave walk, with its
 // conflict-free LDS accesses, is the faster one)
 inline int group_lanes(int n) { return n <= 16 ? 4 : n <= 32 ? 8 : 64; }
+// f(std::integral_constant<int, E>) with E = entries of a row of n per lane of a group of G lanes, for the
+// rows that a lane can keep in registers (at most four entries); false if the row is longer
+template <int G, class F>
+__device__ __forceinline__ bool with_entries(int n, F&& f) {
+    if (n > 4 * G) return false;
+    if (G < 64) {   // groups of 4 / 8 lanes are only used for rows of 16 / 32: four entries
+        f(std::integral_constant<int, 4>{});
+        return true;
+    }
+    switch ((n + G - 1) / G) {
+        case 1: f(std::integral_constant<int, 1>{}); break;
+        case 2: f(std::integral_constant<int, 2>{}); break;
+        case 3: f(std::integral_constant<int, 3>{}); break;
+        default: f(std::integral_constant<int, 4>{}); break;
+    }
+    return true;
+}
 
 // acc[t] += sum_k A(r,k) B(k, 16 t + c) for one 16-row strip of up to four 16-column tiles.
 // A(r,k) = A[r*ars + k*acs], B(k,c) = B[k*brs + c*bcs]; K is a multiple of 16.  Lane (r = lane % 16,
@@ -839,6 +856,50 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
         {
             constexpr int RPP = 64 / GL;
             const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane / GL, cg = lane % GL;
+            // rows of up to four entries per lane stay in registers between the reductions
+            const bool in_regs = with_entries<GL>(M16, [&](auto etag) {
+                constexpr int EPL = decltype(etag)::value;
+                for (int l1 = wave * RPP; l1 < TL; l1 += (NTH / 64) * RPP) {
+                    const int ll = l1 + sub;
+                    float* Ul = U + ll * ldm;
+                    float* Gl = Gg + ll * ldm;
+                    float u[EPL], g[EPL];
+                    float mx = -INFINITY;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        const int k = cg + GL * e;
+                        u[e] = k < M16 ? Ul[k] : -INFINITY;
+                        g[e] = k < M16 ? Gl[k] : 0.f;
+                        mx = fmaxf(mx, u[e]);
+                    }
+                    mx = seg_max<GL>(mx);
+                    float sum = 0.f;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        u[e] = __expf(u[e] - mx);
+                        sum += u[e];
+                    }
+                    const float inv = mfma::rcp(seg_sum<GL>(sum));
+                    float dot = 0.f;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        u[e] *= inv;
+                        dot = fmaf(g[e], u[e], dot);
+                    }
+                    dot = seg_sum<GL>(dot);
+                    const float keep = kZ ? 1.f : qok[ll];
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        const int k = cg + GL * e;
+                        if (k >= M16) continue;
+                        const float du = u[e] * (g[e] - dot);
+                        Gl[k] = du;
+                        G16[ll * ldp + k] = from_f<TQ>(du);
+                        U16[ll * ldu + k] = from_f<TQ>(keep * u[e]);   // over fp32 entries this row's lanes have read
+                    }
+                }
+            });
+            if (!in_regs)
             for (int l1 = wave * RPP; l1 < TL; l1 += (NTH / 64) * RPP) {
                 const int ll = l1 + sub;
                 float* Ul = U + ll * ldm;
@@ -1023,6 +1084,59 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
         {
             constexpr int RPP = 64 / GL;
             const int sub = lane / GL, cg = lane % GL;
+            // rows of up to four entries per lane stay in registers between the reductions
+            const bool in_regs = with_entries<GL>(B16, [&](auto etag) {
+                constexpr int EPL = decltype(etag)::value;
+                for (int j1 = wave * RPP; j1 < TJ; j1 += (NTH / 64) * RPP) {
+                    const int jj = j1 + sub;
+                    const float* Sj = S + jj * ldb;
+                    const float* Gj = Gg + jj * ldb;
+                    float sv[EPL], g[EPL], r[EPL];
+                    // probabilities (ma_torch.py:14-18)
+                    float mx = -INFINITY;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        const int i = cg + GL * e;
+                        sv[e] = i < B16 ? Sj[i] : -INFINITY;
+                        g[e] = i < B16 ? Gj[i] : 0.f;
+                        mx = fmaxf(mx, sv[e]);
+                    }
+                    mx = fmaxf(seg_max<GL>(mx), P.eps);
+                    float sum = 0.f;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        r[e] = __expf(sv[e] - mx);
+                        sum += r[e];
+                    }
+                    const float inv = mfma::rcp(seg_sum<GL>(sum) + P.eps);
+                    // g = gcL (log r + 1) + sm gaL K^T + gY V^T where the clamp did not act, else 0
+                    float dot = 0.f;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        const int i = cg + GL * e;
+                        const float ru = r[e] * inv;
+                        r[e] = i < B ? fmaxf(ru, kTiny) : 0.f;
+                        g[e] = (i < B && ru >= kTiny) ? fmaf(gcl[jj], __logf(r[e]) + 1.0f, g[e]) : 0.f;
+                        dot = fmaf(g[e], r[e], dot);
+                    }
+                    dot = seg_sum<GL>(dot);
+                    // dS, gcR; D16 <- dDot = dS sm / (cR + eps); R16 <- round(r)
+                    float gc = 0.f;
+                    const float cj = c[jj];
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        const int i = cg + GL * e;
+                        if (i >= B16) continue;
+                        const float ds = sv[e] == -INFINITY ? 0.f : r[e] * (g[e] - dot);
+                        if (sv[e] != -INFINITY) gc = fmaf(-ds, sv[e] * cj, gc);
+                        Dd[jj * ldp + i] = from_f<TQ>(ds * sm * cj);   // both over fp32 entries this row's lanes have read
+                        R16[jj * ldp + i] = from_f<TQ>(r[e]);
+                    }
+                    gc = seg_sum<GL>(gc);
+                    if (!first && cg == 0 && j0 + jj < B) G.gcR[(eh * M + k) * B + j0 + jj] = gc;
+                }
+            });
+            if (!in_regs)
             for (int j1 = wave * RPP; j1 < TJ; j1 += (NTH / 64) * RPP) {
                 const int jj = j1 + sub;
                 float* Sj = S + jj * ldb;
