@@ -240,6 +240,9 @@ __device__ __forceinline__ void stage_rows(TD* dst, int ld, int rows, int width,
                 if constexpr (sizeof(TD) == 4) {
                     *reinterpret_cast<f32x4*>(dst + i * ld + 4 * c) = f32x4{scale * to_f(x[u].v[0]), scale * to_f(x[u].v[1]),
                                                                            scale * to_f(x[u].v[2]), scale * to_f(x[u].v[3])};
+                } else if constexpr (std::is_same<T, TD>::value) {   // copied as they are (scale is 1 for these tiles)
+                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c) = Pair{x[u].v[0], x[u].v[1]};
+                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c + 2) = Pair{x[u].v[2], x[u].v[3]};
                 } else {   // 16-bit rows start on 4-byte boundaries only
                     *reinterpret_cast<Pair*>(dst + i * ld + 4 * c) =
                         Pair{from_f<TD>(scale * to_f(x[u].v[0])), from_f<TD>(scale * to_f(x[u].v[1]))};
@@ -290,6 +293,9 @@ struct TileSpec {
             if constexpr (sizeof(TD) == 4) {
                 *reinterpret_cast<f32x4*>(d) = f32x4{scale * to_f(x[u].v[0]), scale * to_f(x[u].v[1]), scale * to_f(x[u].v[2]),
                                                      scale * to_f(x[u].v[3])};
+            } else if constexpr (std::is_same<T, TD>::value) {   // copied as they are (scale is 1 for these tiles)
+                *reinterpret_cast<Pair*>(d) = Pair{x[u].v[0], x[u].v[1]};
+                *reinterpret_cast<Pair*>(d + 2) = Pair{x[u].v[2], x[u].v[3]};
             } else {
                 *reinterpret_cast<Pair*>(d) = Pair{from_f<TD>(scale * to_f(x[u].v[0])), from_f<TD>(scale * to_f(x[u].v[1]))};
                 *reinterpret_cast<Pair*>(d + 2) = Pair{from_f<TD>(scale * to_f(x[u].v[2])), from_f<TD>(scale * to_f(x[u].v[3]))};
