@@ -192,8 +192,12 @@ __device__ __forceinline__ void for_strips(int rows, int cols, F&& body) {
     const int tiles = (rows / 16) * (cols / 16);
     const int wt = tiles >= 4 * (NTH / 64) ? 4 : tiles >= 2 * (NTH / 64) ? 2 : 1;
     const int cg = (cols / 16 + wt - 1) / wt, total = (rows / 16) * cg;
+    // (row tile, column group) of strip s; a power-of-two group count (the usual case) needs no division
+    const bool pow2 = (cg & (cg - 1)) == 0;
+    const int shift = __builtin_ctz(cg);
     for (int s = wave; s < total; s += NTH / 64) {
-        const int rt = s / cg, g = s % cg;
+        const int rt = pow2 ? s >> shift : s / cg;
+        const int g = pow2 ? s & (cg - 1) : s - rt * cg;
         body(16 * rt, 16 * wt * g, min(wt, cols / 16 - wt * g));
     }
 }
