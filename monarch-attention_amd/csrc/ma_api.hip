@@ -540,6 +540,7 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
     G.pk = L.parts ? reinterpret_cast<float*>(ws + L.pk) : nullptr;
     G.pv = L.parts ? reinterpret_cast<float*>(ws + L.pv) : nullptr;
     G.jt_split = 0;
+    G.state16 = (!fma_only && bwd_state16_ok(P, pp.dtype_qk, pp.dtype_v)) ? 1 : 0;
     G.dout = static_cast<const char*>(b->dout);
     for (int i = 0; i < 3; ++i) G.dos[i] = b->dout_stride[i];
     const long long rows = static_cast<long long>(P.E) * P.H * P.M * P.B;

@@ -184,6 +184,23 @@ __device__ __forceinline__ void strip_rmw(const f32x4 (&acc)[4], int nt, int r0,
     }
 }
 
+// base[row * row_stride + col] = value rounded to T, for the elements of the strip inside the valid range
+template <class T>
+__device__ __forceinline__ void strip_store16(const f32x4 (&acc)[4], int nt, int r0, int c0, T* base, long long row_stride,
+                                              int rows_valid, int cols_valid) {
+    const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (t >= nt) break;
+        const int col = c0 + 16 * t + r;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int row = r0 + 4 * q + v;
+            if (row < rows_valid && col < cols_valid) base[row * row_stride + col] = from_f<T>(acc[t][v]);
+        }
+    }
+}
+
 // Strips of a rows x cols output (both multiples of 16) dealt to the waves; body(r0, c0, nt).
 // A strip is as wide as lets every wave have one (1, 2 or 4 tiles).
 template <int NTH, class F>
@@ -244,9 +261,9 @@ __device__ __forceinline__ void stage_rows(TD* dst, int ld, int rows, int width,
                 if constexpr (sizeof(TD) == 4) {
                     *reinterpret_cast<f32x4*>(dst + i * ld + 4 * c) = f32x4{scale * to_f(x[u].v[0]), scale * to_f(x[u].v[1]),
                                                                            scale * to_f(x[u].v[2]), scale * to_f(x[u].v[3])};
-                } else if constexpr (std::is_same<T, TD>::value) {   // copied as they are (scale is 1 for these tiles)
-                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c) = Pair{x[u].v[0], x[u].v[1]};
-                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c + 2) = Pair{x[u].v[2], x[u].v[3]};
+                } else if (std::is_same<T, TD>::value && scale == 1.f) {   // copied as they are
+                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c) = Pair{from_f<TD>(to_f(x[u].v[0])), from_f<TD>(to_f(x[u].v[1]))};
+                    *reinterpret_cast<Pair*>(dst + i * ld + 4 * c + 2) = Pair{from_f<TD>(to_f(x[u].v[2])), from_f<TD>(to_f(x[u].v[3]))};
                 } else {   // 16-bit rows start on 4-byte boundaries only
                     *reinterpret_cast<Pair*>(dst + i * ld + 4 * c) =
                         Pair{from_f<TD>(scale * to_f(x[u].v[0])), from_f<TD>(scale * to_f(x[u].v[1]))};
@@ -297,9 +314,9 @@ struct TileSpec {
             if constexpr (sizeof(TD) == 4) {
                 *reinterpret_cast<f32x4*>(d) = f32x4{scale * to_f(x[u].v[0]), scale * to_f(x[u].v[1]), scale * to_f(x[u].v[2]),
                                                      scale * to_f(x[u].v[3])};
-            } else if constexpr (std::is_same<T, TD>::value) {   // copied as they are (scale is 1 for these tiles)
-                *reinterpret_cast<Pair*>(d) = Pair{x[u].v[0], x[u].v[1]};
-                *reinterpret_cast<Pair*>(d + 2) = Pair{x[u].v[2], x[u].v[3]};
+            } else if (std::is_same<T, TD>::value && scale == 1.f) {   // copied as they are
+                *reinterpret_cast<Pair*>(d) = Pair{from_f<TD>(to_f(x[u].v[0])), from_f<TD>(to_f(x[u].v[1]))};
+                *reinterpret_cast<Pair*>(d + 2) = Pair{from_f<TD>(to_f(x[u].v[2])), from_f<TD>(to_f(x[u].v[3]))};
             } else {
                 *reinterpret_cast<Pair*>(d) = Pair{from_f<TD>(scale * to_f(x[u].v[0])), from_f<TD>(scale * to_f(x[u].v[1]))};
                 *reinterpret_cast<Pair*>(d + 2) = Pair{from_f<TD>(scale * to_f(x[u].v[2])), from_f<TD>(scale * to_f(x[u].v[3]))};
@@ -778,8 +795,12 @@ __host__ __device__ inline LzLayout16 lz_layout16(int M, int D, int W, bool z, i
     return L;
 }
 
-template <class TQ, bool kZ, int NTH, int GL>
+// S16: the state gradients gaL, gY, gaR are kept in the operand dtype instead of fp32 (the host sets it
+// when every stage runs these kernels and no state gradient is accumulated over several tiles: the
+// values are rounded to the operand dtype on their way into the next stage's LDS either way)
+template <class TQ, bool kZ, int NTH, int GL, bool S16>
 __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, int TL) {
+    using TG = typename std::conditional<S16, TQ, float>::type;
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];
     const int M = P.M, D = P.D, B = P.B, W = kZ ? P.Dv : P.D;
     const int M16 = up(M, 16), D16 = up(D, 16), W16 = up(W, 16);
@@ -808,12 +829,13 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
     const TQ* Y = reinterpret_cast<const TQ*>(P.Y) + jm * W;
     auto aL_row = [=](int k) { return k < M ? aL + k * D : nullptr; };
     auto y_row = [=](int k) { return k < M ? Y + k * static_cast<long long>(W) : nullptr; };
-    auto gar_row = [=](int k) { return k < M ? G.gaR + ((eh * M + k) * B + j) * D : nullptr; };
+    const TG* gaR = reinterpret_cast<const TG*>(G.gaR);
+    auto gar_row = [=](int k) { return k < M ? gaR + ((eh * M + k) * B + j) * D : nullptr; };
     constexpr bool kJoint = NTH == 64;   // single-wave workgroups stage all their tiles in one go
     if (!kJoint) {
         stage_rows<NTH, TQ, TQ>(aLt, ldd, M16, D16, D, 1.f, aL_row);
         if (kZ) stage_rows<NTH, TQ, TQ>(Wt, ldw, M16, W16, W, 1.f, y_row);
-        else stage_rows<NTH, float, TQ>(Wt, ldw, M16, W16, W, 1.f, gar_row);
+        else stage_rows<NTH, TG, TQ>(Wt, ldw, M16, W16, W, 1.f, gar_row);
     }
     for (int k = threadIdx.x; k < M16; k += NTH) {
         cl[k] = k < M ? P.cL[jm + k] : 0.f;
@@ -834,7 +856,7 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
                                  tile_of<TQ>(Qt, ldd, TL, D16, D, 1.f, q_row), tile_of<TQ>(dO, ldw, TL, W16, W, 1.f, do_row));
             else
                 stage_tiles<NTH>(tile_of<TQ>(aLt, ldd, state_rows, D16, D, 1.f, aL_row),
-                                 tile_of<float>(Wt, ldw, state_rows, W16, W, 1.f, gar_row), tile_of<TQ>(Qt, ldd, TL, D16, D, 1.f, q_row));
+                                 tile_of<TG>(Wt, ldw, state_rows, W16, W, 1.f, gar_row), tile_of<TQ>(Qt, ldd, TL, D16, D, 1.f, q_row));
         } else {
             stage_rows<NTH, TQ, TQ>(Qt, ldd, TL, D16, D, 1.f, q_row);
             if (kZ) stage_rows<NTH, TQ, TQ>(dO, ldw, TL, W16, W, 1.f, do_row);
@@ -943,7 +965,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
                 f32x4 acc[4];
                 zero_acc(acc);
                 strip_mma16<true, true>(acc, nt, reinterpret_cast<const TQ*>(U16) + r0, ldu, dO + c0, ldw, TL);
-                strip_rmw(acc, nt, r0, c0, l0 != 0, G.gY + jm * W, W, M, W);
+                if (S16) strip_store16(acc, nt, r0, c0, reinterpret_cast<TQ*>(G.gY) + jm * W, W, M, W);
+                else strip_rmw(acc, nt, r0, c0, l0 != 0, G.gY + jm * W, W, M, W);
             });
         }
         // gaL (+)= dU^T Qt
@@ -951,7 +974,8 @@ __global__ __launch_bounds__(NTH) void lz_bwd_mfma16(Problem P, BwdBuffers G, in
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma16<true, true>(acc, nt, G16 + r0, ldp, Qt + c0, ldd, TL);
-            strip_rmw(acc, nt, r0, c0, l0 != 0, G.gaL + jm * D, D, M, D);
+            if (S16) strip_store16(acc, nt, r0, c0, reinterpret_cast<TQ*>(G.gaL) + jm * D, D, M, D);
+            else strip_rmw(acc, nt, r0, c0, l0 != 0, G.gaL + jm * D, D, M, D);
         });
         for (int k = threadIdx.x; k < M; k += NTH) {   // gcL (+)= -sum_l dU
             float acc = l0 ? G.gcL[jm + k] : 0.f;
@@ -1003,8 +1027,9 @@ __host__ __device__ inline RLayout16 r_layout16(int B, int D, int Dv, bool with_
     return L;
 }
 
-template <class TQ, int NTH, int GL>
+template <class TQ, int NTH, int GL, bool S16>
 __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int TJ, int first, int with_v) {
+    using TG = typename std::conditional<S16, TQ, float>::type;
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];
     const int B = P.B, M = P.M, D = P.D, Dv = P.Dv;
     const int B16 = up(B, 16), D16 = up(D, 16), V16 = up(Dv, 16);
@@ -1053,19 +1078,21 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             if (j0 + jj >= B) return nullptr;
             return first ? tok_row<TQ>(P.q, P.qs, e, h, k * B + j0 + jj - P.pad_off, P.N) : aR + (j0 + jj) * D;
         };
-        auto ga_row = [=](int jj) { return j0 + jj < B ? G.gaL + ((eh * B + j0 + jj) * M + k) * D : nullptr; };
+        const TG* gaL = reinterpret_cast<const TG*>(G.gaL);
+        const TG* gY = reinterpret_cast<const TG*>(G.gY);
+        auto ga_row = [=](int jj) { return j0 + jj < B ? gaL + ((eh * B + j0 + jj) * M + k) * D : nullptr; };
         auto gy_row = [=](int jj) {
-            return j0 + jj < B ? G.gY + ((eh * B + j0 + jj) * M + k) * static_cast<long long>(Dv) : nullptr;
+            return j0 + jj < B ? gY + ((eh * B + j0 + jj) * M + k) * static_cast<long long>(Dv) : nullptr;
         };
         if (kJoint) {   // the key / value tiles of the block travel with the first tile of query rows
             const int kv_rows = j0 == j_begin ? B16 : 0;
             stage_tiles<NTH>(tile_of<TQ>(Kt, ldd, kv_rows, D16, D, 1.f, k_row),
                              tile_of<TQ>(Vt, ldv, with_v ? kv_rows : 0, V16, Dv, 1.f, v_row), tile_of<TQ>(X, ldd, TJ, D16, D, 1.f, x_row),
-                             tile_of<float>(Ga, ldd, TJ, D16, D, sm, ga_row), tile_of<float>(Gy, ldv, with_v ? TJ : 0, V16, Dv, 1.f, gy_row));
+                             tile_of<TG>(Ga, ldd, TJ, D16, D, sm, ga_row), tile_of<TG>(Gy, ldv, with_v ? TJ : 0, V16, Dv, 1.f, gy_row));
         } else {
             stage_rows<NTH, TQ, TQ>(X, ldd, TJ, D16, D, 1.f, x_row);
-            stage_rows<NTH, float, TQ>(Ga, ldd, TJ, D16, D, sm, ga_row);
-            if (with_v) stage_rows<NTH, float, TQ>(Gy, ldv, TJ, V16, Dv, 1.f, gy_row);
+            stage_rows<NTH, TG, TQ>(Ga, ldd, TJ, D16, D, sm, ga_row);
+            if (with_v) stage_rows<NTH, TG, TQ>(Gy, ldv, TJ, V16, Dv, 1.f, gy_row);
         }
         for (int jj = threadIdx.x; jj < TJ; jj += NTH) {
             const bool in = j0 + jj < B;
@@ -1193,7 +1220,8 @@ __global__ __launch_bounds__(NTH) void r_bwd_mfma16(Problem P, BwdBuffers G, int
             f32x4 acc[4];
             zero_acc(acc);
             strip_mma16<false, true>(acc, nt, reinterpret_cast<const TQ*>(Dd) + r0 * ldp, ldp, Kt + c0, ldd, B16);
-            strip_rmw(acc, nt, r0, c0, first != 0, (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0) * D, D, B - j0, D);
+            if (S16 && !first) strip_store16(acc, nt, r0, c0, reinterpret_cast<TQ*>(G.gaR) + ((eh * M + k) * B + j0) * D, D, B - j0, D);
+            else strip_rmw(acc, nt, r0, c0, first != 0, (first ? G.dq : G.gaR) + ((eh * M + k) * B + j0) * D, D, B - j0, D);
         });
         // dK += round(r)^T (sm gaL) + dDot^T X
         for_strips<NTH>(B16, D16, [&](int r0, int c0, int nt) {
@@ -1265,12 +1293,16 @@ int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z,
         } else {
             // lanes per probability row: short rows go with the small workgroups
             const int gl = group_lanes(up(P.M, 16));
-            if (nth == 64 && gl == 4) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 4>) : launch(lz_bwd_mfma16<TQ, false, 64, 4>);
-            if (nth == 64 && gl == 8) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 8>) : launch(lz_bwd_mfma16<TQ, false, 64, 8>);
-            if (nth == 64) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 64>) : launch(lz_bwd_mfma16<TQ, false, 64, 64>);
-            if (nth == 256 && gl == 8) return z ? launch(lz_bwd_mfma16<TQ, true, 256, 8>) : launch(lz_bwd_mfma16<TQ, false, 256, 8>);
-            if (nth == 256) return z ? launch(lz_bwd_mfma16<TQ, true, 256, 64>) : launch(lz_bwd_mfma16<TQ, false, 256, 64>);
-            return z ? launch(lz_bwd_mfma16<TQ, true, 1024, 64>) : launch(lz_bwd_mfma16<TQ, false, 1024, 64>);
+            auto pick = [&](auto s16) {
+                constexpr bool S = decltype(s16)::value;
+                if (nth == 64 && gl == 4) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 4, S>) : launch(lz_bwd_mfma16<TQ, false, 64, 4, S>);
+                if (nth == 64 && gl == 8) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 8, S>) : launch(lz_bwd_mfma16<TQ, false, 64, 8, S>);
+                if (nth == 64) return z ? launch(lz_bwd_mfma16<TQ, true, 64, 64, S>) : launch(lz_bwd_mfma16<TQ, false, 64, 64, S>);
+                if (nth == 256 && gl == 8) return z ? launch(lz_bwd_mfma16<TQ, true, 256, 8, S>) : launch(lz_bwd_mfma16<TQ, false, 256, 8, S>);
+                if (nth == 256) return z ? launch(lz_bwd_mfma16<TQ, true, 256, 64, S>) : launch(lz_bwd_mfma16<TQ, false, 256, 64, S>);
+                return z ? launch(lz_bwd_mfma16<TQ, true, 1024, 64, S>) : launch(lz_bwd_mfma16<TQ, false, 1024, 64, S>);
+            };
+            return G.state16 ? pick(std::true_type{}) : pick(std::false_type{});
         }
     });
 }
@@ -1281,6 +1313,16 @@ static int r_tile(const Problem& P, int dt_qk, bool with_v) {
         return dt_qk == MA_F32 ? r_layout<float>(P.B, P.D, P.Dv, with_v, t).total : r_layout16(P.B, P.D, P.Dv, with_v, t).total;
     };
     return pick_tile(P.B, bytes);
+}
+
+// Whether a backward pass of this problem can keep its state gradients in the operand dtype: fp16 /
+// bf16 operands of one dtype, every stage within the 16-bit matrix-core kernels' LDS, and the L / Z
+// stages in a single tile of query blocks (gaL and gY are then written once, not accumulated).
+bool bwd_state16_ok(const Problem& P, int dt_qk, int dt_v) {
+    if (dt_qk == MA_F32 || dt_qk != dt_v) return false;
+    const int M16 = up(P.M, 16);
+    if (lz_layout16(P.M, P.D, P.Dv, true, M16).total > kLdsBudget || lz_layout16(P.M, P.D, P.D, false, M16).total > kLdsBudget) return false;
+    return r_tile(P, dt_qk, true) > 0;
 }
 
 // Number of per-tile partial buffers the R stage wants for dk / dv (0: none).  Splitting a block's
@@ -1328,12 +1370,16 @@ int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G0, int dt_qk, bool fi
             else st = launch(r_bwd_mfma<TQ, 1024>);
         } else {
             const int gl = group_lanes(up(P.B, 16));
-            if (nth == 64 && gl == 4) st = launch(r_bwd_mfma16<TQ, 64, 4>);
-            else if (nth == 64 && gl == 8) st = launch(r_bwd_mfma16<TQ, 64, 8>);
-            else if (nth == 64) st = launch(r_bwd_mfma16<TQ, 64, 64>);
-            else if (nth == 256 && gl == 8) st = launch(r_bwd_mfma16<TQ, 256, 8>);
-            else if (nth == 256) st = launch(r_bwd_mfma16<TQ, 256, 64>);
-            else st = launch(r_bwd_mfma16<TQ, 1024, 64>);
+            auto pick = [&](auto s16) {
+                constexpr bool S = decltype(s16)::value;
+                if (nth == 64 && gl == 4) return launch(r_bwd_mfma16<TQ, 64, 4, S>);
+                if (nth == 64 && gl == 8) return launch(r_bwd_mfma16<TQ, 64, 8, S>);
+                if (nth == 64) return launch(r_bwd_mfma16<TQ, 64, 64, S>);
+                if (nth == 256 && gl == 8) return launch(r_bwd_mfma16<TQ, 256, 8, S>);
+                if (nth == 256) return launch(r_bwd_mfma16<TQ, 256, 64, S>);
+                return launch(r_bwd_mfma16<TQ, 1024, 64, S>);
+            };
+            st = G.state16 ? pick(std::true_type{}) : pick(std::false_type{});
         }
         if (st || !G.jt_split) return st;
         const long long rows = static_cast<long long>(P.E) * P.H * P.M * P.B;

@@ -72,7 +72,9 @@ struct BwdBuffers {
     float* pk;     // (parts,E,H,Np,D) / (parts,E,H,Np,Dv): per-tile parts of dk / dv of an R stage whose
     float* pv;     //   tiles of query rows run in different workgroups; nullptr: never split
     int jt_split;  // set by the launcher: workgroups per block (0 = one workgroup walks all tiles)
+    int state16;   // gaL, gY, gaR hold the operand dtype instead of fp32 (see bwd_state16_ok)
 };
+bool bwd_state16_ok(const Problem& P, int dt_qk, int dt_v);
 // partial buffers the R stage wants for this problem (0: it does not split blocks over workgroups)
 int bwd_r_split_tiles(const Problem& P, int dt_qk, int dt_v);
 bool bwd_fits(const Problem& P);
