@@ -560,13 +560,15 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
             if (st) return st;
         }
     }
-    long long qs[3], ks[3], vs[3];
-    for (int i = 0; i < 3; ++i) { qs[i] = b->dq_stride[i]; ks[i] = b->dk_stride[i]; vs[i] = b->dv_stride[i]; }
-    st = launch_bwd_out(G.dq, b->dq, qs, pp.dtype_qk, P, P.D, s);
-    if (st) return st;
-    st = launch_bwd_out(G.dk, b->dk, ks, pp.dtype_qk, P, P.D, s);
-    if (st) return st;
-    return launch_bwd_out(G.dv, b->dv, vs, pp.dtype_v, P, P.Dv, s);
+    // fp32 accumulators -> the caller's tensors: one launch when dv has the shape and dtype of dq / dk
+    long long st3[3][3];
+    for (int i = 0; i < 3; ++i) { st3[0][i] = b->dq_stride[i]; st3[1][i] = b->dk_stride[i]; st3[2][i] = b->dv_stride[i]; }
+    const float* src[3] = {G.dq, G.dk, G.dv};
+    void* dst[3] = {b->dq, b->dk, b->dv};
+    const bool same = pp.Dv == pp.D && pp.dtype_v == pp.dtype_qk;
+    st = launch_bwd_out(same ? 3 : 2, src, dst, st3, pp.dtype_qk, P, P.D, s);
+    if (st || same) return st;
+    return launch_bwd_out(1, src + 2, dst + 2, st3 + 2, pp.dtype_v, P, P.Dv, s);
 }
 
 }  // extern "C"

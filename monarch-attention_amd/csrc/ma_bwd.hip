@@ -314,11 +314,19 @@ __global__ void fill_zero_kernel(float* p, long long n) {
         p[i] = 0.f;
 }
 
-// real rows of a padded fp32 gradient (E,H,Np,W) -> the caller's tensor (dtype T, its strides).
+// real rows of padded fp32 gradients (E,H,Np,W) -> the caller's tensors (dtype T, their strides); up to three
+// tensors of one width and dtype per launch (blockIdx.y selects).
 // VEC = 4: four consecutive columns per thread (W % 4 == 0, rows of dst aligned to four elements).
+struct GradOut {
+    const float* src[3];
+    char* dst[3];
+    long long st[3][3];
+};
 template <class T, int VEC>
-__global__ void grad_out_kernel(const float* src, char* dst, long long s0, long long s1, long long s2, int E, int H, int N, int Np,
-                                int W, int pad_off) {
+__global__ void grad_out_kernel(GradOut g, int E, int H, int N, int Np, int W, int pad_off) {
+    const float* src = g.src[blockIdx.y];
+    char* dst = g.dst[blockIdx.y];
+    const long long s0 = g.st[blockIdx.y][0], s1 = g.st[blockIdx.y][1], s2 = g.st[blockIdx.y][2];
     const int WV = W / VEC;
     const long long total = static_cast<long long>(E) * H * N * WV;
     for (long long i = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x; i < total;
@@ -403,18 +411,27 @@ int launch_bwd_r(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, boo
     });
 }
 
-int launch_bwd_out(const float* src, void* dst, const long long* st, int dt, const Problem& P, int W, hipStream_t s) {
+// n (1..3) gradients of width W and dtype dt in one launch
+int launch_bwd_out(int n, const float* const* src, void* const* dst, const long long (*st)[3], int dt, const Problem& P, int W,
+                   hipStream_t s) {
     return dispatch_qk(dt, [&](auto t) {
         using T = decltype(t);
-        const bool vec = W % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % (4 * sizeof(T)) == 0 && st[0] % 4 == 0 && st[1] % 4 == 0 &&
-                         st[2] % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0;
+        GradOut g;
+        bool vec = W % 4 == 0;
+        for (int i = 0; i < 3; ++i) {
+            const int j = i < n ? i : 0;
+            g.src[i] = src[j];
+            g.dst[i] = static_cast<char*>(dst[j]);
+            for (int a = 0; a < 3; ++a) g.st[i][a] = st[j][a];
+            vec = vec && reinterpret_cast<uintptr_t>(dst[j]) % (4 * sizeof(T)) == 0 && st[j][0] % 4 == 0 && st[j][1] % 4 == 0 &&
+                  st[j][2] % 4 == 0 && reinterpret_cast<uintptr_t>(src[j]) % 16 == 0;
+        }
         const long long total = static_cast<long long>(P.E) * P.H * P.N * (vec ? W / 4 : W);
+        const dim3 grid(blocks_for(total), n);
         if (vec)
-            hipLaunchKernelGGL((grad_out_kernel<T, 4>), dim3(blocks_for(total)), dim3(256), 0, s, src, static_cast<char*>(dst), st[0],
-                               st[1], st[2], P.E, P.H, P.N, P.M * P.B, W, P.pad_off);
+            hipLaunchKernelGGL((grad_out_kernel<T, 4>), grid, dim3(256), 0, s, g, P.E, P.H, P.N, P.M * P.B, W, P.pad_off);
         else
-            hipLaunchKernelGGL((grad_out_kernel<T, 1>), dim3(blocks_for(total)), dim3(256), 0, s, src, static_cast<char*>(dst), st[0],
-                               st[1], st[2], P.E, P.H, P.N, P.M * P.B, W, P.pad_off);
+            hipLaunchKernelGGL((grad_out_kernel<T, 1>), grid, dim3(256), 0, s, g, P.E, P.H, P.N, P.M * P.B, W, P.pad_off);
         return static_cast<int>(hipGetLastError());
     });
 }

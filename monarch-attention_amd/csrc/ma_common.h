@@ -85,7 +85,8 @@ int launch_bwd_zero(float* p, long long n, hipStream_t s);
 int launch_bwd_z(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, hipStream_t s);
 int launch_bwd_l(const Problem& P, const BwdBuffers& G, int dt_qk, hipStream_t s);
 int launch_bwd_r(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, bool first, bool with_v, hipStream_t s);
-int launch_bwd_out(const float* src, void* dst, const long long* st, int dt, const Problem& P, int W, hipStream_t s);
+int launch_bwd_out(int n, const float* const* src, void* const* dst, const long long (*st)[3], int dt, const Problem& P, int W,
+                   hipStream_t s);
 
 // MFMA stage kernels (fp16 / bf16, Dv == D <= 128, D % 8 == 0, B, M <= 128,
 // 16-byte aligned rows).
