@@ -81,6 +81,12 @@ bool bwd_fits(const Problem& P);
 // matrix-core backward stages: MA_ERR_UNSUPPORTED when the problem's tiles do not fit the LDS
 int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z, hipStream_t s);
 int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool first, bool with_v, hipStream_t s);
+int launch_bwd_lz_mfma_f32(const Problem& P, const BwdBuffers& G, bool z, hipStream_t s);
+int launch_bwd_lz_mfma_f16(const Problem& P, const BwdBuffers& G, bool z, hipStream_t s);
+int launch_bwd_lz_mfma_bf16(const Problem& P, const BwdBuffers& G, bool z, hipStream_t s);
+int launch_bwd_r_mfma_f32(const Problem& P, const BwdBuffers& G, bool first, bool with_v, hipStream_t s);
+int launch_bwd_r_mfma_f16(const Problem& P, const BwdBuffers& G, bool first, bool with_v, hipStream_t s);
+int launch_bwd_r_mfma_bf16(const Problem& P, const BwdBuffers& G, bool first, bool with_v, hipStream_t s);
 int launch_bwd_zero(float* p, long long n, hipStream_t s);
 int launch_bwd_z(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, hipStream_t s);
 int launch_bwd_l(const Problem& P, const BwdBuffers& G, int dt_qk, hipStream_t s);
