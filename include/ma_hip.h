@@ -60,7 +60,8 @@ typedef enum ma_status {
     MA_ERR_WORKSPACE = -5,   /* workspace missing, misaligned or too small        */
     MA_ERR_UNSUPPORTED = -6, /* the requested variant cannot run this problem     */
     MA_ERR_VARIANT = -7,     /* unknown ma_variant                                */
-    MA_ERR_DEVICE = -8       /* no usable gfx950 device / device query failed     */
+    MA_ERR_DEVICE = -8,      /* no usable gfx950 device / device query failed     */
+    MA_ERR_STATIC_LIMIT = -9 /* ma_fwd_static: state beyond the built-in scratch  */
 } ma_status;
 
 /* ma_fwd_params.flags.  MA_FLAG_SYNC_READY: the caller guarantees that the sync
@@ -134,6 +135,23 @@ int ma_fwd_select_variant(const ma_fwd_params* p);
 /* Whole forward pass: replaces monarch_attention_torch (ma/ma_torch.py:65-108).
  * `stream` is a hipStream_t (NULL = the default stream). */
 int ma_fwd(const ma_fwd_params* p, void* stream);
+
+/* ma_fwd for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose intermediates are tensors PyTorch
+ * allocates, ma/ma_torch.py:88-104).  The per-call state lives in an array the
+ * library itself holds on every GPU it runs on (MA_STATIC_WORKSPACE_BYTES per
+ * GPU until the process ends); p->workspace, p->workspace_bytes and
+ * MA_FLAG_SYNC_READY are ignored, everything else is as for ma_fwd and the
+ * results are the same.  Problems whose ma_fwd_workspace_bytes() exceeds
+ * MA_STATIC_WORKSPACE_BYTES return MA_ERR_STATIC_LIMIT and launch nothing (the
+ * metric workload, fp16 E=1 H=16 N=4096 D=64, needs 26.8 MiB).  No device memory
+ * is allocated or freed.  All calls on one GPU share that GPU's array: calls that
+ * overlap in time on one GPU (different streams or threads) race.  The first
+ * call on a device looks up the array's address (not a stream operation: make it
+ * once before capturing a graph). */
+#define MA_STATIC_WORKSPACE_BYTES (32u << 20)
+int ma_fwd_static(const ma_fwd_params* p, void* stream);
 
 /* One stage on the state held in the workspace (stage-level parity tests;
  * variants GENERIC and STAGED; MA_ERR_UNSUPPORTED for FUSED, RESIDENT and

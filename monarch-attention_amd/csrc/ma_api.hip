@@ -6,6 +6,13 @@
 
 #include <cmath>
 #include <cstring>
+#include <mutex>
+
+// Scratch of ma_fwd_static: the per-call state (aR, cR, aL, cL, Y, stats, sync area) of callers that
+// cannot bring a workspace of their own.  One copy per GPU, at that GPU's own address, held until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress: kernels get the
+// address that call returns, never the name itself.
+static __device__ __align__(256) unsigned char scratch[MA_STATIC_WORKSPACE_BYTES];
 
 namespace ma {
 namespace {
@@ -339,6 +346,28 @@ int bwd_prepare(const ma_bwd_params* b, ma_fwd_params* pp, BwdLayout* L) {
     return MA_OK;
 }
 
+// Device address of `scratch` on the current device, resolved once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices];
+
+int static_scratch(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return MA_ERR_DEVICE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (ptr == nullptr) return MA_ERR_DEVICE;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return MA_OK;
+}
+
 }  // namespace
 
 int launch_zero_sync(unsigned* sync, hipStream_t s) {
@@ -366,6 +395,7 @@ const char* ma_strerror(int status) {
         case MA_ERR_UNSUPPORTED: return "the requested variant does not support this problem";
         case MA_ERR_VARIANT: return "unknown variant";
         case MA_ERR_DEVICE: return "no usable gfx950 device";
+        case MA_ERR_STATIC_LIMIT: return "the problem's state exceeds MA_STATIC_WORKSPACE_BYTES, the built-in scratch of ma_fwd_static: call ma_fwd with a workspace";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -437,6 +467,24 @@ int ma_fwd(const ma_fwd_params* p, void* stream) {
     st = run_r(pr, p, p->T == 1, true, s);
     if (st) return st;
     return run_z(pr, p, s);
+}
+
+int ma_fwd_static(const ma_fwd_params* p, void* stream) {
+    if (p == nullptr) return MA_ERR_NULL;
+    ma_ws_layout L;
+    int st = layout_of(p, &L);
+    if (st != MA_OK) return st;
+    if (L.total > MA_STATIC_WORKSPACE_BYTES) return MA_ERR_STATIC_LIMIT;
+    void* ptr = nullptr;
+    st = static_scratch(&ptr);
+    if (st != MA_OK) return st;
+    ma_fwd_params pp = *p;
+    pp.workspace = ptr;
+    pp.workspace_bytes = MA_STATIC_WORKSPACE_BYTES;
+    // the array keeps what the last call left: nothing may be assumed about its sync area, so the
+    // one-launch variants clear it with their fill kernel in front of the forward kernel
+    pp.flags &= ~MA_FLAG_SYNC_READY;
+    return ma_fwd(&pp, stream);
 }
 
 int ma_matrix(const ma_fwd_params* p, float* A, void* stream) {

@@ -20,6 +20,8 @@ VARIANT_NAMES = {v: k for k, v in VARIANTS.items()}
 MA_OK = 0
 MA_ERR_NULL, MA_ERR_SHAPE, MA_ERR_DTYPE, MA_ERR_STRIDE = -1, -2, -3, -4
 MA_ERR_WORKSPACE, MA_ERR_UNSUPPORTED, MA_ERR_VARIANT, MA_ERR_DEVICE = -5, -6, -7, -8
+MA_ERR_STATIC_LIMIT = -9
+MA_STATIC_WORKSPACE_BYTES = 32 << 20
 
 
 class FwdParams(C.Structure):
@@ -53,7 +55,7 @@ class WsLayout(C.Structure):
 MA_FLAG_SYNC_READY = 1
 
 EXPORTS = ("ma_abi_version", "ma_strerror", "ma_fwd_workspace_layout", "ma_fwd_workspace_bytes",
-           "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_r_step", "ma_l_step", "ma_z_step",
+           "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_fwd_static", "ma_r_step", "ma_l_step", "ma_z_step",
            "ma_matrix", "ma_bwd_workspace_bytes", "ma_bwd")
 
 _lock = threading.Lock()
@@ -95,6 +97,8 @@ def load() -> C.CDLL:
         lib.ma_fwd_select_variant.argtypes = [P]
         lib.ma_fwd.restype = C.c_int
         lib.ma_fwd.argtypes = [P, C.c_void_p]
+        lib.ma_fwd_static.restype = C.c_int
+        lib.ma_fwd_static.argtypes = [P, C.c_void_p]
         lib.ma_r_step.restype = C.c_int
         lib.ma_r_step.argtypes = [P, C.c_int, C.c_int, C.c_void_p]
         lib.ma_l_step.restype = C.c_int
