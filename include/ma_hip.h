@@ -70,6 +70,12 @@ typedef enum ma_status {
  * Without the flag the FUSED and CHAINED variants clear the area with one extra small
  * launch in front of the forward kernel. */
 #define MA_FLAG_SYNC_READY 1
+/* MA_FLAG_TEST_NO_SPIN: every wait between workgroups of the one-launch variants gives
+ * up on its first unsuccessful poll.  For tests of the failure path: the call then
+ * reports through the sticky error word and NaN output rows exactly as a wait that ran
+ * out of time would, every kernel still runs to its end, and the next call on the
+ * workspace is a normal one. */
+#define MA_FLAG_TEST_NO_SPIN 2
 
 /* Arguments of one forward call; replaces the argument list of
  * monarch_attention_torch (ma/ma_torch.py:65-73). */

@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
-LIB_PATH = os.path.join(LIB_DIR, "libma_hip.so")
+LIB_PATH = os.environ.get("MA_LIB_OUT") or os.path.join(LIB_DIR, "libma_hip.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
 # -packed-fp32-ops is switched off for the device code on purpose: the packed
@@ -25,7 +25,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-u
          # MFMA results straight into VGPRs: the kernels consume every accumulator on the VALU right
          # away (softmax, rounding), so AGPR accumulators only add a v_accvgpr_read per value
          "-mllvm", "-amdgpu-mfma-vgpr-form",
-         "-I", os.path.join(ROOT, "include"), "-I", CSRC]
+         "-I", os.path.join(ROOT, "include"), "-I", CSRC] + os.environ.get("MA_EXTRA_FLAGS", "").split()
 
 
 def sources():

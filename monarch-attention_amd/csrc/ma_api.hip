@@ -30,7 +30,7 @@ int check_shape(const ma_fwd_params* p) {
     if (p->E < 1 || p->H < 1 || p->N < 1 || p->D < 1 || p->Dv < 1 || p->B < 1 || p->T < 1) return MA_ERR_SHAPE;
     if (!dtype_ok(p->dtype_qk) || !dtype_ok(p->dtype_v)) return MA_ERR_DTYPE;
     if (p->variant < MA_VARIANT_AUTO || p->variant > MA_VARIANT_CHAINED) return MA_ERR_VARIANT;
-    if (p->flags & ~MA_FLAG_SYNC_READY) return MA_ERR_SHAPE;
+    if (p->flags & ~(MA_FLAG_SYNC_READY | MA_FLAG_TEST_NO_SPIN)) return MA_ERR_SHAPE;
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
     const long long Np = M * p->B;
     // every launch grid and every in-kernel int index must stay inside int32
@@ -111,6 +111,7 @@ Problem make_problem(const ma_fwd_params* p, const ma_ws_layout& L) {
     // sm_scale = 1/sqrt(D) as a Python float, used as an fp32 scalar (ma_torch.py:79)
     P.sm_scale = static_cast<float>(1.0 / std::sqrt(static_cast<double>(p->D)));
     P.eps = p->eps;
+    P.test_no_spin = (p->flags & MA_FLAG_TEST_NO_SPIN) ? 1 : 0;
     return P;
 }
 
@@ -283,6 +284,11 @@ int prepare(const ma_fwd_params* p, Prepared* out) {
     if (v < 0) return v;
     out->P = make_problem(p, L);
     out->variant = v;
+    // Streaming stores pay where a launch writes a state that fits the L2 caches and ends right
+    // after (few long heads with 64-row blocks: the metric workload gains 1.5 us per forward);
+    // with more, smaller problems or a state beyond the caches they cost 5-10 %.
+    out->P.stream_stores = v == MA_VARIANT_STAGED && p->dtype_qk != MA_F32 && p->B > 32 && out->P.M > 32 &&
+                           static_cast<long long>(p->E) * p->H * out->P.M * p->B <= 128 * 1024;
     return MA_OK;
 }
 

@@ -30,6 +30,8 @@ struct Problem {
     int E, H, N, D, Dv, B, M, T, pad_off;
     long long qs[3], ks[3], vs[3], os[3], ms[2];
     float sm_scale, eps;
+    int stream_stores;   // state / output rows that are whole 128-byte lines go out as streaming stores
+    int test_no_spin;    // waits between workgroups give up at once (failure-path tests)
 };
 
 __device__ __forceinline__ bool token_ok(const Problem& P, int e, int t) {
@@ -142,7 +144,7 @@ int launch_chain_bf16_d4(const Problem& P, bool sync_ready, hipStream_t s);
 int launch_chain_bf16_d5(const Problem& P, bool sync_ready, hipStream_t s);
 int launch_chain_bf16_d8(const Problem& P, bool sync_ready, hipStream_t s);
 
-constexpr uint64_t kTeamSyncBytes = 4 * (16 + (16 + 3 * 64) * 1024);  // header + one sector per multi-workgroup team
+constexpr uint64_t kTeamSyncBytes = 4 * (32 + 256 * 1024);   // header + one 1 KiB sector per multi-workgroup team
 constexpr uint64_t kChainSyncBytes = 4 * 256 * 1024;                  // flag words of the chained kernel
 constexpr uint64_t kSyncAreaBytes = kTeamSyncBytes + kChainSyncBytes;
 // Zero-fills the sync area of a workspace (a small fill kernel, graph-capture safe).

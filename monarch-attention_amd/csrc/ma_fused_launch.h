@@ -10,26 +10,25 @@
 namespace ma {
 namespace mfma {
 
-// Team size and team count for `heads` heads when `capacity` workgroups are
-// co-resident: as many workgroups per head as there are tasks in the widest
-// phase, but never more than fit at once; tasks are dealt evenly.
+// Team size and team count for `heads` heads when `capacity` workgroups are co-resident: as many
+// workgroups per head as there are tasks in the widest phase if all heads can then run at once,
+// else narrower teams (tasks dealt evenly) and, below one workgroup per head, teams of one that
+// take the heads in turn.  Teams of several workgroups come in multiples of 8, so that the ids
+// x, x + 8, ... of a team sit on one XCD; the grid is rounded up, surplus teams have no head.
 inline FusedPlan plan_teams(long long heads, int tasks_r, int tasks_l, int capacity) {
     FusedPlan pl;
     const int widest = tasks_r > tasks_l ? tasks_r : tasks_l;
-    const long long pairs = (heads + 1) / 2;  // a team keeps two heads in flight
-    long long limit = capacity / pairs;
-    if (limit < 1) limit = 1;
-    if (limit > widest) limit = widest;
-    if (limit > kMaxTeamSize) limit = kMaxTeamSize;
-    const int per_wg = static_cast<int>((widest + limit - 1) / limit);
+    const long long heads8 = (heads + 7) / 8 * 8;
+    long long g = capacity / heads8;
+    if (g > widest) g = widest;
+    if (g > kMaxTeamSize) g = kMaxTeamSize;
+    if (g < 1) g = 1;
+    const int per_wg = static_cast<int>((widest + g - 1) / g);
     pl.G = (widest + per_wg - 1) / per_wg;
-    long long nteams = capacity / pl.G;
-    const long long most = pl.G > 1 ? pairs : heads;  // one-workgroup teams take their heads one at a time
-    if (nteams > most) nteams = most;
-    if (nteams > 8) nteams -= nteams % 8;  // whole teams per XCD
+    long long nteams = pl.G > 1 ? heads8 : (heads < capacity ? heads : capacity);
     pl.nteams = static_cast<int>(nteams);
-    pl.xcd_map = (pl.nteams % 8 == 0) ? 1 : 0;
-    pl.spin_limit = 1u << 22;
+    pl.xcd_map = (pl.G > 1 && pl.nteams % 8 == 0) ? 1 : 0;
+    pl.spin_limit = 1u << 18;   // a legitimate wait lasts one phase of one head (well under a millisecond)
     return pl;
 }
 
@@ -58,13 +57,11 @@ int launch_fused_w(const Problem& P, bool sync_ready, hipStream_t s) {
     const long long heads = static_cast<long long>(P.E) * P.H;
     const int tasks_r = (P.M + Split<NTB, W>::PPW - 1) / Split<NTB, W>::PPW;
     const int tasks_l = (P.B + Split<NTM, W>::PPW - 1) / Split<NTM, W>::PPW;
-    const FusedPlan pl = plan_teams(heads, tasks_r, tasks_l, caps.capacity);
-    {   // the workspace holds one state slot per head: the slots the grid will touch must exist
-        const long long last = pl.nteams - 1;
-        const long long max_slot = pl.G > 1 ? 2 * last + ((last + pl.nteams < heads) ? 1 : 0) : last;
-        if (pl.nteams < 1 || pl.G < 1 || pl.G > kMaxTeamSize || max_slot >= heads) return MA_ERR_UNSUPPORTED;
-        if (pl.xcd_map && (pl.nteams % 8 != 0)) return MA_ERR_UNSUPPORTED;
-    }
+    FusedPlan pl = plan_teams(heads, tasks_r, tasks_l, caps.capacity);
+    if (P.test_no_spin) pl.spin_limit = 0;
+    // the grid must be co-resident (workgroups wait for each other) and the teams need their sync sectors
+    if (pl.nteams < 1 || pl.G < 1 || pl.G > kMaxTeamSize) return MA_ERR_UNSUPPORTED;
+    if (static_cast<long long>(pl.nteams) * pl.G > caps.capacity) return MA_ERR_UNSUPPORTED;
     if (pl.G > 1 && pl.nteams > kMaxTeams) return MA_ERR_UNSUPPORTED;
     if (!sync_ready) {
         const int err = launch_zero_sync(P.sync, s);

@@ -468,7 +468,7 @@ struct Resident {
                 }
                 O[dt] = acc;
             }
-            store_row<T, DT>(S.out, l < M ? tok_off(t, P.N, S.ost) : kOob, D, O, q);   // padded query rows are dropped
+            store_row<T, DT>(S.out, l < M ? tok_off(t, P.N, S.ost) : kOob, D, O, q, S.stream_out);   // padded query rows are dropped
         }
         round_end<WPM>(P, rd);
     }

@@ -53,6 +53,7 @@ class WsLayout(C.Structure):
 
 
 MA_FLAG_SYNC_READY = 1
+MA_FLAG_TEST_NO_SPIN = 2
 
 EXPORTS = ("ma_abi_version", "ma_strerror", "ma_fwd_workspace_layout", "ma_fwd_workspace_bytes",
            "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_fwd_static", "ma_r_step", "ma_l_step", "ma_z_step",
