@@ -178,38 +178,54 @@ bool resident_fits(const ma_fwd_params* p) {
     return run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
 }
 
+// Tasks (workgroups) of one phase of one head in the one-launch kernels: four waves per workgroup; a
+// block problem of n rows takes min(ceil(n / 16), 4) waves, rounded up to a power of two.
+long long phase_tasks(long long count, long long rows) {
+    const long long strips = (rows + 15) / 16;
+    const long long waves = strips <= 1 ? 1 : strips <= 2 ? 2 : 4;
+    const long long per_wg = 4 / waves;
+    return (count + per_wg - 1) / per_wg;
+}
+
 // Can the chained kernel take the problem?  Mirrors the launcher's limits: at most 128 tasks per
-// head and phase (one poll covers 128 flags), the heads' flag words fit their part of the sync area,
-// the grid is a 31-bit count.  Four waves per workgroup; a block problem of n rows takes
-// min(ceil(n / 16), 4) waves, rounded up to a power of two.
+// head and phase, the heads' sync words (64-bit counters and release words of the 2T - 1 publishing
+// phases, in whole 128-byte lines) fit their part of the sync area, the grid is a 31-bit count.
 bool chain_fits(const ma_fwd_params* p) {
-    auto tasks = [](long long count, long long rows) {
-        const long long strips = (rows + 15) / 16;
-        const long long waves = strips <= 1 ? 1 : strips <= 2 ? 2 : 4;
-        const long long per_wg = 4 / waves;
-        return (count + per_wg - 1) / per_wg;
-    };
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-    const long long tR = tasks(M, p->B), tL = tasks(p->B, M);
+    const long long tR = phase_tasks(M, p->B), tL = phase_tasks(p->B, M);
     const long long heads = static_cast<long long>(p->E) * p->H;
-    const long long stride = p->T * (tR + tL) + 1;
+    const long long nph1 = 2ll * p->T - 1;
+    const long long stride = (2 * nph1 + 2 + 31) / 32 * 32 + (nph1 + 31) / 32 * 32;
     if (tR > 128 || tL > 128) return false;
     if (heads * stride > static_cast<long long>(kChainSyncBytes / 4)) return false;
     return 8 * ((heads + 7) / 8) * p->T * (tR + tL) <= 0x7fffffffLL;
+}
+
+// Few heads of 64-row problems: every head gets a team with one workgroup per block problem and
+// all teams are on the device at once (256 CUs x 4 workgroups) - the fused kernel then runs each
+// phase like a per-stage launch would, without the launch boundaries.
+bool fused_full_width(const ma_fwd_params* p) {
+    const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+    if (p->B > 64 || M > 64) return false;
+    const long long tR = phase_tasks(M, p->B), tL = phase_tasks(p->B, M);
+    const long long widest = tR > tL ? tR : tL;
+    const long long heads = static_cast<long long>(p->E) * p->H;
+    return heads < 32 && widest > 1 && (heads + 7) / 8 * 8 * widest <= 1024;
 }
 
 // The variant a problem resolves to.  AUTO: the MFMA kernels when the problem
 // qualifies; among them (measured on MI355X)
 //  * the resident kernel when a head's state fits in LDS and there are enough
 //    heads to occupy the device with one workgroup per head,
+//  * else the fused kernel (one launch, one team of workgroups per head) for fewer
+//    than 32 heads of problems of up to 64 rows when every head gets a full-width
+//    team at once (the metric workload: 18 us against 19.4 us for T = 1, 42 us
+//    against 55 us for T = 3),
 //  * else the chained kernel (one launch) from 32 heads on for blocks and block
 //    counts of at most 64: with many heads the wait of one head's phase is
-//    covered by other heads' problems; with few heads nothing covers it, and with
-//    128-row problems the one kernel is held to the register / LDS needs of its
-//    largest phase, so there
-//  * one launch per half step is the fastest.
-// The team kernel (FUSED) is never chosen automatically: the per-stage launches
-// beat it for few heads and the chained kernel for many.
+//    covered by other heads' problems; with 128-row problems the one kernel is
+//    held to the register / LDS needs of its largest phase, so there
+//  * one launch per half step is as fast or faster.
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
     const bool fast32 = mfma32_supported(p);   // fp32 operands: per-stage launches only
@@ -224,6 +240,7 @@ int select_variant(const ma_fwd_params* p) {
             if (fast32) return MA_VARIANT_STAGED;
             if (!fast) return MA_VARIANT_GENERIC;
             if (heads >= 128 && resident_fits(p)) return MA_VARIANT_RESIDENT;
+            if (fused_full_width(p)) return MA_VARIANT_FUSED;
             if (heads >= 32 && p->B <= 64 && (static_cast<long long>(p->N) + p->B - 1) / p->B <= 64 && chain_fits(p)) return MA_VARIANT_CHAINED;
             return MA_VARIANT_STAGED;
     }

@@ -23,9 +23,11 @@ int launch_chain_one(const Problem& P, bool sync_ready, hipStream_t s) {
     pl.hx = static_cast<int>((heads + 7) / 8);
     pl.tR = (P.M + Split<NTB, W>::PPW - 1) / Split<NTB, W>::PPW;
     pl.tL = (P.B + Split<NTM, W>::PPW - 1) / Split<NTM, W>::PPW;
-    pl.stride = P.T * (pl.tR + pl.tL) + 1;
+    pl.stride = chain_stride(P.T);
+    pl.go_off = chain_go_offset(P.T);
     pl.spin_limit = P.test_no_spin ? 0u : 1u << 18;   // a legitimate wait lasts one phase of one head (well under a millisecond)
-    // one poll covers 128 flags; the heads' flag words must fit their part of the sync area;
+    // the task count of a phase is a 16-bit field of its arrival counter (and so are the sums of the
+    // XCC ids: at most 15 and 225 per task); the heads' sync words must fit their part of the sync area;
     // the grid must stay a 31-bit count
     if (pl.tR > 128 || pl.tL > 128) return MA_ERR_UNSUPPORTED;
     if (heads * pl.stride > kChainWords) return MA_ERR_UNSUPPORTED;

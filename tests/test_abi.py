@@ -141,7 +141,7 @@ def test_pointer_and_workspace_checks_precede_any_launch():
 def test_select_variant_reports_a_known_variant():
     lib = L.load()
     v = lib.ma_fwd_select_variant(good_params())
-    assert v in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["chained"], L.VARIANTS["resident"])
+    assert v in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["chained"], L.VARIANTS["resident"], L.VARIANTS["fused"])
     p32 = good_params(dtype_qk=L.MA_F32, dtype_v=L.MA_F32)
     assert lib.ma_fwd_select_variant(p32) in (L.VARIANTS["generic"], L.VARIANTS["staged"])
 
@@ -158,8 +158,9 @@ def test_check_maps_status_to_python_exceptions():
 
 def test_auto_variant_policy():
     """AUTO: generic when the MFMA kernels do not apply; resident when a head's
-    state fits in LDS and there are many heads; the chained kernel from 32 heads
-    for problems of up to 64 rows; per-stage launches otherwise."""
+    state fits in LDS and there are many heads; the fused kernel for a few heads of
+    problems of up to 64 rows; the chained kernel from 32 heads for such problems;
+    per-stage launches otherwise."""
     lib = L.load()
 
     def auto(E, H, N, D, B, dt=L.MA_F16, Dv=None):
@@ -171,14 +172,17 @@ def test_auto_variant_policy():
         p.eps = 1e-12
         return L.VARIANT_NAMES[lib.ma_fwd_select_variant(p)]
 
-    assert auto(1, 16, 4096, 64, 64) == "staged"
+    assert auto(1, 16, 4096, 64, 64) == "fused"         # 16 heads x 64 workgroups: every head has a full team at once
+    assert auto(2, 16, 4096, 64, 64) == "chained"
+    assert auto(1, 8, 1024, 64, 32) == "fused"
     assert auto(1, 16, 16384, 64, 128) == "staged"
     assert auto(64, 12, 197, 64, 16) == "resident"
     assert auto(16, 12, 512, 64, 32) == "chained"      # state of a 512-token head does not fit in LDS
     assert auto(8, 16, 1024, 72, 32) == "chained"
     assert auto(4, 16, 16384, 64, 128) == "staged"      # many heads, but 128-row problems
     assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for
-    assert auto(2, 2, 197, 64, 16) == "staged"          # few heads
+    assert auto(2, 2, 197, 64, 16) == "fused"           # few heads
+    assert auto(1, 1, 16, 64, 4) == "staged"            # one workgroup per phase: nothing to fuse
     assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "staged"       # fp32 MFMA stage kernels
     assert auto(1, 2, 7600, 48, 128, dt=L.MA_F32) == "staged"
     assert auto(1, 16, 16384, 128, 128, dt=L.MA_F32) == "generic"   # 128 x 128 fp32 tiles do not fit the LDS
