@@ -71,7 +71,7 @@ typedef enum ma_status {
  * launch in front of the forward kernel. */
 #define MA_FLAG_SYNC_READY 1
 /* MA_FLAG_TEST_NO_SPIN: every wait between workgroups of the one-launch variants gives
- * up on its first unsuccessful poll.  For tests of the failure path: the call then
+ * up at once, without looking at what it waits for.  For tests of the failure path: the call then
  * reports through the sticky error word and NaN output rows exactly as a wait that ran
  * out of time would, every kernel still runs to its end, and the next call on the
  * workspace is a normal one. */

@@ -80,6 +80,10 @@ __device__ __forceinline__ unsigned release_of(unsigned long long total, unsigne
 // one thread: poll the release word of the previous phase; returns it, or 0 if the wait ran out
 __device__ __forceinline__ unsigned chain_wait(const unsigned* go, unsigned spin_limit, unsigned* error) {
     unsigned spins = 0;
+    if (spin_limit == 0u) {   // failure-path tests: give up without looking, whatever the word holds
+        __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return 0u;
+    }
     for (;;) {
         const unsigned w = __hip_atomic_load(go, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (w != 0u) return w;

@@ -121,6 +121,10 @@ __device__ __forceinline__ void team_arrive(TeamSync& ts) {
 // one thread: poll the release word until the barrier of ts.epoch is complete; false if the wait ran out
 __device__ __forceinline__ bool poll_release(const TeamSync& ts) {
     unsigned spins = 0;
+    if (ts.spin_limit == 0u) {   // failure-path tests: give up without looking, whatever the word holds
+        __hip_atomic_store(ts.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return false;
+    }
     for (;;) {
         const unsigned f = __hip_atomic_load(ts.go, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (static_cast<int>(f - ts.epoch) >= 0) return true;

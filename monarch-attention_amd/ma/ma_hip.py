@@ -32,18 +32,80 @@ DEFAULT_VARIANT = "auto"
 # One workspace per (device, stream), grown on demand and reused call after
 # call: calls on one stream are ordered, so they can share it.  It is allocated
 # zero-filled, and every forward call leaves its sync area in the state the next
-# call needs (flags cleared, barrier epochs continuing), which is what
+# call needs (counters and epochs continuing), which is what
 # MA_FLAG_SYNC_READY promises to the library.
-_WORKSPACES: dict[tuple[int, int], Tensor] = {}
+#
+# The one-launch kernels (fused, chained) wait for each other's workgroups with
+# bounded waits; a wait that runs out raises a sticky error word in the
+# workspace and the workgroup writes NaN instead of results.  That word is
+# brought to the host WITHOUT synchronising: every few calls a 4-byte copy into
+# pinned memory is queued on a side stream behind the forward kernel, and the
+# next call on the workspace that finds the copy complete looks at it - a failed
+# call is reported by a RuntimeError from a later call, the sync area is cleared
+# again, and the call after that is a normal one.
+_CHECK_EVERY = 16          # calls between two looks at the error word (the first call always looks)
+_TEST_FLAGS = 0            # extra ma_fwd_params.flags for the failure-path tests (MA_FLAG_TEST_NO_SPIN)
+_SYNCING = (L.VARIANTS["fused"], L.VARIANTS["chained"])
 
 
-def _workspace(device: torch.device, stream_ptr: int, nbytes: int) -> Tensor:
+class _Workspace:
+    def __init__(self, device: torch.device, nbytes: int):
+        self.buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        self.err_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        self.pending = None     # (event on the side stream, buffer the copy reads from)
+        self.calls = 0
+        self.dirty = False      # the sync area must be cleared before the next one-launch kernel
+
+
+_WORKSPACES: dict[tuple[int, int], _Workspace] = {}
+_SIDE_STREAMS: dict[int, torch.cuda.Stream] = {}
+
+
+def _workspace(device: torch.device, stream_ptr: int, nbytes: int) -> _Workspace:
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
-    ws = _WORKSPACES.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _WORKSPACES[key] = ws
-    return ws
+    w = _WORKSPACES.get(key)
+    if w is None:
+        w = _WORKSPACES[key] = _Workspace(device, nbytes)
+    elif w.buf.numel() < nbytes:
+        if w.pending is not None:          # let the queued look at the old buffer finish first
+            w.pending[0].synchronize()
+            _collect(w)
+        w.buf = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    return w
+
+
+def _collect(w: _Workspace) -> None:
+    """Look at a completed copy of the error word; raise if a call on this workspace failed."""
+    w.pending = None
+    code = int(w.err_host.item())
+    if code == 0:
+        return
+    w.err_host.zero_()
+    w.dirty = True
+    w.buf[4:8].zero_()      # the word is sticky: clear it for the calls to come
+    what = {1: "a bounded wait between workgroups ran out",
+            2: "workgroups of one head ran on different XCDs (the one-launch kernels rely on ids x, x + 8, ... "
+               "sharing an XCD)"}.get(code, f"error word {code}")
+    raise RuntimeError(f"monarch_attention_hip: an earlier forward call on this stream failed: {what}; its output "
+                       f"holds NaN rows.  The workspace has been reset; pass variant='staged' to avoid the "
+                       f"one-launch kernels")
+
+
+def _queue_check(w: _Workspace, device: torch.device, main: "torch.cuda.Stream") -> None:
+    """Queue a copy of the error word to pinned memory behind the work queued on `main` so far,
+    on a side stream: the main stream never waits for it."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    side = _SIDE_STREAMS.get(idx)
+    if side is None:
+        side = _SIDE_STREAMS[idx] = torch.cuda.Stream(device=device)
+    after = torch.cuda.Event()
+    after.record(main)
+    side.wait_event(after)
+    with torch.cuda.stream(side):
+        w.err_host.copy_(w.buf[4:8].view(torch.int32), non_blocking=True)
+        done = torch.cuda.Event()
+        done.record(side)
+    w.pending = (done, w.buf)
 
 
 def sync_status() -> int:
@@ -51,16 +113,19 @@ def sync_status() -> int:
     workspaces (synchronises the device): 0 = every wait between workgroups was
     satisfied; 1 = a bounded wait ran out (results of that call are invalid);
     2 = a producer ran on another XCD than its consumer (the device does not
-    deal workgroup ids to XCDs the way the chained kernel is built on)."""
+    deal workgroup ids to XCDs the way the one-launch kernels are built on)."""
     worst = 0
-    for ws in _WORKSPACES.values():
-        torch.cuda.synchronize(ws.device)
-        worst = max(worst, int(ws[4:8].view(torch.int32).item()))
+    for w in _WORKSPACES.values():
+        torch.cuda.synchronize(w.buf.device)
+        worst = max(worst, int(w.buf[4:8].view(torch.int32).item()))
     return worst
 
 
 def clear_workspace_cache() -> None:
     """Drop the cached per-stream workspaces (frees their device memory)."""
+    for w in _WORKSPACES.values():
+        if w.pending is not None:
+            w.pending[0].synchronize()
     _WORKSPACES.clear()
 
 
@@ -154,11 +219,11 @@ def _params_for(lib, q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: i
             L.check(lib.ma_fwd_workspace_layout(tmpl, L.WsLayout()), "monarch_attention_hip")
         if len(_PARAM_CACHE) >= _PARAM_CACHE_MAX:
             _PARAM_CACHE.clear()
-        hit = _PARAM_CACHE[key] = (bytes(tmpl), nbytes)
+        hit = _PARAM_CACHE[key] = (bytes(tmpl), nbytes, lib.ma_fwd_select_variant(tmpl))
     p = L.FwdParams.from_buffer_copy(hit[0])
     p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     p.mask = mask_u8.data_ptr() if mask_u8 is not None else None
-    return p, hit[1]
+    return p, hit[1], hit[2]
 
 
 def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, T: int, B: int,
@@ -182,12 +247,19 @@ def _forward(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int, pre_pad
     E, H, N, _ = q.shape
     with torch.cuda.device(q.device):
         out = _empty_like_layout(v, (E, H, N, v.shape[-1]))
-        p, nbytes = _params_for(lib, q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
-        stream = torch.cuda.current_stream(q.device).cuda_stream
-        ws = _workspace(q.device, stream, nbytes)
-        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
-        p.flags = L.MA_FLAG_SYNC_READY
-        L.check(lib.ma_fwd(p, stream), "ma_fwd")
+        p, nbytes, resolved = _params_for(lib, q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
+        main = torch.cuda.current_stream(q.device)
+        w = _workspace(q.device, main.cuda_stream, nbytes)
+        if w.pending is not None and w.pending[0].query():
+            _collect(w)   # raises if an earlier call on this workspace failed
+        p.workspace, p.workspace_bytes = w.buf.data_ptr(), w.buf.numel()
+        p.flags = (0 if w.dirty else L.MA_FLAG_SYNC_READY) | _TEST_FLAGS
+        L.check(lib.ma_fwd(p, main.cuda_stream), "ma_fwd")
+        if resolved in _SYNCING:
+            w.dirty = False   # the library cleared the sync area in front of this launch if it had to
+            if w.pending is None and (w.calls % _CHECK_EVERY == 0 or _TEST_FLAGS):
+                _queue_check(w, q.device, main)
+            w.calls += 1
     return out
 
 
@@ -223,7 +295,7 @@ def monarch_matrix_hip(q: Tensor, k: Tensor, attn_mask: Tensor | None, T: int, B
         if nbytes == 0:
             L.check(lib.ma_fwd_workspace_layout(p, L.WsLayout()), "monarch_matrix_hip")
         stream = torch.cuda.current_stream(q.device).cuda_stream
-        ws = _workspace(q.device, stream, nbytes)
+        ws = _workspace(q.device, stream, nbytes).buf
         p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
         p.flags = L.MA_FLAG_SYNC_READY
         st = lib.ma_matrix(p, A.data_ptr(), stream)

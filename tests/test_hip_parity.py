@@ -518,3 +518,72 @@ def test_random_shapes_every_variant(idx, E, H, N, D, B, T, pre, dt, masked):
         ran.append(variant)
     assert "auto" in ran and "generic" in ran
     assert sync_status() == 0
+
+
+# ---------------------------------------------------------------- a wait between workgroups that runs out is loud
+@pytest.mark.parametrize("variant", ["fused", "chained"])
+def test_wait_that_runs_out_is_loud_and_leaves_the_workspace_usable(variant):
+    """MA_FLAG_TEST_NO_SPIN makes every wait of the one-launch kernels give up at once (forced from the
+    host; every kernel still runs to its end).  The call must then raise the sticky error word and
+    write NaN rows instead of results computed from a state that may be incomplete, and the next
+    call on the same workspace must be an ordinary, correct one."""
+    lib = L.load()
+    E, H, N, D, B, T = 1, 2, 1024, 64, 32, 2
+    q, k, v = to_dev(*seeded_qkv(E, H, N, D, torch.float16, seed=3))
+    want = monarch_attention_oracle(q.cpu(), k.cpu(), v.cpu(), None, T, B, False)
+    out = torch.zeros_like(v)
+    p = make_params(q, k, v, None, out, T, B, False, variant)
+    nbytes = lib.ma_fwd_workspace_bytes(p)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    word = ws[4:8].view(torch.int32)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
+    stream = torch.cuda.current_stream().cuda_stream
+
+    p.flags = L.MA_FLAG_SYNC_READY
+    L.check(lib.ma_fwd(p, stream), "ma_fwd")
+    torch.cuda.synchronize()
+    assert int(word.item()) == 0
+    assert_parity(out.cpu(), want, "f16", f"{variant} before")
+
+    out.zero_()
+    p.flags = L.MA_FLAG_SYNC_READY | L.MA_FLAG_TEST_NO_SPIN
+    L.check(lib.ma_fwd(p, stream), "ma_fwd")
+    torch.cuda.synchronize()
+    assert int(word.item()) == 1, "the wait that ran out was not reported"
+    assert torch.isnan(out.float()).any(dim=-1).all(), "every output row depends on a wait that gave up: all must be NaN"
+
+    word.zero_()
+    out.zero_()
+    p.flags = L.MA_FLAG_SYNC_READY   # no clearing of the sync area: the failed call must have left it consistent
+    for _ in range(2):
+        L.check(lib.ma_fwd(p, stream), "ma_fwd")
+    torch.cuda.synchronize()
+    assert int(word.item()) == 0
+    assert_parity(out.cpu(), want, "f16", f"{variant} after")
+
+
+def test_module_reports_a_failed_call_at_a_later_call(monkeypatch):
+    """The Python operator never synchronises to look at the error word: a failed call is reported
+    by a RuntimeError from a later call on the same stream, after which calls are normal again."""
+    from ma import ma_hip
+    E, H, N, D, B, T = 1, 2, 1024, 64, 32, 2
+    q, k, v = to_dev(*seeded_qkv(E, H, N, D, torch.float16, seed=4))
+    want = monarch_attention_oracle(q.cpu(), k.cpu(), v.cpu(), None, T, B, False)
+    ma_hip.clear_workspace_cache()
+    good = monarch_attention_hip(q, k, v, None, T, B, False, variant="fused")
+    torch.cuda.synchronize()
+    monkeypatch.setattr(ma_hip, "_TEST_FLAGS", L.MA_FLAG_TEST_NO_SPIN)
+    bad = monarch_attention_hip(q, k, v, None, T, B, False, variant="fused")   # returns: nothing is known yet
+    monkeypatch.setattr(ma_hip, "_TEST_FLAGS", 0)
+    torch.cuda.synchronize()
+    assert torch.isnan(bad.float()).any()
+    with pytest.raises(RuntimeError, match="earlier forward call"):
+        for _ in range(3):    # the look at the error word is queued behind a call and read by a later one
+            monarch_attention_hip(q, k, v, None, T, B, False, variant="fused")
+            torch.cuda.synchronize()
+    again = monarch_attention_hip(q, k, v, None, T, B, False, variant="fused")
+    torch.cuda.synchronize()
+    assert_parity(good.cpu(), want, "f16", "before the failure")
+    assert_parity(again.cpu(), want, "f16", "after the failure")
+    assert sync_status() == 0
+    ma_hip.clear_workspace_cache()
