@@ -3,26 +3,41 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cM] [--T 1]
                     [--variant auto|generic|staged|fused|resident|chained] [--no-cpu] [--no-sdpa] [--no-sweep]
+    python bench.py --sweep-n | --sweep-e        # the reference's own sweep protocol, against dense SDPA
+    python bench.py --record-traffic FETCH.csv WRITE.csv [--config cM --T 1 --variant auto]
 
 A step is ONE forward call of the hot path (monarch_attention, all T steps)
 through the C ABI on synthetic inputs that are already resident in HBM.  The
 default workload is the configuration the headline metric is quoted on: fp16,
 E=1, H=16, N=4096, D=64, block B=64 (=sqrt(N)), post-pad, no mask, with T=1 as in
-the reference's own micro-benchmark protocol (perfbench/bench.py:427-431); the
-sweep over T = 1, 2, 3 is reported next to it.  Inputs rotate over enough
-distinct (q, k, v, out) sets to exceed the 256 MB Infinity Cache, so every step
-reads its operands from HBM.
+the reference's own micro-benchmark protocol (perfbench/bench.py:427-431); T = 1,
+2, 3 are reported next to it.  Inputs rotate over enough distinct (q, k, v, out)
+sets to exceed the 256 MB Infinity Cache, so every step reads its operands from
+HBM.
 
 Prints ONE JSON line.  `value` is the forward throughput in TFLOP/s (matmul
 FLOPs on padded sizes, the reference's bmm convention,
-experiments/vit/evaluation.py:50-59); `roofline` prices the dominant kernel's
-algorithmic bytes against the 8 TB/s HBM peak using that kernel's average
-duration measured with HIP events on the launch stream; `cpu_baseline` is the
-CPU oracle (a port of the reference's ma_torch.py) timed on this host.
+experiments/vit/evaluation.py:50-59) over the K timed steps.
+
+`roofline` prices the forward against the 8 TB/s HBM peak: `achieved` is the
+COMPULSORY bytes of one forward (read Q, K, V once, write the output once)
+divided by the summed average durations of the kernels one forward launches,
+each measured with HIP events around back-to-back launches on the launch
+stream.  With a one-launch variant that is one kernel and one launch is one
+forward; with the per-stage launches the per-kernel figures (which count the
+state a stage reads and writes as well) are listed under `stages`, labelled as
+including intermediates.  `traffic` is the memory-side bytes one forward moved in
+a `rocprofv3 --pmc` run (FETCH_SIZE x 2.00, the factor a plain copy of known size
+calibrates, + WRITE_SIZE), read from profiles/traffic.json and only reported when
+that file was recorded for the kernel sources as they are now.  `cpu_baseline` is
+the CPU oracle (a port of the reference's ma_torch.py) timed on this host.
 """
 import argparse
+import csv
+import hashlib
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -47,18 +62,80 @@ CONFIGS = {  # name: (E, H, N, D, B, T, dtype, scale)  - BASELINE.json configs +
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
 MFMA_PEAK_TFLOPS_F32 = 157.3   # dense fp32
+FETCH_SIZE_FACTOR = 2.00       # FETCH_SIZE under-reports a plain copy of known size by this factor (profiles/traffic_cM_T1.md)
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+KERNEL_DIR = os.path.join(ROOT, "monarch-attention_amd", "csrc")
+ONE_LAUNCH = {"fused": "fused_fwd_mfma", "resident": "resident_fwd_mfma", "chained": "chain_fwd_mfma"}
 
-# HBM-side bytes per launch of the dominant kernels on the metric workload, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for a plain
-# 256 MiB device copy (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); see profiles/traffic_cM_T1.md.
-MEASURED_TRAFFIC_BYTES = {
-    ("cM", 1, "r_step(with V)"): 44_188_000,
-    ("cM", 1, "z_step"): 33_935_000,
-    ("cM", 1, "fused_fwd_mfma"): 71_980_000,
-    ("cM", 1, "chain_fwd_mfma"): 70_300_000,
-    ("c3", 2, "chain_fwd_mfma"): 175_100_000,
-    ("c2", 2, "resident_fwd_mfma"): 102_330_000,
-}
+
+def kernel_source_hash() -> str:
+    """Hash of the kernel sources: measured traffic is only quoted for the sources it was measured on."""
+    h = hashlib.sha1()
+    for name in sorted(os.listdir(KERNEL_DIR)):
+        if name.endswith((".h", ".hip")):
+            with open(os.path.join(KERNEL_DIR, name), "rb") as f:
+                h.update(name.encode())
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic(config: str, T: int, variant: str):
+    """Bytes one forward moved on the memory side according to profiles/traffic.json, or None."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            db = json.load(f)
+    except (OSError, ValueError):
+        return None
+    e = db.get(f"{config}:T{T}:{variant}")
+    if not e or e.get("kernel_source_hash") != kernel_source_hash():
+        return None
+    return e["bytes_per_forward"]
+
+
+def record_traffic(args) -> None:
+    """Fold two rocprofv3 --pmc counter files (FETCH_SIZE and WRITE_SIZE runs of this script, same
+    --config / --T / --variant) into profiles/traffic.json: per forward, the mean KiB per dispatch of
+    every forward kernel times the kernels one forward launches."""
+    fetch_csv, write_csv = args.record_traffic
+
+    names = ("r_step_mfma", "l_step_mfma", "z_step_mfma", "fused_fwd_mfma", "chain_fwd_mfma", "resident_fwd_mfma")
+
+    def per_kernel(path, counter):
+        acc = {}
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] != counter:
+                    continue
+                for short in names:   # mangled or demangled, the kernel's name is in there
+                    if short in row["Kernel_Name"]:
+                        acc.setdefault(short, []).append(float(row["Counter_Value"]))
+        return {k: (sum(v) / len(v), len(v)) for k, v in acc.items()}
+
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    E, H, N, D, B, T, dt, _ = CONFIGS[args.config]
+    T = args.T or T
+    # launches of each kernel in one forward (the bench also launches single stages for the per-stage timings:
+    # the per-dispatch means make that irrelevant)
+    per_fwd = {"r_step_mfma": T, "l_step_mfma": T - 1, "z_step_mfma": 1, "fused_fwd_mfma": 1, "chain_fwd_mfma": 1, "resident_fwd_mfma": 1}
+    kernels, total = {}, 0.0
+    for name in sorted(set(fetch) & set(write)):
+        rd, wr = fetch[name][0] * 1024 * FETCH_SIZE_FACTOR, write[name][0] * 1024
+        n = per_fwd.get(name, 0)
+        kernels[name] = {"read_bytes_per_launch": round(rd), "written_bytes_per_launch": round(wr), "launches_per_forward": n,
+                         "dispatches_averaged": fetch[name][1]}
+        total += n * (rd + wr)
+    try:
+        with open(TRAFFIC_JSON) as f:
+            db = json.load(f)
+    except (OSError, ValueError):
+        db = {}
+    db[f"{args.config}:T{T}:{args.variant}"] = {"bytes_per_forward": round(total), "kernels": kernels,
+                                                 "kernel_source_hash": kernel_source_hash(),
+                                                 "fetch_size_factor": FETCH_SIZE_FACTOR}
+    with open(TRAFFIC_JSON, "w") as f:
+        json.dump(db, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps({"recorded": f"{args.config}:T{T}:{args.variant}", "bytes_per_forward": round(total), "kernels": kernels}))
 
 
 def main():
@@ -71,7 +148,14 @@ def main():
     ap.add_argument("--variant", default="auto", choices=["auto", "generic", "staged", "fused", "resident", "chained"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sdpa", action="store_true", help="skip the dense SDPA comparison")
-    ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep over the variants")
+    ap.add_argument("--sweep-n", action="store_true",
+                    help="the reference's sequence-length sweep (perfbench/bench.py:87-127): fp16 E=1 H=12 D=64, N = 2^10..2^14, "
+                         "block floor(sqrt(N)), T=1, against dense SDPA")
+    ap.add_argument("--sweep-e", action="store_true",
+                    help="the reference's batch sweep (perfbench/bench.py:42-85): fp16 N=256 H=12 D=64 block 16, E = 2^3..2^13, T=1")
+    ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="fold two rocprofv3 --pmc counter_collection.csv files into profiles/traffic.json (no GPU needed)")
     ap.add_argument("--matrix", action="store_true",
                     help="time ma_matrix (the dense (E,H,N,N) attention matrix of get_matrix) instead of the forward metric")
     ap.add_argument("--backward", action="store_true",
@@ -80,6 +164,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE GPU (heads are independent problems: more GPUs would each take "
                  "a share of E*H with no communication) - run with --gpus 1")
+    if args.record_traffic:
+        record_traffic(args)
+        return
 
     import torch
 
@@ -92,12 +179,86 @@ def main():
     lib = L.load()   # fails loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+    stream = torch.cuda.current_stream(dev)
+    sp = stream.cuda_stream
+    F = torch.nn.functional
+
+    def checked(status):
+        if status:
+            L.check(status, "launch")
+
+    def event_avg(fn, n):
+        """Average duration (ms) of n back-to-back calls of fn between two events on the launch stream."""
+        for i in range(3):
+            fn(i)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        for i in range(n):
+            fn(i)
+        b.record(stream)
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n
+
+    def batch_stats(fn, steps):
+        """median / min / mean ms per call over batches of 20 back-to-back calls."""
+        per = 20
+        nb = max(5, steps // per)
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(nb + 1)]
+        evs[0].record(stream)
+        for b in range(nb):
+            for i in range(per):
+                fn(b * per + i)
+            evs[b + 1].record(stream)
+        torch.cuda.synchronize()
+        ts = [evs[b].elapsed_time(evs[b + 1]) / per for b in range(nb)]
+        return {"median_ms": round(statistics.median(ts), 5), "min_ms": round(min(ts), 5), "mean_ms": round(statistics.fmean(ts), 5),
+                "batches": nb, "calls_per_batch": per}
+
+    # ------------------------------------------------------------------ the reference's sweep protocol
+    if args.sweep_n or args.sweep_e:
+        rows = []
+        if args.sweep_n:
+            shapes = [(1, 12, 2 ** k, 64, int((2 ** k) ** 0.5)) for k in range(10, 15)]
+            name = "sweep_n: fp16 E1 H12 D64, block floor(sqrt(N)), T=1 (perfbench/bench.py:87-127)"
+        else:
+            shapes = [(2 ** k, 12, 256, 64, 16) for k in range(3, 14)]
+            name = "sweep_e: fp16 N256 H12 D64 block 16, T=1 (perfbench/bench.py:42-85)"
+        for (E, H, N, D, B) in shapes:
+            gen = torch.Generator().manual_seed(0)
+            set_bytes = 4 * E * H * N * D * 2
+            nbuf = max(2, min(16, -(-640 * 2 ** 20 // set_bytes)))
+            base = [torch.randn(min(E, 64), H, N, D, generator=gen).to(torch.float16) for _ in range(3)]
+            sets = []
+            for i in range(nbuf):
+                q, k, v = (t.to(dev).roll(i, dims=2).repeat(-(-E // t.shape[0]), 1, 1, 1)[:E].contiguous() for t in base)
+                sets.append((q, k, v, torch.empty_like(q)))
+            ps = [make_params(q, k, v, None, o, 1, B, False, "auto") for (q, k, v, o) in sets]
+            nbytes = lib.ma_fwd_workspace_bytes(ps[0])
+            ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+            for p in ps:
+                p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), nbytes, L.MA_FLAG_SYNC_READY
+            variant = L.VARIANT_NAMES[lib.ma_fwd_select_variant(ps[0])]
+            n = 100 if set_bytes < (1 << 30) else 20
+            ma = batch_stats(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), n)
+            sd = batch_stats(lambda i: F.scaled_dot_product_attention(*sets[i % nbuf][:3]), max(n // 2, 20))
+            rows.append({"E": E, "H": H, "N": N, "D": D, "block": B, "variant": variant, "monarch": ma, "sdpa": sd,
+                         "speedup_vs_sdpa": round(sd["median_ms"] / ma["median_ms"], 2),
+                         "monarch_tflops": round(forward_flops(E, H, N, D, D, B, 1) / (ma["median_ms"] * 1e-3) / 1e12, 2),
+                         "fwd_hbm_frac": round(forward_bytes(E, H, N, D, D, 2) / (ma["median_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+            del sets, ps, ws
+            torch.cuda.empty_cache()
+        faster = [r for r in rows if r["speedup_vs_sdpa"] > 1.0]
+        print(json.dumps({"metric": "MonarchAttn fwd vs dense SDPA (reference sweep protocol)", "sweep": name, "unit": "ms",
+                          "n_gpus": 1, "dtype": "f16", "data": "synthetic", "higher_is_better": False,
+                          "first_faster_than_sdpa": ({"E": faster[0]["E"], "N": faster[0]["N"]} if faster else None),
+                          "rows": rows}))
+        return
+
     E, H, N, D, B, T, dt, scale = CONFIGS[args.config]
     if args.T is not None:
         T = args.T
     dtype = DT[dt]
     elt = torch.empty((), dtype=dtype).element_size()
-    stream = torch.cuda.current_stream(dev)
 
     # ---- synthetic inputs: torch.manual_seed(0), q, k, v = randn on the CPU in fp32, in that order
     gen = torch.Generator().manual_seed(0)
@@ -119,7 +280,6 @@ def main():
         return ps, ws
 
     def run_steps(ps, n):
-        sp = stream.cuda_stream
         fwd = lib.ma_fwd
         for i in range(n):
             st = fwd(ps[i % nbuf], sp)
@@ -178,57 +338,57 @@ def main():
                           "config": {"workload": f"{args.config}: E{E} H{H} N{N} D{D} block {B} T={T}", "variant": variant}}))
         return
 
-    resolved = L.VARIANT_NAMES[lib.ma_fwd_select_variant(make_params(*sets[0][:3], None, sets[0][3], T, B, False, args.variant))]
-    flops = forward_flops(E, H, N, D, D, B, T)
+    M = -(-N // B)
+    Np = M * B
     cbytes = forward_bytes(E, H, N, D, D, elt)
+    mfma_peak = MFMA_PEAK_TFLOPS_F32 if dt == "f32" else MFMA_PEAK_TFLOPS
+
+    def resolve(T_, variant):
+        return L.VARIANT_NAMES[lib.ma_fwd_select_variant(make_params(*sets[0][:3], None, sets[0][3], T_, B, False, variant))]
+
+    def roofline_of(T_, variant, ps, n):
+        """Roofline entry of one forward with T_ steps: compulsory bytes over the summed average
+        durations of the kernels it launches (events on the launch stream, back-to-back launches)."""
+        res = resolve(T_, variant)
+        stages = {}
+        if res in ONE_LAUNCH:
+            kernels = {ONE_LAUNCH[res]: (event_avg(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), n), 1)}
+        else:
+            # per-stage kernels on the state a full forward left in the workspace; (average ms, launches per forward)
+            kernels = {"r_step(with V)": (event_avg(lambda i: checked(lib.ma_r_step(ps[i % nbuf], int(T_ == 1), 1, sp)), n), 1),
+                       "z_step": (event_avg(lambda i: checked(lib.ma_z_step(ps[i % nbuf], sp)), n), 1)}
+            stage_bytes = {"r_step(with V)": E * H * ((2 * N * D + N * D) * elt + 2 * Np * D * elt + 4 * Np),
+                           "z_step": E * H * (N * D * elt + 2 * Np * D * elt + 4 * Np + N * D * elt)}
+            if T_ > 1:
+                kernels["l_step"] = (event_avg(lambda i: checked(lib.ma_l_step(ps[i % nbuf], sp)), n), T_ - 1)
+                kernels["r_step"] = (event_avg(lambda i: checked(lib.ma_r_step(ps[i % nbuf], 0, 0, sp)), n), T_ - 1)
+                stage_bytes["l_step"] = E * H * (N * D * elt + Np * D * elt + 4 * Np + Np * D * elt + 4 * Np)
+                stage_bytes["r_step"] = E * H * (2 * N * D * elt + Np * D * elt + 4 * Np + 4 * Np)
+            # secondary figure per stage: bytes INCLUDING the state it reads and writes over its own duration
+            stages = {k: {"avg_launch_us": round(v[0] * 1e3, 2), "launches_per_forward": v[1],
+                          "bytes_incl_intermediates": stage_bytes[k],
+                          "stage_copy_frac": round(stage_bytes[k] / (v[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)} for k, v in kernels.items()}
+        fwd_ms = sum(ms_ * cnt for ms_, cnt in kernels.values())
+        dom = max(kernels, key=lambda k: kernels[k][0] * kernels[k][1])
+        achieved = cbytes / (fwd_ms * 1e-3) / 1e9
+        r = {"bound": "hbm", "T": T_, "variant": res, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": recorded_traffic(args.config, T_, variant),
+             "algorithmic_bytes_per_forward": cbytes, "kernel_time_per_forward_us": round(fwd_ms * 1e3, 2),
+             "kernel": dom, "kernel_share": round(kernels[dom][0] * kernels[dom][1] / fwd_ms, 3),
+             "kernels_us": {k: round(v[0] * 1e3, 2) for k, v in kernels.items()},
+             "mfma_frac": round(forward_flops(E, H, N, D, D, B, T_) / (fwd_ms * 1e-3) / 1e12 / mfma_peak, 5)}
+        if stages:
+            r["stages"] = stages
+        return r
+
+    resolved = resolve(T, args.variant)
+    flops = forward_flops(E, H, N, D, D, B, T)
 
     # ---- the timed region: exactly K steps between two synchronisations
     wall_ms, ev_ms, ps, ws = time_forward(T, args.variant, args.steps, args.warmup)
     ms = wall_ms
-
-    # ---- dominant kernel: average launch duration with HIP events on the launch stream
-    def event_avg(fn, n):
-        """Average duration of n back-to-back launches of one kernel between two events."""
-        for i in range(3):
-            fn(i)
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record(stream)
-        for i in range(n):
-            fn(i)
-        b.record(stream)
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) / n
-
-    sp = stream.cuda_stream
-    M = -(-N // B)
-    Np = M * B
-    kernels = {}
-    def checked(status):
-        if status:
-            L.check(status, "stage launch")
-
-    if resolved in ("fused", "resident", "chained"):   # the whole forward is one kernel
-        kname = {"fused": "fused_fwd_mfma", "resident": "resident_fwd_mfma", "chained": "chain_fwd_mfma"}[resolved]
-        kernels[kname] = (event_avg(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), min(args.steps, 200)), cbytes)
-    else:
-        # per-stage kernels on the state a full forward left in the workspace
-        n = min(args.steps, 200)
-        rv_bytes = E * H * ((2 * N * D + N * D) * elt + 2 * Np * D * elt + 4 * Np)          # Q,K,V -> aL,Y,cL
-        kernels["r_step(with V)"] = (event_avg(lambda i: checked(lib.ma_r_step(ps[i % nbuf], int(T == 1), 1, sp)), n), rv_bytes)
-        z_bytes = E * H * (N * D * elt + 2 * Np * D * elt + 4 * Np + N * D * elt)            # Q,aL,Y,cL -> out
-        kernels["z_step"] = (event_avg(lambda i: checked(lib.ma_z_step(ps[i % nbuf], sp)), n), z_bytes)
-        if T > 1:
-            l_bytes = E * H * (N * D * elt + Np * D * elt + 4 * Np + Np * D * elt + 4 * Np)  # Q,aL,cL -> aR,cR
-            kernels["l_step"] = (event_avg(lambda i: checked(lib.ma_l_step(ps[i % nbuf], sp)), n), l_bytes)
-            r_bytes = E * H * (2 * N * D * elt + Np * D * elt + 4 * Np + 4 * Np)              # aR,cR,K -> aL,cL
-            kernels["r_step"] = (event_avg(lambda i: checked(lib.ma_r_step(ps[i % nbuf], 0, 0, sp)), n), r_bytes)
-    dom = max(kernels, key=lambda kname: kernels[kname][0])
-    dom_ms, dom_bytes = kernels[dom]
-    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, T, dom)),
-                "algorithmic_bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_ms * 1e3, 2),
-                "kernels_us": {kname: round(v[0] * 1e3, 2) for kname, v in kernels.items()}}
+    timing = batch_stats(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), max(args.steps, 100))
+    roofline = roofline_of(T, args.variant, ps, min(max(args.steps, 100), 200))
 
     out = {
         "metric": "MonarchAttn fwd TFLOP/s (fp16 B1 H16 N4096 d64, b=64)" if args.config == "cM" else f"MonarchAttn fwd TFLOP/s ({args.config})",
@@ -238,10 +398,12 @@ def main():
         "config": {"workload": f"{args.config}: {dt} E{E} H{H} N{N} D{D} block{B} T{T} post-pad no-mask", "variant": resolved,
                    "flop_per_fwd": flops, "compulsory_bytes_per_fwd": cbytes, "rotating_input_sets": nbuf},
         "stream_ms_per_step": round(ev_ms, 5),
+        "ms_per_step_stats": timing,
         "fwd_hbm_frac": round(cbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-        "fwd_mfma_frac": round(flops / (ev_ms * 1e-3) / 1e12 / (MFMA_PEAK_TFLOPS_F32 if dt == "f32" else MFMA_PEAK_TFLOPS), 5),
+        "fwd_mfma_frac": round(flops / (ev_ms * 1e-3) / 1e12 / mfma_peak, 5),
         "roofline": roofline,
     }
+    del ps, ws
 
     # ---- the same forward through the nn.Module-level host wrapper (allocates its output per call)
     q0, k0, v0, _ = sets[0]
@@ -256,8 +418,15 @@ def main():
     torch.cuda.synchronize()
     out["module_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / nmod, 5)
 
-    # ---- sweep over T and variants (same protocol, fewer steps)
+    # ---- T = 1, 2, 3 with the selected variant: one roofline entry each; and every variant (same protocol, fewer steps)
     if not args.no_sweep:
+        by_T = []
+        for T_ in (1, 2, 3):
+            ps_, ws_ = prepared(T_, args.variant)
+            run_steps(ps_, 10)
+            by_T.append(roofline_of(T_, args.variant, ps_, 100))
+            del ps_, ws_
+        out["roofline_by_T"] = by_T
         sweep = {}
         for T_ in (1, 2, 3):
             for variant in ("staged", "fused", "chained", "resident"):
@@ -272,7 +441,6 @@ def main():
 
     # ---- dense softmax attention on the same GPU (PyTorch's own SDPA backend), same harness
     if not args.no_sdpa and dt != "f32":
-        F = torch.nn.functional
         for _ in range(3):
             F.scaled_dot_product_attention(q0, k0, v0)
         torch.cuda.synchronize()
