@@ -18,7 +18,7 @@
  *
  * Tensor conventions (the reference's, ma/ma_torch.py:74-90):
  *   q, k : (E, H, N, D)   v : (E, H, N, Dv)   out : (E, H, N, Dv) in v's dtype
- *   mask : (E, N) bytes, non-zero = keep the key/query token, or NULL
+ *   mask : (E, N), non-zero = keep the key/query token (see ma_mask_dtype), or NULL
  *   B block size, M = ceil(N / B) blocks, Np = M * B; zero padding at the
  *   front (pre_pad != 0) or the back; T alternating steps.
  * Strides are in ELEMENTS for the dims (e, h, n); the innermost dim must be
@@ -37,6 +37,23 @@ extern "C" {
 #define MA_ABI_VERSION 1
 
 typedef enum ma_dtype { MA_F32 = 0, MA_F16 = 1, MA_BF16 = 2 } ma_dtype;
+
+/* Element type of the (E, N) mask.  The reference combines the mask with
+ * torch.logical_and (ma/ma_torch.py:98): any non-zero element keeps the token
+ * (for floating-point masks -0.0 is zero and NaN is non-zero).  Callers pass bool
+ * masks (its tests), int64 tokenizer masks (experiments/roberta/model.py:104-106) and
+ * float 1.0 / 0.0 masks (experiments/bart/model.py:145-147); the kernels read all of
+ * them in place.  mask_stride is in elements of this type. */
+typedef enum ma_mask_dtype {
+    MA_MASK_U8 = 0,   /* bool / uint8 / int8 */
+    MA_MASK_I16 = 1,
+    MA_MASK_I32 = 2,
+    MA_MASK_I64 = 3,
+    MA_MASK_F16 = 4,
+    MA_MASK_BF16 = 5,
+    MA_MASK_F32 = 6,
+    MA_MASK_F64 = 7
+} ma_mask_dtype;
 
 typedef enum ma_variant {
     MA_VARIANT_AUTO = 0,    /* fastest variant that supports the problem            */
@@ -83,7 +100,7 @@ typedef struct ma_fwd_params {
     const void* q;           /* device pointers                                   */
     const void* k;
     const void* v;
-    const uint8_t* mask;     /* (E, N) or NULL (ma/ma_torch.py:96-98)             */
+    const void* mask;        /* (E, N) of mask_dtype, or NULL (ma/ma_torch.py:96-98) */
     void* out;               /* (E, H, N, Dv), dtype_v                            */
     void* workspace;         /* >= ma_fwd_workspace_bytes(), 256-byte aligned     */
     uint64_t workspace_bytes;
@@ -99,9 +116,9 @@ typedef struct ma_fwd_params {
     int64_t k_stride[3];
     int64_t v_stride[3];
     int64_t out_stride[3];
-    int64_t mask_stride[2];  /* element (byte) strides of (e, n)                 */
+    int64_t mask_stride[2];  /* element strides of (e, n)                        */
     float eps;               /* 1e-12 in the reference (ma/ma_torch.py:10,38)    */
-    int32_t reserved2;       /* must be 0                                        */
+    int32_t mask_dtype;      /* ma_mask_dtype of the mask's elements (0 = bytes)   */
 } ma_fwd_params;
 
 /* Byte offsets of the per-call state inside the workspace.  The arrays have

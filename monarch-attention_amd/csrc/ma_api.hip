@@ -48,6 +48,7 @@ int check_shape(const ma_fwd_params* p) {
     // inputs may be broadcast over batch / heads (stride 0); output slices must not coincide
     if ((p->E > 1 && p->out_stride[0] == 0) || (p->H > 1 && p->out_stride[1] == 0)) return MA_ERR_STRIDE;
     if (p->mask_stride[0] < 0 || p->mask_stride[1] < 0) return MA_ERR_STRIDE;
+    if (p->mask_dtype < MA_MASK_U8 || p->mask_dtype > MA_MASK_F64) return MA_ERR_DTYPE;
     if (!(p->eps >= 0.0f)) return MA_ERR_SHAPE;
     return MA_OK;
 }
@@ -91,7 +92,12 @@ Problem make_problem(const ma_fwd_params* p, const ma_ws_layout& L) {
     P.q = static_cast<const char*>(p->q);
     P.k = static_cast<const char*>(p->k);
     P.v = static_cast<const char*>(p->v);
-    P.mask = p->mask;
+    P.mask = static_cast<const uint8_t*>(p->mask);
+    {
+        static const int shift[8] = {0, 1, 2, 3, 1, 1, 2, 3};
+        P.mask_shift = shift[p->mask_dtype];
+        P.mask_float = p->mask_dtype >= MA_MASK_F16 ? 1 : 0;
+    }
     P.out = static_cast<char*>(p->out);
     P.aR = ws + L.aR;
     P.cR = reinterpret_cast<float*>(ws + L.cR);
@@ -134,7 +140,7 @@ bool mfma_supported(const ma_fwd_params* p) {
     const unsigned long long n1 = static_cast<unsigned long long>(p->N - 1), db = 2ull * p->D;
     if (n1 * p->q_stride[2] * 2 + db >= lim || n1 * p->k_stride[2] * 2 + db >= lim || n1 * p->v_stride[2] * 2 + db >= lim ||
         n1 * p->out_stride[2] * 2 + db >= lim || static_cast<unsigned long long>(M) * p->B * db >= lim ||
-        n1 * static_cast<unsigned long long>(p->mask_stride[1]) >= lim)
+        n1 * static_cast<unsigned long long>(p->mask_stride[1]) * 8 >= lim)
         return false;
     return true;
 }
@@ -155,7 +161,7 @@ bool mfma32_supported(const ma_fwd_params* p) {
     const unsigned long long n1 = static_cast<unsigned long long>(p->N - 1), db = 4ull * p->D;
     if (n1 * p->q_stride[2] * 4 + db >= lim || n1 * p->k_stride[2] * 4 + db >= lim || n1 * p->v_stride[2] * 4 + db >= lim ||
         n1 * p->out_stride[2] * 4 + db >= lim || static_cast<unsigned long long>(M) * p->B * db >= lim ||
-        n1 * static_cast<unsigned long long>(p->mask_stride[1]) >= lim)
+        n1 * static_cast<unsigned long long>(p->mask_stride[1]) * 8 >= lim)
         return false;
     return mfma32_lds_needed(p->D, p->B, static_cast<int>(M)) <= 160 * 1024;
 }

@@ -30,13 +30,36 @@ struct Problem {
     int E, H, N, D, Dv, B, M, T, pad_off;
     long long qs[3], ks[3], vs[3], os[3], ms[2];
     float sm_scale, eps;
+    int mask_shift;      // log2 of the mask element size in bytes (ms strides are in elements)
+    int mask_float;      // the mask holds floating-point values: -0.0 counts as zero
     int stream_stores;   // state / output rows that are whole 128-byte lines go out as streaming stores
     int test_no_spin;    // waits between workgroups give up at once (failure-path tests)
 };
 
+// Is a mask element non-zero (torch.logical_and's truthiness, ma/ma_torch.py:98)?  `lo` / `hi` are
+// its low and high 32 bits (zero-extended for narrow elements); for floating-point masks the
+// sign bit, which is the top bit of the element, does not count (-0.0 is false, NaN is true).
+__device__ __forceinline__ bool mask_nonzero(const Problem& P, unsigned lo, unsigned hi) {
+    if (P.mask_float) {
+        if (P.mask_shift == 3) hi &= 0x7fffffffu;
+        else if (P.mask_shift == 2) lo &= 0x7fffffffu;
+        else lo &= 0x7fffu;
+    }
+    return (lo | hi) != 0u;
+}
+
 __device__ __forceinline__ bool token_ok(const Problem& P, int e, int t) {
     if (t < 0 || t >= P.N) return false;
-    return P.mask == nullptr || P.mask[e * P.ms[0] + t * P.ms[1]] != 0;
+    if (P.mask == nullptr) return true;
+    const uint8_t* p = P.mask + ((e * P.ms[0] + t * P.ms[1]) << P.mask_shift);
+    unsigned lo = 0, hi = 0;
+    switch (P.mask_shift) {
+        case 0: lo = *p; break;
+        case 1: lo = *reinterpret_cast<const uint16_t*>(p); break;
+        case 2: lo = *reinterpret_cast<const uint32_t*>(p); break;
+        default: lo = reinterpret_cast<const uint32_t*>(p)[0]; hi = reinterpret_cast<const uint32_t*>(p)[1]; break;
+    }
+    return mask_nonzero(P, lo, hi);
 }
 
 template <class T>

@@ -312,7 +312,7 @@ struct Lds {
 // Uniform (per problem) description of the tensors: resources and row pitches in bytes.
 struct Slices {
     rsrc_t q, k, v, out, aR, cR, aL, cL, Y, mask;
-    unsigned qst, kst, vst, ost, mst;   // mst: byte pitch of the mask row, 0 = no mask
+    unsigned qst, kst, vst, ost, mst;   // mst: byte pitch of the mask's token dimension, 0 = no mask
     bool stream_state, stream_out;      // rows of the state arrays / of out are whole, aligned 128-byte lines
 };
 
@@ -328,8 +328,8 @@ __device__ __forceinline__ Slices make_slices(const Problem& P, int e, int h, lo
     S.k = make_rsrc(P.k + (e * P.ks[0] + h * P.ks[1]) * static_cast<long long>(sizeof(T)), n1 * S.kst + db);
     S.v = make_rsrc(P.v + (e * P.vs[0] + h * P.vs[1]) * static_cast<long long>(sizeof(T)), n1 * S.vst + db);
     S.out = make_rsrc(P.out + (e * P.os[0] + h * P.os[1]) * static_cast<long long>(sizeof(T)), n1 * S.ost + db);
-    S.mst = P.mask ? static_cast<unsigned>(P.ms[1]) : 0u;
-    S.mask = make_rsrc(P.mask ? P.mask + e * P.ms[0] : nullptr, P.mask ? n1 * S.mst + 1u : 0u);
+    S.mst = P.mask ? static_cast<unsigned>(P.ms[1]) << P.mask_shift : 0u;
+    S.mask = make_rsrc(P.mask ? P.mask + ((e * P.ms[0]) << P.mask_shift) : nullptr, P.mask ? n1 * S.mst + (1u << P.mask_shift) : 0u);
     const long long np = static_cast<long long>(P.M) * P.B;
     const unsigned state = static_cast<unsigned>(np) * db, stat4 = static_cast<unsigned>(np) * 4u;
     S.aR = make_rsrc(P.aR + wh * np * db, state);
@@ -349,17 +349,29 @@ __device__ __forceinline__ unsigned tok_off(int t, int N, unsigned st) {
     return static_cast<unsigned>(t) < static_cast<unsigned>(N) ? static_cast<unsigned>(t) * st : kOob;
 }
 
-// Mask byte of token t, started as a load and NOT looked at here (a test would wait for it and
+// Mask element of token t, started as a load and NOT looked at here (a test would wait for it and
 // for every load issued before it): padding positions and "no mask" read 0 through the bounds
-// check.  token_kept() decodes it once the problem runs.
+// check.  The element's words are folded into one (a 64-bit element is non-zero iff the OR of its
+// halves is, once the sign bit of a floating-point mask is dropped from the high half; that fold is
+// plain ALU work on the loaded registers and waits for nothing until its result is used).
+// token_kept() decodes it once the problem runs.
 __device__ __forceinline__ unsigned mask_load(const Slices& S, const Problem& P, int t, bool want) {
     if (P.mask == nullptr) return 1u;   // uniform: without a mask nothing is loaded
     const bool in = want && static_cast<unsigned>(t) < static_cast<unsigned>(P.N);
-    return __builtin_amdgcn_raw_buffer_load_b8(S.mask, in ? static_cast<unsigned>(t) * S.mst : kOob, 0, 0);
+    const unsigned off = in ? (static_cast<unsigned>(t) * S.mst) : kOob;
+    switch (P.mask_shift) {   // uniform
+        case 0: return __builtin_amdgcn_raw_buffer_load_b8(S.mask, off, 0, 0);
+        case 1: return __builtin_amdgcn_raw_buffer_load_b16(S.mask, off, 0, 0) & (P.mask_float ? 0x7fffu : 0xffffu);
+        case 2: return __builtin_amdgcn_raw_buffer_load_b32(S.mask, off, 0, 0) & (P.mask_float ? 0x7fffffffu : 0xffffffffu);
+        default: {
+            const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(S.mask, off, 0, 0);
+            return w[0] | (w[1] & (P.mask_float ? 0x7fffffffu : 0xffffffffu));
+        }
+    }
 }
 // real (in range) and not masked out
-__device__ __forceinline__ bool token_kept(const Problem& P, int t, unsigned mask_byte) {
-    return static_cast<unsigned>(t) < static_cast<unsigned>(P.N) && (P.mask == nullptr || mask_byte != 0u);
+__device__ __forceinline__ bool token_kept(const Problem& P, int t, unsigned mask_word) {
+    return static_cast<unsigned>(t) < static_cast<unsigned>(P.N) && (P.mask == nullptr || mask_word != 0u);
 }
 
 // Orders the LDS tile writes of a problem's waves before their reads.  A problem that a single

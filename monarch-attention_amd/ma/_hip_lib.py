@@ -34,7 +34,7 @@ class FwdParams(C.Structure):
         ("dtype_qk", C.c_int32), ("dtype_v", C.c_int32), ("variant", C.c_int32), ("flags", C.c_int32),
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("out_stride", C.c_int64 * 3), ("mask_stride", C.c_int64 * 2),
-        ("eps", C.c_float), ("reserved2", C.c_int32),
+        ("eps", C.c_float), ("mask_dtype", C.c_int32),
     ]
 
 
@@ -52,6 +52,7 @@ class WsLayout(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("aR", "cR", "aL", "cL", "Y", "stats", "sync", "total")]
 
 
+MA_MASK_U8, MA_MASK_I16, MA_MASK_I32, MA_MASK_I64, MA_MASK_F16, MA_MASK_BF16, MA_MASK_F32, MA_MASK_F64 = range(8)
 MA_FLAG_SYNC_READY = 1
 MA_FLAG_TEST_NO_SPIN = 2
 

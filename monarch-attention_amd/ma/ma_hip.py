@@ -24,6 +24,9 @@ from . import _hip_lib as L
 Tensor = torch.Tensor
 
 _DTYPES = {torch.float32: L.MA_F32, torch.float16: L.MA_F16, torch.bfloat16: L.MA_BF16}
+_MASK_DTYPES = {torch.bool: L.MA_MASK_U8, torch.uint8: L.MA_MASK_U8, torch.int8: L.MA_MASK_U8, torch.int16: L.MA_MASK_I16,
+                torch.int32: L.MA_MASK_I32, torch.int64: L.MA_MASK_I64, torch.float16: L.MA_MASK_F16,
+                torch.bfloat16: L.MA_MASK_BF16, torch.float32: L.MA_MASK_F32, torch.float64: L.MA_MASK_F64}
 
 # default variant of monarch_attention_hip; tests and the benchmark switch it
 # per call through the `variant` keyword
@@ -162,7 +165,14 @@ def _check_inputs(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int) ->
 
 
 def _inner_contiguous(t: Tensor) -> Tensor:
-    return t if t.stride(-1) == 1 or t.shape[-1] == 1 else t.contiguous()
+    """The library wants unit stride along the last dimension and token rows that do not overlap
+    (stride(2) >= row width); batch and head dimensions may be broadcast.  Anything else - e.g. an
+    expand() along the tokens - is copied once."""
+    if not (t.stride(-1) == 1 or t.shape[-1] == 1):
+        return t.contiguous()
+    if t.shape[2] > 1 and t.stride(2) < t.shape[-1]:
+        return t.contiguous()
+    return t
 
 
 def _empty_like_layout(v: Tensor, shape) -> Tensor:
@@ -186,6 +196,7 @@ def make_params(q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B
     p = L.FwdParams()
     p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     p.mask = mask_u8.data_ptr() if mask_u8 is not None else None
+    p.mask_dtype = _MASK_DTYPES[mask_u8.dtype] if mask_u8 is not None else L.MA_MASK_U8
     p.E, p.H, p.N, p.D, p.Dv = E, H, N, D, v.shape[-1]
     p.B, p.T, p.pre_pad = B, T, int(bool(pre_pad))
     p.dtype_qk, p.dtype_v = _DTYPES[q.dtype], _DTYPES[v.dtype]
@@ -210,7 +221,7 @@ _PARAM_CACHE_MAX = 256
 def _params_for(lib, q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B: int, pre_pad: bool,
                 variant: str) -> tuple:
     key = (q.shape, q.stride(), k.stride(), v.shape, v.stride(), out.stride(),
-           None if mask_u8 is None else mask_u8.stride(), q.dtype, v.dtype, T, B, bool(pre_pad), variant)
+           None if mask_u8 is None else (mask_u8.stride(), mask_u8.dtype), q.dtype, v.dtype, T, B, bool(pre_pad), variant)
     hit = _PARAM_CACHE.get(key)
     if hit is None:
         tmpl = make_params(q, k, v, mask_u8, out, T, B, pre_pad, variant)
@@ -264,14 +275,16 @@ def _forward(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int, pre_pad
 
 
 def _mask_bytes(attn_mask):
-    """One byte per token, non-zero = keep: truthiness as torch.logical_and sees it
-    (ma/ma_torch.py:98).  bool / uint8 / int8 masks already are that and are read in place
-    (any strides); other dtypes are reduced to bytes by one small elementwise kernel."""
+    """The mask as the library reads it: in place, whatever its dtype (bool, any integer, any
+    float: non-zero = keep, the truthiness torch.logical_and sees, ma/ma_torch.py:98) and whatever
+    its strides.  bool is reinterpreted as bytes; nothing is copied or converted."""
     if attn_mask is None:
         return None
-    if attn_mask.dtype in (torch.bool, torch.uint8, torch.int8):
+    if attn_mask.dtype == torch.bool:
         return attn_mask.view(torch.uint8)
-    return (attn_mask != 0).to(torch.uint8)
+    if attn_mask.dtype not in _MASK_DTYPES:
+        raise TypeError(f"attn_mask dtype {attn_mask.dtype} is not supported")
+    return attn_mask
 
 
 def monarch_matrix_hip(q: Tensor, k: Tensor, attn_mask: Tensor | None, T: int, B: int, pre_pad: bool, *,

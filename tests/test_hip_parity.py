@@ -142,6 +142,33 @@ def test_benchmark_shapes_against_oracle(name, E, H, N, D, B, T, pre, dt, scale,
     assert_parity(out.cpu(), ref, dt, f"{name}/{variant}")
 
 
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("B", [24, 48, 96, 128])
+def test_roberta_block_sizes_with_tokenizer_mask(B, variant):
+    """The block sizes the reference's RoBERTa evaluation sweeps (experiments/roberta/benchmark.py:67-89):
+    N = 384 (max_length padding), T = 1, post-pad, the tokenizer's int64 attention mask with the tail
+    of every sequence masked out."""
+    E, H, N, D, T = 3, 12, 384, 64, 1
+    q, k, v = seeded_qkv(E, H, N, D, torch.float16, seed=B)
+    lengths = torch.tensor([384, 201, 77])
+    mask = (torch.arange(N)[None] < lengths[:, None]).long()
+    ref = monarch_attention_oracle(q, k, v, mask != 0, T, B, False, upcast=True)
+    out = run_hip(*to_dev(q, k, v, mask), T, B, False, variant)
+    assert_parity(out.cpu(), ref, "f16", f"roberta B={B}/{variant}")
+
+
+def test_broadcast_over_tokens_is_accepted():
+    """expand()-ed inputs (stride 0 along N) are legal for the reference (it pads, i.e. copies); the
+    operator takes them too, by making the one copy the library's row-overlap check asks for."""
+    E, H, N, D, B, T = 1, 2, 64, 32, 16, 2
+    q, k, v = seeded_qkv(E, H, N, D, torch.float16)
+    kx = k[:, :, :1].expand(E, H, N, D)
+    ref = monarch_attention_oracle(q, kx, v, None, T, B, False, upcast=True)
+    qd, kd, vd = to_dev(q, k, v)
+    out = run_hip(qd, kd[:, :, :1].expand(E, H, N, D), vd, None, T, B, False, "auto")
+    assert_parity(out.cpu(), ref, "f16")
+
+
 # ---------------------------------------------------------------- stage-level parity (workspace state against the oracle trace)
 def _stage_setup(E, H, N, D, Dv, B, T, pre, dt, vdt, variant, with_mask):
     q, k, v = seeded_qkv(E, H, N, D, DT[dt], Dv=Dv)
@@ -325,15 +352,33 @@ def test_broadcast_keys_and_values(variant):
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
-@pytest.mark.parametrize("kind", ["bool", "int64", "float"])
+@pytest.mark.parametrize("kind", ["bool", "uint8", "int16", "int32", "int64", "float16", "bfloat16", "float32", "float64"])
 def test_mask_dtypes(kind, variant):
+    """The mask is read in place by the kernels, whatever its element type: truthy = keep, the way
+    torch.logical_and sees it (ma/ma_torch.py:98) - for floats -0.0 is false and NaN is true, for
+    wide integers a value with only high bits set is true.  Callers pass int64 tokenizer masks
+    (experiments/roberta/model.py:104-106) and float masks (experiments/bart/model.py:145-147)."""
     E, H, N, D, B, T = 2, 2, 384, 64, 32, 2
     q, k, v = seeded_qkv(E, H, N, D, torch.float16)
     keep = torch.arange(N)[None] < torch.tensor([N, N - 131])[:, None]
-    mask = dict(bool=keep, int64=keep.long(), float=keep.float())[kind]
-    ref = monarch_attention_oracle(q, k, v, mask, T, B, False, upcast=True)
+    dt = getattr(torch, kind)
+    mask = keep.to(dt)
+    if dt.is_floating_point:
+        mask[0, 5], mask[1, 7] = float("nan"), 0.25           # kept
+        mask[1, N - 100] = -0.0                                 # dropped, although its bits are not zero
+    elif kind == "int64":
+        mask[0, 5], mask[1, 7] = 1 << 40, -(1 << 35)           # kept: only high bits set
+    elif kind in ("int16", "int32"):
+        mask[0, 5], mask[1, 7] = -2, 1 << 9
+    ref = monarch_attention_oracle(q, k, v, mask != 0, T, B, False, upcast=True)
     out = run_hip(*to_dev(q, k, v, mask), T, B, False, variant)
     assert_parity(out.cpu(), ref, "f16")
+    # the same mask as a strided view (every other element of a wider buffer), still without a copy
+    wide = torch.zeros(E, 2 * N, dtype=dt)
+    wide[:, ::2] = mask
+    qd, kd, vd, wd = to_dev(q, k, v, wide)
+    out2 = run_hip(qd, kd, vd, wd[:, ::2], T, B, False, variant)
+    assert torch.equal(out2.view(torch.uint8), out.view(torch.uint8))
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
