@@ -150,7 +150,7 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
         constexpr int WPP = Split<NTM, W>::WPP, PPW = Split<NTM, W>::PPW;
         const int sub = wave / WPP, wig = wave % WPP;
         const int j = task * PPW + sub;
-        const bool active = j < P.B;
+        const bool active = sub < PPW && j < P.B;
         char* sm = smem + sub * Lds<T, DT, NTM>::Z;
         typename ZP::Pre pre;
         typename ZP::St st;
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
         constexpr int WPP = Split<NTM, W>::WPP, PPW = Split<NTM, W>::PPW;
         const int sub = wave / WPP, wig = wave % WPP;
         const int j = task * PPW + sub;
-        const bool active = j < P.B;
+        const bool active = sub < PPW && j < P.B;
         char* sm = smem + sub * Lds<T, DT, NTM>::L;
         typename LP::Pre pre;
         typename LP::St st;
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
         constexpr int WPP = Split<NTB, W>::WPP, PPW = Split<NTB, W>::PPW;
         const int sub = wave / WPP, wig = wave % WPP;
         const int m = task * PPW + sub;
-        const bool active = m < P.M;
+        const bool active = sub < PPW && m < P.M;
         const bool first = p == 0, with_v = p == nph - 2;
         char* sm = smem + sub * Lds<T, DT, NTB>::R;
         typename RP::Pre pre;

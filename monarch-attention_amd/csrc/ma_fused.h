@@ -205,7 +205,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, i
         bool first = true;
         for (int task = member; task < tasks || first; task += G) {
             const int j = task * PPW + slot;
-            const bool active = task < tasks && j < P.B;
+            const bool active = task < tasks && slot < PPW && j < P.B;
             typename ZP::Pre pre;
             typename ZP::St st;
             if (!ts.failed) ZP::issue(P, S, pre, active, active ? j : 0, wig, lane);
@@ -230,7 +230,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, i
         bool first = true;
         for (int task = member; task < tasks || first; task += G) {
             const int j = task * PPW + slot;
-            const bool active = task < tasks && j < P.B;
+            const bool active = task < tasks && slot < PPW && j < P.B;
             typename LP::Pre pre;
             typename LP::St st;
             if (!ts.failed) LP::issue(P, S, pre, active, e, active ? j : 0, wig, lane);
@@ -251,7 +251,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, i
         bool first = true;
         for (int task = member; task < tasks || first; task += G) {
             const int m = task * PPW + slot;
-            const bool active = task < tasks && m < P.M;
+            const bool active = task < tasks && slot < PPW && m < P.M;
             typename RP::Pre pre;
             typename RP::St st;
             if (!ts.failed) RP::issue(P, S, pre, active, e, active ? m : 0, first_step, with_v, wig, lane);

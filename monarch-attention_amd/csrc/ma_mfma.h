@@ -166,8 +166,8 @@ template <class T, int DT, int ROWS, int NTH>
 struct TileCopy {
     static constexpr int CH = Geom<DT>::COLS / 8;
     static constexpr int LD = Geom<DT>::LD;
-    static constexpr int CNT = ROWS * CH / NTH;
-    static_assert(ROWS * CH % NTH == 0, "tile chunks must divide evenly among the threads");
+    static constexpr int CNT = (ROWS * CH + NTH - 1) / NTH;
+    static constexpr bool EVEN = ROWS * CH % NTH == 0;   // else the last round of chunks is not for every thread
     u32x4 val[CNT];
 
     template <bool SHARED, class RowOff>
@@ -176,7 +176,7 @@ struct TileCopy {
         for (int i = 0; i < CNT; ++i) {
             const int c = tix + i * NTH;
             const int row = c / CH, ch = c % CH;
-            const unsigned ro = rowoff(row);
+            const unsigned ro = (EVEN || c < ROWS * CH) ? rowoff(row) : kOob;
             val[i] = bload16<SHARED>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
         }
     }
@@ -184,7 +184,7 @@ struct TileCopy {
 #pragma unroll
         for (int i = 0; i < CNT; ++i) {
             const int c = tix + i * NTH;
-            *reinterpret_cast<u32x4*>(tile + (c / CH) * LD + (c % CH) * 8) = val[i];
+            if (EVEN || c < ROWS * CH) *reinterpret_cast<u32x4*>(tile + (c / CH) * LD + (c % CH) * 8) = val[i];
         }
     }
 };
@@ -288,12 +288,16 @@ __device__ __forceinline__ void store_row(rsrc_t dst, unsigned ro, int D, const 
 }
 
 // How a workgroup's W waves are shared among block problems with NT strips:
-// WPP waves per problem (at most four), PPW problems per workgroup.
+// WPP waves per problem (at most four), PPW problems per workgroup.  Problems of 3 or 6 strips
+// (blocks and block counts of 33-48 / 81-96, e.g. the 48- and 96-token blocks of the reference's
+// RoBERTa sweep, experiments/roberta/benchmark.py:78) run on three waves: a per-stage launch uses
+// workgroups of three waves (WG), a one-launch kernel leaves its fourth wave idle in such a phase.
 template <int NT, int W = kWaves>
 struct Split {
-    static_assert(NT == 1 || NT == 2 || NT == 4 || NT == 8, "strip counts are rounded up to a power of two");
-    static constexpr int WPP = NT < kWaves ? NT : kWaves;
+    static_assert(NT == 1 || NT == 2 || NT == 3 || NT == 4 || NT == 6 || NT == 8, "strip counts are 1, 2, 3, 4, 6 or 8");
+    static constexpr int WPP = (NT == 3 || NT == 6) ? 3 : (NT < kWaves ? NT : kWaves);
     static constexpr int PPW = W / WPP;
+    static constexpr int WG = (NT == 3 || NT == 6) ? 3 : kWaves;   // waves of a per-stage launch's workgroup
 };
 
 // LDS bytes of one problem slot of each stage
@@ -875,9 +879,9 @@ __device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool act
 
 // ---- staged kernels: one launch per half step ---------------------------------
 template <class T, int DT, int NWT>
-__global__ __launch_bounds__(kThreads) void r_step_mfma(Problem P, int first, int with_v) {
+__global__ __launch_bounds__(64 * Split<NWT>::WG) void r_step_mfma(Problem P, int first, int with_v) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
+    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT, Split<NWT>::WG>::PPW;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
     // E * H * Np fits int32 (validated by the host), so all problem indices are 32-bit
@@ -894,9 +898,9 @@ __global__ __launch_bounds__(kThreads) void r_step_mfma(Problem P, int first, in
 }
 
 template <class T, int DT, int NWT>
-__global__ __launch_bounds__(kThreads) void l_step_mfma(Problem P) {
+__global__ __launch_bounds__(64 * Split<NWT>::WG) void l_step_mfma(Problem P) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
+    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT, Split<NWT>::WG>::PPW;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
     const unsigned total = static_cast<unsigned>(P.E) * P.H * P.B;
@@ -911,9 +915,9 @@ __global__ __launch_bounds__(kThreads) void l_step_mfma(Problem P) {
 }
 
 template <class T, int DT, int NWT>
-__global__ __launch_bounds__(kThreads) void z_step_mfma(Problem P) {
+__global__ __launch_bounds__(64 * Split<NWT>::WG) void z_step_mfma(Problem P) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT>::PPW;
+    constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT, Split<NWT>::WG>::PPW;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
     const unsigned total = static_cast<unsigned>(P.E) * P.H * P.B;

@@ -12,9 +12,14 @@ namespace ma {
 namespace mfma {
 
 inline int dt_class(int D) { return D <= 32 ? 2 : D <= 64 ? 4 : D <= 80 ? 5 : 8; }
+// the one-launch kernels are built for fewer classes: 96-row problems run as 128-row ones there
+inline int nt_class_one_launch(int n) {
+    const int t = (n + 15) / 16;
+    return t <= 4 ? (t < 1 ? 1 : t) : 8;
+}
 inline int nt_class(int n) {
     const int t = (n + 15) / 16;
-    return t <= 1 ? 1 : t <= 2 ? 2 : t <= 4 ? 4 : 8;
+    return t <= 4 ? (t < 1 ? 1 : t) : t <= 6 ? 6 : 8;
 }
 
 // Raises a kernel's dynamic-LDS limit to `bytes`, once per (kernel, device): the attribute belongs
@@ -44,7 +49,9 @@ int for_classes(int dt, int nt, F&& f) {
     switch (nt) {                                                                             \
         case 1: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 1>{}); \
         case 2: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 2>{}); \
+        case 3: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 3>{}); \
         case 4: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 4>{}); \
+        case 6: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 6>{}); \
         default: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 8>{}); \
     }
     switch (dt) {
@@ -60,12 +67,12 @@ template <class T>
 int launch_r(const Problem& P, bool first, bool with_v, hipStream_t s) {
     return for_classes(dt_class(P.D), nt_class(P.B), [&](auto dt, auto nt) {
         constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
-        constexpr int PPW = Split<NWT>::PPW;
+        constexpr int WG = Split<NWT>::WG, PPW = Split<NWT, WG>::PPW;
         constexpr size_t lds = PPW * Lds<T, DT, NWT>::R;
         const int attr = set_lds_limit(r_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
         const long long problems = static_cast<long long>(P.E) * P.H * P.M;
-        hipLaunchKernelGGL((r_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P,
+        hipLaunchKernelGGL((r_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(64 * WG), lds, s, P,
                            first ? 1 : 0, with_v ? 1 : 0);
         return static_cast<int>(hipGetLastError());
     });
@@ -75,12 +82,12 @@ template <class T>
 int launch_l(const Problem& P, hipStream_t s) {
     return for_classes(dt_class(P.D), nt_class(P.M), [&](auto dt, auto nt) {
         constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
-        constexpr int PPW = Split<NWT>::PPW;
+        constexpr int WG = Split<NWT>::WG, PPW = Split<NWT, WG>::PPW;
         constexpr size_t lds = PPW * Lds<T, DT, NWT>::L;
         const int attr = set_lds_limit(l_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
         const long long problems = static_cast<long long>(P.E) * P.H * P.B;
-        hipLaunchKernelGGL((l_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P);
+        hipLaunchKernelGGL((l_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(64 * WG), lds, s, P);
         return static_cast<int>(hipGetLastError());
     });
 }
@@ -89,12 +96,12 @@ template <class T>
 int launch_z(const Problem& P, hipStream_t s) {
     return for_classes(dt_class(P.D), nt_class(P.M), [&](auto dt, auto nt) {
         constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
-        constexpr int PPW = Split<NWT>::PPW;
+        constexpr int WG = Split<NWT>::WG, PPW = Split<NWT, WG>::PPW;
         constexpr size_t lds = PPW * Lds<T, DT, NWT>::Z;
         const int attr = set_lds_limit(z_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
         const long long problems = static_cast<long long>(P.E) * P.H * P.B;
-        hipLaunchKernelGGL((z_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(kThreads), lds, s, P);
+        hipLaunchKernelGGL((z_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(64 * WG), lds, s, P);
         return static_cast<int>(hipGetLastError());
     });
 }

@@ -66,7 +66,8 @@ int launch_resident_one(const Problem& P, bool dry_run, hipStream_t s) {
 template <class T, int DT>
 int launch_resident(const Problem& P, bool dry_run, hipStream_t s) {
     if (P.B > 64 || P.M > 64) return MA_ERR_UNSUPPORTED;
-    const int ntb = nt_class(P.B), ntm = nt_class(P.M);
+    // one strip per wave and whole tiles of 16, 32 or 64 rows: 48-row blocks run as 64-row ones here
+    const int ntb = nt_class(P.B) == 3 ? 4 : nt_class(P.B), ntm = nt_class(P.M) == 3 ? 4 : nt_class(P.M);
 #define MA_NTM(NB)                                                            \
     switch (ntm) {                                                            \
         case 1: return launch_resident_one<T, DT, NB, 1>(P, dry_run, s);      \

@@ -113,6 +113,9 @@ CONFIGS = [  # name, E, H, N, D, B, T, pre, dt, scale
     ("gps", 1, 2, 7600, 48, 128, 2, False, "f32", 1.0),
     ("vit_b14", 2, 12, 197, 64, 14, 2, True, "f16", 0.125),
     ("roberta_b24", 2, 12, 384, 64, 24, 1, False, "f16", 1.0),
+    ("b48_m40", 2, 4, 1900, 64, 48, 2, False, "f16", 1.0),         # 3-strip problems in both kinds of phases
+    ("b96_m90", 1, 2, 8600, 64, 96, 2, True, "bf16", 1.0),         # 6-strip problems (per-stage launches; 8-strip class in one launch)
+    ("b40_m6_d72", 2, 3, 230, 72, 40, 3, False, "f16", 1.0),       # 3 strips of keys, one of blocks, head dim 72
     ("big_block", 1, 2, 600, 64, 200, 2, False, "f16", 1.0),       # B > 128: beyond the MFMA tiles, AUTO -> generic
     ("many_blocks", 1, 2, 4096, 32, 16, 2, False, "bf16", 1.0),    # M = 256 > 128: AUTO -> generic
     ("one_block", 2, 2, 100, 64, 128, 3, True, "f16", 1.0),        # M = 1: dense softmax attention
