@@ -37,31 +37,20 @@ int launch_fused_w(const Problem& P, bool sync_ready, hipStream_t s) {
     using FL = FusedLds<T, DT, NTB, NTM, W>;
     if (FL::bytes > 160 * 1024) return MA_ERR_UNSUPPORTED;
     auto kernel = fused_fwd_mfma<T, DT, NTB, NTM, W>;
-    struct Caps {
-        int err = 0, capacity = 0;
-    };
     const int lds_err = set_lds_limit(kernel, FL::bytes);
     if (lds_err) return lds_err;
-    static const Caps caps = [&] {
-        Caps c;
-        int dev = 0, cus = 0, per_cu = 0;
-        if (!c.err) c.err = static_cast<int>(hipGetDevice(&dev));
-        if (!c.err) c.err = static_cast<int>(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        if (!c.err)
-            c.err = static_cast<int>(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), 64 * W, FL::bytes));
-        c.capacity = cus * per_cu;
-        return c;
-    }();
-    if (caps.err) return caps.err;
-    if (caps.capacity < 1) return MA_ERR_UNSUPPORTED;
+    const DeviceCaps dc = device_caps(kernel, 64 * W, FL::bytes);
+    if (dc.err) return dc.err;
+    const int capacity = dc.cus * dc.per_cu;
+    if (capacity < 1) return MA_ERR_UNSUPPORTED;
     const long long heads = static_cast<long long>(P.E) * P.H;
     const int tasks_r = (P.M + Split<NTB, W>::PPW - 1) / Split<NTB, W>::PPW;
     const int tasks_l = (P.B + Split<NTM, W>::PPW - 1) / Split<NTM, W>::PPW;
-    FusedPlan pl = plan_teams(heads, tasks_r, tasks_l, caps.capacity);
+    FusedPlan pl = plan_teams(heads, tasks_r, tasks_l, capacity);
     if (P.test_no_spin) pl.spin_limit = 0;
     // the grid must be co-resident (workgroups wait for each other) and the teams need their sync sectors
     if (pl.nteams < 1 || pl.G < 1 || pl.G > kMaxTeamSize) return MA_ERR_UNSUPPORTED;
-    if (static_cast<long long>(pl.nteams) * pl.G > caps.capacity) return MA_ERR_UNSUPPORTED;
+    if (static_cast<long long>(pl.nteams) * pl.G > capacity) return MA_ERR_UNSUPPORTED;
     if (pl.G > 1 && pl.nteams > kMaxTeams) return MA_ERR_UNSUPPORTED;
     if (!sync_ready) {
         const int err = launch_zero_sync(P.sync, s);

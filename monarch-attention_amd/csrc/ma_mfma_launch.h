@@ -4,6 +4,7 @@
 #pragma once
 
 #include <map>
+#include <utility>
 #include <mutex>
 
 #include "ma_mfma.h"
@@ -40,6 +41,30 @@ int set_lds_limit(K kernel, size_t bytes) {
     const int rc = static_cast<int>(hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
     if (rc == 0) mask |= bit;
     return rc;
+}
+
+// What the current device offers a kernel: its CU count and, when `threads` > 0, how many workgroups
+// of `threads` lanes and `lds` bytes a CU holds at once.  Looked up once per (kernel, device): a
+// process may drive devices that differ.
+struct DeviceCaps {
+    int err = 0, cus = 0, per_cu = 0;
+};
+template <class K>
+DeviceCaps device_caps(K kernel, int threads, size_t lds) {
+    static std::mutex mu;
+    static std::map<std::pair<const void*, int>, DeviceCaps> known;
+    DeviceCaps c;
+    int dev = 0;
+    c.err = static_cast<int>(hipGetDevice(&dev));
+    if (c.err) return c;
+    const void* key = reinterpret_cast<const void*>(kernel);
+    std::lock_guard<std::mutex> lock(mu);
+    const auto it = known.find({key, dev});
+    if (it != known.end()) return it->second;
+    c.err = static_cast<int>(hipDeviceGetAttribute(&c.cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (!c.err && threads > 0) c.err = static_cast<int>(hipOccupancyMaxActiveBlocksPerMultiprocessor(&c.per_cu, key, threads, lds));
+    if (!c.err) known[{key, dev}] = c;
+    return c;
 }
 
 // calls f(dt_tag, nt_tag) with integral_constant tags for the problem's classes

@@ -28,18 +28,9 @@ int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
     if (lds > kLdsPerCu) return MA_ERR_UNSUPPORTED;   // the head's state does not fit in LDS
     if (dry_run) return MA_OK;
     auto kernel = resident_fwd_mfma<T, DT, NTB, NTM, W>;
-    struct Caps {
-        int err = 0, cus = 0;
-    };
     const int lds_err = set_lds_limit(kernel, kLdsPerCu);
     if (lds_err) return lds_err;
-    static const Caps caps = [&] {
-        Caps c;
-        int dev = 0;
-        if (!c.err) c.err = static_cast<int>(hipGetDevice(&dev));
-        if (!c.err) c.err = static_cast<int>(hipDeviceGetAttribute(&c.cus, hipDeviceAttributeMultiprocessorCount, dev));
-        return c;
-    }();
+    const DeviceCaps caps = device_caps(kernel, 0, 0);
     if (caps.err) return caps.err;
     if (caps.cus < 1) return MA_ERR_DEVICE;
     // one workgroup per CU at a time when the state takes more than half the LDS, else two;
