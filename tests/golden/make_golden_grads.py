@@ -2,7 +2,7 @@
 
 Run ONCE, in the build container only (the reference tree does not travel):
 
-    python tests/golden/make_golden_grads.py [/root/reference]
+    python tests/golden/make_golden_grads.py [/root/reference [case-name ...]]
 
 The reference has no backward code of its own; training differentiates its
 pure-PyTorch forward (``ma/ma_torch.py``, ``monarch_attention_torch``) with
@@ -35,6 +35,8 @@ CASES = [  # name, E, H, N, D, Dv, B, T, pre, dtype, mask
     ("grad_f16_T2", 1, 2, 32, 32, 32, 8, 2, False, "f16", None),
     ("grad_f16_T3_mask_pre", 2, 1, 27, 16, 16, 4, 3, True, "f16", "safe"),
     ("grad_bf16_T2", 1, 2, 32, 32, 32, 8, 2, False, "bf16", "safe"),
+    # a long-document training shape (the BART recipe's block size): 64-row blocks on the matrix-core backward kernels
+    ("grad_bf16_T2_N512_b64", 1, 1, 512, 64, 64, 64, 2, False, "bf16", None),
 ]
 
 
@@ -43,7 +45,10 @@ def main():
     from ma.ma_torch import monarch_attention_torch  # the reference (namespace package)
 
     os.makedirs(OUT, exist_ok=True)
+    only = sys.argv[2:]
     for name, E, H, N, D, Dv, B, T, pre, dt, mk in CASES:
+        if only and name not in only:
+            continue
         gen = torch.Generator().manual_seed(0)
         q = torch.randn(E, H, N, D, generator=gen).to(DT[dt]).requires_grad_()
         k = torch.randn(E, H, N, D, generator=gen).to(DT[dt]).requires_grad_()
@@ -63,7 +68,7 @@ def main():
         if mask is not None:
             arrays["mask"] = mask.numpy()
         np.savez_compressed(os.path.join(OUT, name + ".npz"), **arrays)
-    print(f"wrote {len(CASES)} gradient fixtures to {OUT}")
+    print(f"wrote {len(only) or len(CASES)} gradient fixtures to {OUT}")
 
 
 if __name__ == "__main__":

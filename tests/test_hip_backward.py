@@ -3,9 +3,10 @@ gradients autograd yields through the reference / the CPU oracle.  Runs on a
 MI355X only (``-m gpu``).
 
 Gate: fp32 relative Frobenius error <= 1e-4 per gradient (and max-abs <= 1e-4
-of the gradient's largest entry); fp16 / bf16 <= 3e-2 relative: the reference's
-autograd rounds every intermediate gradient to the operand dtype, the HIP
-backward keeps fp32 between its kernels and rounds once at the end.
+of the gradient's largest entry); fp16 <= 4e-3 (max-abs 8e-3), bf16 <= 1.5e-2
+(max-abs 3e-2) - a few units of the operand type's rounding step (2^-10, 2^-7):
+the reference's autograd rounds every intermediate gradient to the operand
+dtype, the HIP backward keeps fp32 between its kernels and rounds once at the end.
 """
 import pytest
 import torch
@@ -31,14 +32,14 @@ def oracle_grads(q, k, v, mask, w, T, B, pre):
 
 
 def assert_grads(got, ref, dt, what=""):
-    tol = 1e-4 if dt == "f32" else 3e-2
+    tol, tol_max = {"f32": (1e-4, 1e-4), "f16": (4e-3, 8e-3), "bf16": (1.5e-2, 3e-2)}[dt]
     for x, r, name in zip(got, ref, ("dq", "dk", "dv")):
         x, r = x.detach().double().cpu(), r.detach().double().cpu()
         assert x.shape == r.shape
         assert torch.isfinite(x).all(), (what, name)
         rel = ((x - r).norm() / r.norm().clamp(min=1e-30)).item()
         mx = ((x - r).abs().max() / r.abs().max().clamp(min=1e-30)).item()
-        assert rel <= tol and mx <= (1e-4 if dt == "f32" else 6e-2), (what, name, rel, mx)
+        assert rel <= tol and mx <= tol_max, (what, name, rel, mx)
 
 
 @pytest.mark.parametrize("variant", ["generic", "auto"])
