@@ -146,6 +146,8 @@ def main():
     ap.add_argument("--config", default="cM", choices=sorted(CONFIGS))
     ap.add_argument("--T", type=int, default=None, help="override the number of alternating steps")
     ap.add_argument("--variant", default="auto", choices=["auto", "generic", "staged", "fused", "resident", "chained"])
+    ap.add_argument("--rotate-workspaces", action="store_true",
+                    help="a workspace per input set (default: all sets share one, like the calls of a model)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sdpa", action="store_true", help="skip the dense SDPA comparison")
     ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep over the variants")
@@ -270,13 +272,18 @@ def main():
         q, k, v = (t.to(dev).roll(i, dims=2).contiguous() for t in base)   # distinct addresses and contents
         sets.append((q, k, v, torch.empty(E, H, N, D, dtype=dtype, device=dev)))
 
-    def prepared(T_, variant):
-        """One ma_fwd_params per buffer set, all on one zero-initialised workspace."""
+    def prepared(T_, variant, rotate=None):
+        """One ma_fwd_params per buffer set.  All sets share ONE zero-initialised workspace, as the
+        calls of a model do (the host wrapper keeps one per device and stream), so the state arrays
+        can stay in the 256 MB Infinity Cache between calls; with `rotate` every set has a workspace of
+        its own (as long as they total at most 2 GiB) and the state rotates through memory like the inputs."""
         ps = [make_params(q, k, v, None, o, T_, B, False, variant) for (q, k, v, o) in sets]
         nbytes = lib.ma_fwd_workspace_bytes(ps[0])
-        ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
-        for p in ps:
-            p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), nbytes, L.MA_FLAG_SYNC_READY
+        rotate = args.rotate_workspaces if rotate is None else rotate
+        nws = max(1, min(nbuf, (2 << 30) // max(nbytes, 1))) if rotate else 1
+        ws = [torch.zeros(nbytes, dtype=torch.uint8, device=dev) for _ in range(nws)]
+        for i, p in enumerate(ps):
+            p.workspace, p.workspace_bytes, p.flags = ws[i % nws].data_ptr(), nbytes, L.MA_FLAG_SYNC_READY
         return ps, ws
 
     def run_steps(ps, n):
@@ -286,9 +293,9 @@ def main():
             if st:
                 L.check(st, "ma_fwd")
 
-    def time_forward(T_, variant, steps, warmup):
-        ps, ws = prepared(T_, variant)
-        run_steps(ps, warmup)
+    def time_forward(T_, variant, steps, warmup, rotate=None):
+        ps, ws = prepared(T_, variant, rotate)
+        run_steps(ps, max(warmup, nbuf))
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
@@ -396,13 +403,18 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dt, "data": "synthetic",
         "config": {"workload": f"{args.config}: {dt} E{E} H{H} N{N} D{D} block{B} T{T} post-pad no-mask", "variant": resolved,
-                   "flop_per_fwd": flops, "compulsory_bytes_per_fwd": cbytes, "rotating_input_sets": nbuf},
+                   "flop_per_fwd": flops, "compulsory_bytes_per_fwd": cbytes, "rotating_input_sets": nbuf, "rotating_workspaces": len(ws)},
         "stream_ms_per_step": round(ev_ms, 5),
         "ms_per_step_stats": timing,
         "fwd_hbm_frac": round(cbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "fwd_mfma_frac": round(flops / (ev_ms * 1e-3) / 1e12 / mfma_peak, 5),
         "roofline": roofline,
     }
+    del ps, ws
+    # the same K steps with a workspace per input set: what the Infinity Cache contributes to the state exchange
+    _, rot_ms, ps, ws = time_forward(T, args.variant, max(args.steps, 100), max(args.warmup, 10), rotate=True)
+    out["stream_ms_per_step_rotating_workspaces"] = round(rot_ms, 5)
+    out["config"]["rotating_workspaces_in_that_run"] = len(ws)
     del ps, ws
 
     # ---- the same forward through the nn.Module-level host wrapper (allocates its output per call)
@@ -423,7 +435,7 @@ def main():
         by_T = []
         for T_ in (1, 2, 3):
             ps_, ws_ = prepared(T_, args.variant)
-            run_steps(ps_, 10)
+            run_steps(ps_, max(10, nbuf))   # every workspace holds the state of a full forward
             by_T.append(roofline_of(T_, args.variant, ps_, 100))
             del ps_, ws_
         out["roofline_by_T"] = by_T
