@@ -60,12 +60,19 @@ typedef enum ma_variant {
     MA_VARIANT_GENERIC = 1, /* FMA kernels, 2T(+T-1) launches: any dtype/shape/stride */
     MA_VARIANT_STAGED = 2,  /* MFMA kernels, one launch per half step (2T launches)  */
     MA_VARIANT_FUSED = 3,   /* MFMA, all T steps in ONE launch, teams of workgroups  */
-                            /* per head, state exchanged through the workspace       */
+                            /* per head, state exchanged through the workspace.  Its */
+                            /* workgroups wait for each other, so the grid is sized  */
+                            /* to what the device holds at once when idle: a kernel  */
+                            /* of another stream that occupies compute units for     */
+                            /* longer than the bounded waits (about a millisecond)   */
+                            /* makes the call fail loudly (NaN rows + error word)    */
     MA_VARIANT_RESIDENT = 4,/* MFMA, ONE launch, one workgroup per head with the     */
                             /* whole per-head state resident in LDS (small heads)    */
     MA_VARIANT_CHAINED = 5  /* MFMA, ONE launch, one workgroup per block problem of  */
                             /* every phase; a problem starts when its head's         */
-                            /* previous phase has raised its flags in the workspace  */
+                            /* previous phase has released it through the workspace. */
+                            /* Producers are always dispatched before consumers: no  */
+                            /* co-residency requirement, safe beside other kernels   */
 } ma_variant;
 
 typedef enum ma_status {
