@@ -31,9 +31,11 @@
 // consumer on another XCD than its producers cannot rely on what it reads: it
 // raises the sync area's error word (2) and treats the phase as failed.
 //
-// The state arrays are the per-head ones of the staged variant.  The last Z task
-// of a head to finish (a counter per head) clears the head's words, so the area
-// is zero again when the launch is over.  Every wait is bounded (spin_limit
+// The state arrays are the per-head ones of the staged variant.  Every task
+// counts itself as finished once its arrival (and release) has been performed;
+// the task of a head that finishes last - normally a Z task, but tasks whose wait
+// ran out do not run in phase order - clears the head's words, so the area is
+// zero again when the launch is over, also after a failed one.  Every wait is bounded (spin_limit
 // polls).  A task that gives up - or whose producers failed - raises the error
 // word, computes nothing, still counts itself in (marked as failed, which its
 // consumers inherit), and as a Z task writes NaN into the output rows it owns: a
@@ -57,7 +59,7 @@ constexpr int kChainWords = 256 * 1024;   // sync words of the chained kernel, b
 static_assert(static_cast<uint64_t>(kSyncWords + kChainWords) * 4 == kSyncAreaBytes, "sync area size mismatch");
 
 // A head's sync words: 64-bit arrival counters of the 2T-1 publishing phases and the 64-bit counter
-// of finished Z tasks, rounded up to whole 128-byte lines; then one release word per publishing
+// of finished tasks, rounded up to whole 128-byte lines; then one release word per publishing
 // phase, rounded up likewise.
 __host__ __device__ inline int chain_go_offset(int T) { return (2 * (2 * T - 1) + 2 + 31) / 32 * 32; }
 __host__ __device__ inline int chain_stride(int T) { return chain_go_offset(T) + ((2 * T - 1) + 31) / 32 * 32; }
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
     const int e = static_cast<unsigned>(head) / static_cast<unsigned>(P.H), h = static_cast<unsigned>(head) % static_cast<unsigned>(P.H);
 
     unsigned* words = P.sync + kSyncWords + static_cast<size_t>(head) * plan.stride;   // this head's sync words
-    unsigned long long* count = reinterpret_cast<unsigned long long*>(words);        // [phase] arrivals, [2T-1] finished Z tasks
+    unsigned long long* count = reinterpret_cast<unsigned long long*>(words);        // [phase] arrivals, [2T-1] finished tasks of all phases
     unsigned* go = words + plan.go_off;                                               // [phase] release word
     unsigned* error = P.sync + 1;
     const unsigned prev_count = odd ? plan.tR : plan.tL;   // tasks of the previous phase (p > 0)
@@ -196,23 +198,24 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
     // every wave's stores have reached L2 before the task is published
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (p < nph - 1) {
-        if (threadIdx.x == 0) {
+    if (threadIdx.x == 0) {
+        if (p < nph - 1) {
             const unsigned long long mine = arrival_of(my_xcc, failed);
             const unsigned long long before = __hip_atomic_fetch_add(count + p, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (((before + mine) & 0xffffull) == tasks)   // this add completes the phase: release its consumers
                 __hip_atomic_store(go + p, release_of(before + mine, tasks), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // the arrival and the release have been performed before this task counts as finished
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
-    } else {
-        // Z tasks: the last one of the head to finish clears the head's words
-        if (threadIdx.x == 0) {
-            const unsigned long long before = __hip_atomic_fetch_add(count + (nph - 1), 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            wg_word = before + 1ull == static_cast<unsigned long long>(plan.tL) ? 2u : 0u;
-        }
-        __syncthreads();
-        if (wg_word == 2u)
-            for (int i = threadIdx.x; i < plan.stride; i += 64 * W) __hip_atomic_store(words + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // The task of the head that finishes LAST - of any phase: tasks whose wait ran out do not run in
+        // phase order - clears the head's words; nothing of this head touches them after that.
+        const unsigned long long all = static_cast<unsigned long long>(P.T) * (plan.tR + plan.tL);
+        const unsigned long long done = __hip_atomic_fetch_add(count + (nph - 1), 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        wg_word = done + 1ull == all ? 2u : 0u;
     }
+    __syncthreads();
+    if (wg_word == 2u)
+        for (int i = threadIdx.x; i < plan.stride; i += 64 * W) __hip_atomic_store(words + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace mfma

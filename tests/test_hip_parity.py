@@ -569,14 +569,17 @@ def test_random_shapes_every_variant(idx, E, H, N, D, B, T, pre, dt, masked):
 
 
 # ---------------------------------------------------------------- a wait between workgroups that runs out is loud
+@pytest.mark.parametrize("shape", [(1, 2, 1024, 64, 32, 2), (3, 8, 512, 64, 32, 3), (1, 16, 2048, 64, 64, 1)])
 @pytest.mark.parametrize("variant", ["fused", "chained"])
-def test_wait_that_runs_out_is_loud_and_leaves_the_workspace_usable(variant):
+def test_wait_that_runs_out_is_loud_and_leaves_the_workspace_usable(variant, shape):
     """MA_FLAG_TEST_NO_SPIN makes every wait of the one-launch kernels give up at once (forced from the
     host; every kernel still runs to its end).  The call must then raise the sticky error word and
     write NaN rows instead of results computed from a state that may be incomplete, and the next
-    call on the same workspace must be an ordinary, correct one."""
+    call on the same workspace must be an ordinary, correct one.  Tasks that do not wait run in no
+    particular order, so the failed call is repeated: whatever order they finish in, the sync area
+    must come out consistent."""
     lib = L.load()
-    E, H, N, D, B, T = 1, 2, 1024, 64, 32, 2
+    E, H, N, D, B, T = shape
     q, k, v = to_dev(*seeded_qkv(E, H, N, D, torch.float16, seed=3))
     want = monarch_attention_oracle(q.cpu(), k.cpu(), v.cpu(), None, T, B, False)
     out = torch.zeros_like(v)
@@ -593,21 +596,23 @@ def test_wait_that_runs_out_is_loud_and_leaves_the_workspace_usable(variant):
     assert int(word.item()) == 0
     assert_parity(out.cpu(), want, "f16", f"{variant} before")
 
-    out.zero_()
-    p.flags = L.MA_FLAG_SYNC_READY | L.MA_FLAG_TEST_NO_SPIN
-    L.check(lib.ma_fwd(p, stream), "ma_fwd")
-    torch.cuda.synchronize()
-    assert int(word.item()) == 1, "the wait that ran out was not reported"
-    assert torch.isnan(out.float()).any(dim=-1).all(), "every output row depends on a wait that gave up: all must be NaN"
+    for rep in range(4):
+        out.zero_()
+        p.flags = L.MA_FLAG_SYNC_READY | L.MA_FLAG_TEST_NO_SPIN
+        for _ in range(1 + rep % 2):   # also two failed calls back to back
+            L.check(lib.ma_fwd(p, stream), "ma_fwd")
+        torch.cuda.synchronize()
+        assert int(word.item()) == 1, "the wait that ran out was not reported"
+        assert torch.isnan(out.float()).any(dim=-1).all(), "every output row depends on a wait that gave up: all must be NaN"
 
-    word.zero_()
-    out.zero_()
-    p.flags = L.MA_FLAG_SYNC_READY   # no clearing of the sync area: the failed call must have left it consistent
-    for _ in range(2):
-        L.check(lib.ma_fwd(p, stream), "ma_fwd")
-    torch.cuda.synchronize()
-    assert int(word.item()) == 0
-    assert_parity(out.cpu(), want, "f16", f"{variant} after")
+        word.zero_()
+        out.zero_()
+        p.flags = L.MA_FLAG_SYNC_READY   # no clearing of the sync area: the failed call must have left it consistent
+        for _ in range(2):
+            L.check(lib.ma_fwd(p, stream), "ma_fwd")
+        torch.cuda.synchronize()
+        assert int(word.item()) == 0
+        assert_parity(out.cpu(), want, "f16", f"{variant} after failed call {rep}")
 
 
 def test_module_reports_a_failed_call_at_a_later_call(monkeypatch):
