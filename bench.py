@@ -411,11 +411,6 @@ def main():
         "roofline": roofline,
     }
     del ps, ws
-    # the same K steps with a workspace per input set: what the Infinity Cache contributes to the state exchange
-    _, rot_ms, ps, ws = time_forward(T, args.variant, max(args.steps, 100), max(args.warmup, 10), rotate=True)
-    out["stream_ms_per_step_rotating_workspaces"] = round(rot_ms, 5)
-    out["config"]["rotating_workspaces_in_that_run"] = len(ws)
-    del ps, ws
 
     # ---- the same forward through the nn.Module-level host wrapper (allocates its output per call)
     q0, k0, v0, _ = sets[0]
@@ -432,6 +427,11 @@ def main():
 
     # ---- T = 1, 2, 3 with the selected variant: one roofline entry each; and every variant (same protocol, fewer steps)
     if not args.no_sweep:
+        # the same K steps with a workspace per input set: what the Infinity Cache contributes to the state exchange
+        _, rot_ms, ps, ws = time_forward(T, args.variant, max(args.steps, 100), max(args.warmup, 10), rotate=True)
+        out["stream_ms_per_step_rotating_workspaces"] = round(rot_ms, 5)
+        out["config"]["rotating_workspaces_in_that_run"] = len(ws)
+        del ps, ws
         by_T = []
         for T_ in (1, 2, 3):
             ps_, ws_ = prepared(T_, args.variant)
