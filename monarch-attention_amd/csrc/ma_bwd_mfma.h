@@ -1258,6 +1258,8 @@ __global__ void add_parts_kernel(float* dst, const float* part, long long n, int
 // threads per workgroup for a stage whose probability matrix has `tiles` 16 x 16 tiles
 int threads_for(int tiles) { return tiles <= 2 ? 64 : tiles <= 8 ? 256 : 1024; }
 
+#include "ma_bwd_reg.h"
+
 template <class T>
 constexpr int dtype_of() { return sizeof(T) == 4 ? MA_F32 : std::is_same<T, f16>::value ? MA_F16 : MA_BF16; }
 
@@ -1336,11 +1338,17 @@ int launch_r_t(const Problem& P, const BwdBuffers& G0, bool first, bool with_v, 
     auto bytes = [&](int t) -> size_t {
         return k32 ? r_layout<TQ>(P.B, P.D, P.Dv, with_v, t).total : r_layout16(P.B, P.D, P.Dv, with_v, t).total;
     };
+    // the partial buffers are sized for the tiling of the step that also forms dv (the smallest tile)
+    const int parts = G0.pk != nullptr ? r_split_tiles(P, dt_qk, dt_qk) : 0;
+    if constexpr (!k32) {   // 16-bit operands: the register kernel where it applies
+        if (parts <= 1) {
+            const int st = launch_r_reg<TQ>(P, G0, first, with_v, s);
+            if (st != static_cast<int>(MA_ERR_UNSUPPORTED)) return st;
+        }
+    }
     int TJ = pick_tile(P.B, bytes);
     if (TJ == 0) return static_cast<int>(MA_ERR_UNSUPPORTED);
     BwdBuffers G = G0;
-    // the partial buffers are sized for the tiling of the step that also forms dv (the smallest tile)
-    const int parts = G.pk != nullptr ? r_split_tiles(P, dt_qk, dt_qk) : 0;
     G.jt_split = 0;
     if (parts > 1) {
         TJ = min(TJ, r_tile(P, dt_qk, true));

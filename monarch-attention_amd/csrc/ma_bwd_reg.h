@@ -1,0 +1,312 @@
+// Backward R stage for fp16 / bf16 operands with the probabilities and their
+// gradients kept in MFMA accumulator registers, the way the forward stages keep
+// theirs (ma_mfma.h): no fp32 matrices in LDS, no LDS round trip between the
+// products.  Included by ma_bwd_mfma.h inside namespace ma::{anonymous}; the
+// formulas are at the top of ma_bwd.hip, the reference is autograd through
+// al_cl_ref / al_y_cl_ref (ma/ma_torch.py:10-23, :38-52).
+//
+// One workgroup per block problem (e, h, k), one wave per 16-row strip.  LDS holds
+// five 16-bit operand tiles - K, V, X (aR rows, or Q rows in the first step),
+// Ga = round(sm * gaL), Gy = round(gY) - and seven floats per row.  The products
+// of the stage contract over three different indices, and a lane of the 16x16x32
+// instruction can only feed a B operand from accumulators whose ROWS are the
+// contraction index.  So the stage runs in two passes over the same logits:
+//
+//   pass 1, wave = strip of QUERY rows j (accumulator rows = keys i):
+//     S = X K^T, Gg = Ga K^T + Gy V^T  ->  r, g, dS, dDot in registers;
+//     gaR[j] = sum_i dDot[j,i] K[i]  (dDot straight into the B operand),
+//     gcR[j]; the row statistics (max, 1 / sum, sum_i g r, ...) go to LDS.
+//   pass 2, wave = strip of KEYS i (accumulator rows = query rows j):
+//     the same two products with the operand roles swapped, r and dDot formed
+//     again from the row statistics of pass 1;
+//     dK[i] += sum_j r[j,i] Ga[j] + dDot[j,i] X[j],  dV[i] = sum_j r[j,i] Gy[j].
+//
+// The recomputation costs four more small products on matrix pipes that are
+// otherwise idle and the softmax arithmetic a second time; it saves three fp32
+// B x B matrices in LDS (the tiles of a 64-row block take 46 KB instead of 150 KB,
+// so three workgroups share a compute unit) and every pass over them.
+// Rounding points are those of the LDS kernels: logits rounded to the operand
+// dtype, probabilities, dDot, sm * gaL and gY rounded to it as operands.
+
+template <class T, int DT, int NWT>
+struct RBwdReg {
+    using Gm = mfma::Geom<DT>;
+    static constexpr int ROWS = 16 * NWT, LD = Gm::LD, KS = Gm::KS, COLS = Gm::COLS, TILE = ROWS * LD;
+    static constexpr int kStats = 7;   // kok, cj, gcl, mx, inv, lg1, dot
+    static constexpr size_t kLds = 5 * static_cast<size_t>(TILE) * sizeof(T) + kStats * ROWS * sizeof(float);
+};
+
+// O[dt] += sum_w tile[w][4*DT*q + 4*dt + v] * P[w][lane column]   (gemm2 of ma_mfma.h, accumulating)
+template <class T, int DT, int NWT>
+__device__ __forceinline__ void gemm2_acc(f32x4 (&O)[DT], const T* tile, const typename mfma::Ops<T>::v8 (&pb)[(NWT + 1) / 2], int r, int q) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int g = 0; g < (NWT + 1) / 2; ++g)
+            O[dt] = mfma::Ops<T>::mma(mfma::lds_tr8<T, DT>(tile, 32 * g + 4 * q, 16, 2 * g + 1 < NWT, dt, r), pb[g], O[dt]);
+}
+
+template <class T, int DT, int NWT, bool S16>
+__global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, int first, int with_v) {
+    using mfma::lds_row8;
+    using mfma::quad_rows_max;
+    using mfma::quad_rows_sum;
+    using RB = RBwdReg<T, DT, NWT>;
+    using TG = typename std::conditional<S16, T, float>::type;
+    using V8 = typename mfma::Ops<T>::v8;
+    using V4 = typename mfma::Ops<T>::v4;
+    using MM = mfma::Ops<T>;
+    constexpr int NTH = 64 * NWT, ROWS = RB::ROWS, LD = RB::LD, KS = RB::KS, COLS = RB::COLS, TILE = RB::TILE;
+    constexpr float kLog2e = mfma::kLog2e;
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+    T* Kt = reinterpret_cast<T*>(lds_raw);
+    T* Vt = Kt + TILE;
+    T* Xt = Vt + TILE;
+    T* Gat = Xt + TILE;
+    T* Gyt = Gat + TILE;
+    float* kok = reinterpret_cast<float*>(Gyt + TILE);
+    float* cjs = kok + ROWS;
+    float* gcls = cjs + ROWS;
+    float* mxs = gcls + ROWS;
+    float* invs = mxs + ROWS;
+    float* lg1s = invs + ROWS;
+    float* dots = lg1s + ROWS;
+
+    const int B = P.B, M = P.M, D = P.D;
+    int w = blockIdx.x;
+    const int k = w % M; w /= M;
+    const int h = w % P.H, e = w / P.H;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const long long blk = (eh * M + k) * B;   // first row of block k in the (E,H,M,B,.) arrays
+    const float sm = P.sm_scale;
+    const int wave = mfma::wave_id(), lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+
+    // ---- operand tiles, zero-padded to the tile grid
+    {
+        const T* aR = reinterpret_cast<const T*>(P.aR) + blk * D;
+        const TG* gaL = reinterpret_cast<const TG*>(G.gaL);
+        const TG* gY = reinterpret_cast<const TG*>(G.gY);
+        auto k_row = [=](int i) { return i < B ? tok_row<T>(P.k, P.ks, e, h, k * B + i - P.pad_off, P.N) : nullptr; };
+        auto v_row = [=](int i) { return i < B ? tok_row<T>(P.v, P.vs, e, h, k * B + i - P.pad_off, P.N) : nullptr; };
+        auto x_row = [=](int j) -> const T* {
+            if (j >= B) return nullptr;
+            return first ? tok_row<T>(P.q, P.qs, e, h, k * B + j - P.pad_off, P.N) : aR + j * D;
+        };
+        auto ga_row = [=](int j) { return j < B ? gaL + ((eh * B + j) * M + k) * D : nullptr; };
+        auto gy_row = [=](int j) { return j < B ? gY + ((eh * B + j) * M + k) * D : nullptr; };
+        stage_rows<NTH, T, T>(Kt, LD, ROWS, COLS, D, 1.f, k_row);
+        stage_rows<NTH, T, T>(Xt, LD, ROWS, COLS, D, 1.f, x_row);
+        stage_rows<NTH, TG, T>(Gat, LD, ROWS, COLS, D, sm, ga_row);
+        if (with_v) {
+            stage_rows<NTH, T, T>(Vt, LD, ROWS, COLS, D, 1.f, v_row);
+            stage_rows<NTH, TG, T>(Gyt, LD, ROWS, COLS, D, 1.f, gy_row);
+        }
+        const float* cR = P.cR + blk;
+        for (int i = threadIdx.x; i < ROWS; i += NTH) {
+            const bool in = i < B;
+            kok[i] = (in && token_ok(P, e, k * B + i - P.pad_off)) ? 1.f : 0.f;
+            cjs[i] = 1.0f / (((first || !in) ? 1.0f : cR[i]) + P.eps);   // 1 / (cR + eps)
+            gcls[i] = in ? G.gcL[(eh * B + i) * M + k] : 0.f;
+        }
+    }
+    __syncthreads();
+
+    // Probability r (clamped, ma_torch.py:18) and gradient g of one entry from its logit sv (-inf:
+    // masked key), the gradient part gg = (sm gaL K^T + gY V^T) and its row's statistics.  g is 0
+    // where the clamp acted; log r = (S - max) + log(1 / (sum + eps)).
+    auto prob_grad = [](float sv, float gg, bool key_in, float gcl, float mx, float inv, float lg1, float& rc, float& g) {
+        const float d = sv - mx;
+        const float ru = __builtin_amdgcn_exp2f(kLog2e * d) * inv;
+        rc = key_in ? fmaxf(ru, kTiny) : 0.f;
+        g = (key_in && ru >= kTiny) ? fmaf(gcl, d + lg1, gg) : 0.f;
+    };
+
+    // ---- pass 1: this wave's strip of query rows (accumulator rows = keys)
+    {
+        const int j = 16 * wave + r;
+        const bool jv = j < B;
+        V8 xb[KS], ga[KS], gy[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            xb[ks] = lds_row8<T>(Xt + j * LD + 32 * ks + 8 * q);
+            ga[ks] = lds_row8<T>(Gat + j * LD + 32 * ks + 8 * q);
+            if (with_v) gy[ks] = lds_row8<T>(Gyt + j * LD + 32 * ks + 8 * q);
+        }
+        const float cj = cjs[j], gcl = gcls[j];
+        f32x4 S[NWT], Gg[NWT];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int wt = 0; wt < NWT; ++wt) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, g = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const V8 kr = lds_row8<T>(Kt + (16 * wt + r) * LD + 32 * ks + 8 * q);
+                a = MM::mma(kr, xb[ks], a);
+                g = MM::mma(kr, ga[ks], g);
+                if (with_v) g = MM::mma(lds_row8<T>(Vt + (16 * wt + r) * LD + 32 * ks + 8 * q), gy[ks], g);
+            }
+            const f32x4 ok = *reinterpret_cast<const f32x4*>(kok + 16 * wt + 4 * q);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                a[v] = ok[v] != 0.f ? sm * round_to<T>(a[v]) * cj : -INFINITY;   // S, -inf for masked / padded keys
+                mx = fmaxf(mx, a[v]);
+            }
+            S[wt] = a;
+            Gg[wt] = g;
+        }
+        // row statistics: clamped maximum, 1 / (sum + eps)   (ma_torch.py:14-17)
+        mx = fmaxf(quad_rows_max(mx), P.eps);
+        float sum = 0.f;
+#pragma unroll
+        for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) sum += __builtin_amdgcn_exp2f(kLog2e * (S[wt][v] - mx));
+        const float inv = mfma::rcp(quad_rows_sum(sum) + P.eps);
+        const float lg1 = __logf(inv) + 1.0f;
+        f32x4 Rc[NWT];
+        float dot = 0.f;   // sum_i g r
+#pragma unroll
+        for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float rc, g;
+                prob_grad(S[wt][v], Gg[wt][v], 16 * wt + 4 * q + v < B, gcl, mx, inv, lg1, rc, g);
+                Rc[wt][v] = rc;
+                Gg[wt][v] = g;
+                dot = fmaf(g, rc, dot);
+            }
+        dot = quad_rows_sum(dot);
+        // dS = r (g - dot), gcR = -sum_i dS S / (cR + eps), dDot = dS sm / (cR + eps)
+        float gc = 0.f;
+#pragma unroll
+        for (int wt = 0; wt < NWT; ++wt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const bool live = S[wt][v] != -INFINITY;
+                const float ds = live ? Rc[wt][v] * (Gg[wt][v] - dot) : 0.f;
+                gc = live ? fmaf(-ds, S[wt][v] * cj, gc) : gc;
+                Rc[wt][v] = ds * (sm * cj);
+            }
+        gc = quad_rows_sum(gc);
+        if (q == 0) {
+            mxs[j] = mx;
+            invs[j] = inv;
+            lg1s[j] = lg1;
+            dots[j] = dot;
+            if (!first && jv) G.gcR[blk + j] = gc;
+        }
+        // gaR[j] = sum_i dDot[j,i] K[i]   (first step: aR is q, the rows of block k of dq)
+        V8 pb[(NWT + 1) / 2];
+        mfma::pack_p<T, NWT>(pb, Rc);
+        f32x4 O[DT];
+        mfma::gemm2<T, DT, NWT>(O, Kt, pb, r, q);
+        if (jv) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d0 = 4 * DT * q + 4 * dt;
+                if (d0 >= D) continue;   // D is a multiple of 4 (checked by the launcher)
+                if (first) {
+                    f32x4* dst = reinterpret_cast<f32x4*>(G.dq + (blk + j) * D + d0);
+                    *dst = *dst + O[dt];
+                } else if (S16) {
+                    const V4 o = {from_f<T>(O[dt][0]), from_f<T>(O[dt][1]), from_f<T>(O[dt][2]), from_f<T>(O[dt][3])};
+                    *reinterpret_cast<V4*>(reinterpret_cast<T*>(G.gaR) + (blk + j) * D + d0) = o;
+                } else {
+                    *reinterpret_cast<f32x4*>(G.gaR + (blk + j) * D + d0) = O[dt];
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- pass 2: this wave's strip of keys (accumulator rows = query rows)
+    {
+        const int i = 16 * wave + r;
+        const bool key_in = i < B, key_ok = kok[i] != 0.f;
+        V8 kb[KS], vb[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            kb[ks] = lds_row8<T>(Kt + i * LD + 32 * ks + 8 * q);
+            if (with_v) vb[ks] = lds_row8<T>(Vt + i * LD + 32 * ks + 8 * q);
+        }
+        f32x4 PR[NWT], DD[NWT];
+#pragma unroll
+        for (int jt = 0; jt < NWT; ++jt) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, g = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                a = MM::mma(lds_row8<T>(Xt + (16 * jt + r) * LD + 32 * ks + 8 * q), kb[ks], a);
+                g = MM::mma(lds_row8<T>(Gat + (16 * jt + r) * LD + 32 * ks + 8 * q), kb[ks], g);
+                if (with_v) g = MM::mma(lds_row8<T>(Gyt + (16 * jt + r) * LD + 32 * ks + 8 * q), vb[ks], g);
+            }
+            const int j0 = 16 * jt + 4 * q;
+            const f32x4 cj4 = *reinterpret_cast<const f32x4*>(cjs + j0), gcl4 = *reinterpret_cast<const f32x4*>(gcls + j0);
+            const f32x4 mx4 = *reinterpret_cast<const f32x4*>(mxs + j0), inv4 = *reinterpret_cast<const f32x4*>(invs + j0);
+            const f32x4 lg4 = *reinterpret_cast<const f32x4*>(lg1s + j0), dot4 = *reinterpret_cast<const f32x4*>(dots + j0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float sv = key_ok ? sm * round_to<T>(a[v]) * cj4[v] : -INFINITY;
+                float rc, gv;
+                prob_grad(sv, g[v], key_in, gcl4[v], mx4[v], inv4[v], lg4[v], rc, gv);
+                PR[jt][v] = rc;
+                DD[jt][v] = key_ok ? rc * (gv - dot4[v]) * (sm * cj4[v]) : 0.f;
+            }
+        }
+        V8 pr[(NWT + 1) / 2], pd[(NWT + 1) / 2];
+        mfma::pack_p<T, NWT>(pr, PR);
+        mfma::pack_p<T, NWT>(pd, DD);
+        // dK[i] += sum_j round(r)[j,i] (sm gaL)[j] + dDot[j,i] X[j]
+        f32x4 O[DT];
+        mfma::gemm2<T, DT, NWT>(O, Gat, pr, r, q);
+        gemm2_acc<T, DT, NWT>(O, Xt, pd, r, q);
+        if (key_in) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d0 = 4 * DT * q + 4 * dt;
+                if (d0 >= D) continue;
+                f32x4* dst = reinterpret_cast<f32x4*>(G.dk + (blk + i) * D + d0);
+                *dst = *dst + O[dt];
+            }
+        }
+        if (with_v) {   // dV[i] = sum_j round(r)[j,i] gY[j]: this stage is dv's only writer
+            mfma::gemm2<T, DT, NWT>(O, Gyt, pr, r, q);
+            if (key_in) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const int d0 = 4 * DT * q + 4 * dt;
+                    if (d0 >= D) continue;
+                    *reinterpret_cast<f32x4*>(G.dv + (blk + i) * D + d0) = O[dt];
+                }
+            }
+        }
+    }
+}
+
+// The register kernel takes problems with Dv = D, D a multiple of 4 and at most 128, blocks of at
+// most 128 rows, whose blocks are not split over workgroups; MA_ERR_UNSUPPORTED sends the caller on
+// to the LDS kernels.
+template <class T>
+int launch_r_reg(const Problem& P, const BwdBuffers& G, bool first, bool with_v, hipStream_t s) {
+    if (P.Dv != P.D || P.D % 4 != 0 || P.D > 128 || P.B > 128) return static_cast<int>(MA_ERR_UNSUPPORTED);
+    const long long grid = static_cast<long long>(P.E) * P.H * P.M;
+    auto launch = [&](auto dt, auto nt) {
+        constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
+        constexpr size_t lds = RBwdReg<T, DT, NWT>::kLds;
+        auto go = [&](auto kernel) {
+            const int attr = mfma::set_lds_limit(kernel, lds);
+            if (attr) return attr;
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * NWT), lds, s, P, G, first ? 1 : 0, with_v ? 1 : 0);
+            return static_cast<int>(hipGetLastError());
+        };
+        return G.state16 ? go(r_bwd_reg<T, DT, NWT, true>) : go(r_bwd_reg<T, DT, NWT, false>);
+    };
+    auto by_rows = [&](auto dt) {
+        if (P.B <= 16) return launch(dt, std::integral_constant<int, 1>{});
+        if (P.B <= 32) return launch(dt, std::integral_constant<int, 2>{});
+        if (P.B <= 64) return launch(dt, std::integral_constant<int, 4>{});
+        return launch(dt, std::integral_constant<int, 8>{});
+    };
+    if (P.D <= 64) return by_rows(std::integral_constant<int, 4>{});
+    if (P.D <= 80) return by_rows(std::integral_constant<int, 5>{});
+    return by_rows(std::integral_constant<int, 8>{});
+}

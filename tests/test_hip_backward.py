@@ -65,6 +65,10 @@ CASES = [  # E, H, N, D, Dv, B, T, pre, dt, masked
     (1, 2, 256, 128, 128, 128, 2, False, "f16", False), (1, 1, 256, 128, 128, 128, 2, True, "f32", True),
     # few large blocks: the R stage gives a block's tiles of query rows to different workgroups (partial dk / dv)
     (1, 2, 300, 48, 48, 128, 2, False, "f32", True), (1, 3, 260, 64, 64, 128, 3, True, "bf16", False),
+    # 16-bit R stage with the probabilities in registers: head dims of 72 and 128, 64-row blocks with a mask,
+    # 128-row blocks in enough blocks (512) that they are not split over workgroups
+    (1, 2, 224, 72, 72, 32, 3, True, "f16", True), (1, 2, 512, 128, 128, 64, 2, False, "bf16", False),
+    (2, 2, 512, 64, 64, 64, 2, False, "f16", True), (1, 8, 8192, 32, 32, 128, 2, False, "bf16", False),
 ]
 
 
