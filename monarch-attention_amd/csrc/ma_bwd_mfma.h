@@ -1301,6 +1301,10 @@ int launch_lz_t(const Problem& P, const BwdBuffers& G, bool z, hipStream_t s) {
     auto bytes = [&](int t) -> size_t {
         return k32 ? lz_layout<TQ>(P.M, P.D, W, z, t).total : lz_layout16(P.M, P.D, W, z, t).total;
     };
+    if constexpr (!k32) {   // 16-bit operands: the register kernel where it applies
+        const int st = launch_lz_reg<TQ>(P, G, z, s);
+        if (st != static_cast<int>(MA_ERR_UNSUPPORTED)) return st;
+    }
     const int TL = pick_tile(P.M, bytes);
     if (TL == 0) return static_cast<int>(MA_ERR_UNSUPPORTED);
     const size_t lds = bytes(TL);

@@ -1,11 +1,11 @@
-// Backward R stage for fp16 / bf16 operands with the probabilities and their
+// Backward stages for fp16 / bf16 operands with the probabilities and their
 // gradients kept in MFMA accumulator registers, the way the forward stages keep
 // theirs (ma_mfma.h): no fp32 matrices in LDS, no LDS round trip between the
 // products.  Included by ma_bwd_mfma.h inside namespace ma::{anonymous}; the
 // formulas are at the top of ma_bwd.hip, the reference is autograd through
 // al_cl_ref / al_y_cl_ref (ma/ma_torch.py:10-23, :38-52).
 //
-// One workgroup per block problem (e, h, k), one wave per 16-row strip.  LDS holds
+// R stage: one workgroup per block problem (e, h, k), one wave per 16-row strip.  LDS holds
 // five 16-bit operand tiles - K, V, X (aR rows, or Q rows in the first step),
 // Ga = round(sm * gaL), Gy = round(gY) - and seven floats per row.  The products
 // of the stage contract over three different indices, and a lane of the 16x16x32
@@ -280,6 +280,259 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
             }
         }
     }
+}
+
+// ---------------------------------------------------------------- L and Z stages
+// The same scheme for one in-block position j (e, h, j): an M x M problem over query blocks l and
+// key blocks k (formulas at the top of ma_bwd.hip; reference: autograd through ar_cr_ref and z_ref,
+// ma/ma_torch.py:26-35, :55-62).  LDS: aL_j, W (Z: Y_j; L: round(gaR_j)), the Q rows (l, j), in the
+// Z stage the dout rows (l, j), and six floats per row.
+//   pass 1, wave = strip of query blocks l (accumulator rows = key blocks k): U, g -> p, dU;
+//     dq[(l,j)] (+)= sum_k dU[l,k] aL[j,k]  (L: + round(mask_q p)[l,k] gaR[k,j]); row statistics to LDS.
+//   pass 2, wave = strip of key blocks k (accumulator rows = query blocks l): p, dU again;
+//     gaL[j,k] = sum_l dU[l,k] Q[l],  gcL[j,k] = -sum_l dU[l,k],  Z: gY[j,k] = sum_l round(p)[l,k] dout[l].
+template <class T, int DT, int NWT, bool kZ>
+struct LzBwdReg {
+    using Gm = mfma::Geom<DT>;
+    static constexpr int ROWS = 16 * NWT, LD = Gm::LD, TILE = ROWS * LD;
+    static constexpr size_t kLds = (kZ ? 4 : 3) * static_cast<size_t>(TILE) * sizeof(T) + 6 * ROWS * sizeof(float);
+};
+
+template <class T, int DT, int NWT, bool kZ, bool S16>
+__global__ __launch_bounds__(64 * NWT) void lz_bwd_reg(Problem P, BwdBuffers G) {
+    using mfma::lds_row8;
+    using mfma::quad_rows_max;
+    using mfma::quad_rows_sum;
+    using LB = LzBwdReg<T, DT, NWT, kZ>;
+    using TG = typename std::conditional<S16, T, float>::type;
+    using V8 = typename mfma::Ops<T>::v8;
+    using V4 = typename mfma::Ops<T>::v4;
+    using MM = mfma::Ops<T>;
+    constexpr int NTH = 64 * NWT, ROWS = LB::ROWS, LD = LB::LD, KS = mfma::Geom<DT>::KS, COLS = mfma::Geom<DT>::COLS, TILE = LB::TILE;
+    constexpr float kLog2e = mfma::kLog2e;
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+    T* aLt = reinterpret_cast<T*>(lds_raw);
+    T* Wt = aLt + TILE;
+    T* Qt = Wt + TILE;
+    T* dOt = Qt + TILE;   // Z stage only
+    float* cl = reinterpret_cast<float*>(Qt + (kZ ? 2 : 1) * TILE);
+    float* cw = cl + ROWS;
+    float* qok = cw + ROWS;
+    float* mxs = qok + ROWS;
+    float* invs = mxs + ROWS;
+    float* dots = invs + ROWS;
+
+    const int M = P.M, D = P.D, B = P.B;
+    int w = blockIdx.x;
+    const int j = w % B; w /= B;
+    const int h = w % P.H, e = w / P.H;
+    const long long eh = static_cast<long long>(e) * P.H + h;
+    const long long jm = (eh * B + j) * M;   // first row of position j in the (E,H,B,M,.) arrays
+    const int wave = mfma::wave_id(), lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+
+    {
+        const T* aL = reinterpret_cast<const T*>(P.aL) + jm * D;
+        const T* Y = reinterpret_cast<const T*>(P.Y) + jm * D;
+        const TG* gaR = reinterpret_cast<const TG*>(G.gaR);
+        auto aL_row = [=](int k) { return k < M ? aL + k * D : nullptr; };
+        auto y_row = [=](int k) { return k < M ? Y + k * D : nullptr; };
+        auto gar_row = [=](int k) { return k < M ? gaR + ((eh * M + k) * B + j) * D : nullptr; };
+        auto q_row = [=](int l) { return l < M ? tok_row<T>(P.q, P.qs, e, h, l * B + j - P.pad_off, P.N) : nullptr; };
+        auto do_row = [=](int l) { return l < M ? tok_row<T>(G.dout, G.dos, e, h, l * B + j - P.pad_off, P.N) : nullptr; };
+        stage_rows<NTH, T, T>(aLt, LD, ROWS, COLS, D, 1.f, aL_row);
+        stage_rows<NTH, T, T>(Qt, LD, ROWS, COLS, D, 1.f, q_row);
+        if (kZ) {
+            stage_rows<NTH, T, T>(Wt, LD, ROWS, COLS, D, 1.f, y_row);
+            stage_rows<NTH, T, T>(dOt, LD, ROWS, COLS, D, 1.f, do_row);
+        } else {
+            stage_rows<NTH, TG, T>(Wt, LD, ROWS, COLS, D, 1.f, gar_row);
+        }
+        for (int i = threadIdx.x; i < ROWS; i += NTH) {
+            cl[i] = i < M ? P.cL[jm + i] : 0.f;
+            cw[i] = (!kZ && i < M) ? G.gcR[(eh * M + i) * B + j] : 0.f;
+            qok[i] = (i < M && token_ok(P, e, i * B + j - P.pad_off)) ? 1.f : 0.f;
+        }
+    }
+    __syncthreads();
+
+    // ---- pass 1: this wave's strip of query blocks (accumulator rows = key blocks)
+    {
+        const int l = 16 * wave + r;
+        V8 xq[KS], xo[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            xq[ks] = lds_row8<T>(Qt + l * LD + 32 * ks + 8 * q);
+            if (kZ) xo[ks] = lds_row8<T>(dOt + l * LD + 32 * ks + 8 * q);
+        }
+        const float keep = kZ ? 1.f : qok[l];
+        f32x4 U[NWT], Gg[NWT];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < NWT; ++kt) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, g = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                a = MM::mma(lds_row8<T>(aLt + (16 * kt + r) * LD + 32 * ks + 8 * q), xq[ks], a);
+                g = MM::mma(lds_row8<T>(Wt + (16 * kt + r) * LD + 32 * ks + 8 * q), kZ ? xo[ks] : xq[ks], g);
+            }
+            const f32x4 cl4 = *reinterpret_cast<const f32x4*>(cl + 16 * kt + 4 * q), cw4 = *reinterpret_cast<const f32x4*>(cw + 16 * kt + 4 * q);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const bool kin = 16 * kt + 4 * q + v < M;
+                a[v] = kin ? round_to<T>(a[v]) - cl4[v] : -INFINITY;   // U, -inf beyond the M key blocks
+                if (!kZ) g[v] = kin ? keep * (g[v] + cw4[v]) : 0.f;     // gLm = mask_q (Q gaR^T + gcR)
+                mx = fmaxf(mx, a[v]);
+            }
+            U[kt] = a;
+            Gg[kt] = g;
+        }
+        mx = quad_rows_max(mx);
+        float sum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < NWT; ++kt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                U[kt][v] = __builtin_amdgcn_exp2f(kLog2e * (U[kt][v] - mx));
+                sum += U[kt][v];
+            }
+        const float inv = mfma::rcp(quad_rows_sum(sum));
+        float dot = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < NWT; ++kt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                U[kt][v] *= inv;
+                dot = fmaf(Gg[kt][v], U[kt][v], dot);
+            }
+        dot = quad_rows_sum(dot);
+        if (q == 0) {
+            mxs[l] = mx;
+            invs[l] = inv;
+            dots[l] = dot;
+        }
+#pragma unroll
+        for (int kt = 0; kt < NWT; ++kt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                Gg[kt][v] = U[kt][v] * (Gg[kt][v] - dot);   // dU
+                if (!kZ) U[kt][v] *= keep;                  // Lm = mask_q Lp
+            }
+        // dq rows (l, j) (+)= dU aL  (L: + round(Lm) gaR)
+        V8 pd[(NWT + 1) / 2];
+        mfma::pack_p<T, NWT>(pd, Gg);
+        f32x4 O[DT];
+        mfma::gemm2<T, DT, NWT>(O, aLt, pd, r, q);
+        if (!kZ) {
+            V8 pp[(NWT + 1) / 2];
+            mfma::pack_p<T, NWT>(pp, U);
+            gemm2_acc<T, DT, NWT>(O, Wt, pp, r, q);
+        }
+        if (l < M) {
+            float* row = G.dq + ((eh * M + l) * B + j) * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d0 = 4 * DT * q + 4 * dt;
+                if (d0 >= D) continue;
+                f32x4* dst = reinterpret_cast<f32x4*>(row + d0);
+                // the Z stage runs first and every dq row belongs to one workgroup: it is written, not added to
+                *dst = kZ ? O[dt] : *dst + O[dt];
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- pass 2: this wave's strip of key blocks (accumulator rows = query blocks)
+    {
+        const int k = 16 * wave + r;
+        const bool kin = k < M;
+        V8 ak[KS], wk[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            ak[ks] = lds_row8<T>(aLt + k * LD + 32 * ks + 8 * q);
+            wk[ks] = lds_row8<T>(Wt + k * LD + 32 * ks + 8 * q);
+        }
+        const float clk = cl[k], cwk = cw[k];
+        f32x4 PR[NWT], DU[NWT];
+        float gcl = 0.f;
+#pragma unroll
+        for (int lt = 0; lt < NWT; ++lt) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, g = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const V8 qr = lds_row8<T>(Qt + (16 * lt + r) * LD + 32 * ks + 8 * q);
+                a = MM::mma(qr, ak[ks], a);
+                if (kZ) g = MM::mma(lds_row8<T>(dOt + (16 * lt + r) * LD + 32 * ks + 8 * q), wk[ks], g);
+                else g = MM::mma(qr, wk[ks], g);
+            }
+            const int l0 = 16 * lt + 4 * q;
+            const f32x4 mx4 = *reinterpret_cast<const f32x4*>(mxs + l0), inv4 = *reinterpret_cast<const f32x4*>(invs + l0);
+            const f32x4 dot4 = *reinterpret_cast<const f32x4*>(dots + l0), keep4 = *reinterpret_cast<const f32x4*>(qok + l0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float u = kin ? round_to<T>(a[v]) - clk : -INFINITY;
+                const float p = __builtin_amdgcn_exp2f(kLog2e * (u - mx4[v])) * inv4[v];
+                const float gv = kZ ? g[v] : (kin ? keep4[v] * (g[v] + cwk) : 0.f);
+                const float du = p * (gv - dot4[v]);
+                PR[lt][v] = kZ ? p : keep4[v] * p;
+                DU[lt][v] = du;
+                gcl -= du;
+            }
+        }
+        gcl = quad_rows_sum(gcl);
+        if (q == 0 && kin) G.gcL[jm + k] = gcl;   // gcL[j,k] = -sum_l dU
+        V8 pd[(NWT + 1) / 2];
+        mfma::pack_p<T, NWT>(pd, DU);
+        f32x4 O[DT];
+        auto store_state = [&](float* base32) {   // row (j, k) of gaL / gY, in the operand dtype or fp32
+            if (!kin) return;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d0 = 4 * DT * q + 4 * dt;
+                if (d0 >= D) continue;
+                if (S16) {
+                    const V4 o = {from_f<T>(O[dt][0]), from_f<T>(O[dt][1]), from_f<T>(O[dt][2]), from_f<T>(O[dt][3])};
+                    *reinterpret_cast<V4*>(reinterpret_cast<T*>(base32) + (jm + k) * D + d0) = o;
+                } else {
+                    *reinterpret_cast<f32x4*>(base32 + (jm + k) * D + d0) = O[dt];
+                }
+            }
+        };
+        mfma::gemm2<T, DT, NWT>(O, Qt, pd, r, q);   // gaL[j,k] = sum_l dU[l,k] Q[l]
+        store_state(G.gaL);
+        if (kZ) {   // gY[j,k] = sum_l round(Lz)[l,k] dout[l]
+            V8 pp[(NWT + 1) / 2];
+            mfma::pack_p<T, NWT>(pp, PR);
+            mfma::gemm2<T, DT, NWT>(O, dOt, pp, r, q);
+            store_state(G.gY);
+        }
+    }
+}
+
+template <class T>
+int launch_lz_reg(const Problem& P, const BwdBuffers& G, bool z, hipStream_t s) {
+    if (P.Dv != P.D || P.D % 4 != 0 || P.D > 128 || P.M > 128) return static_cast<int>(MA_ERR_UNSUPPORTED);
+    const long long grid = static_cast<long long>(P.E) * P.H * P.B;
+    auto launch = [&](auto dt, auto nt) {
+        constexpr int DT = decltype(dt)::value, NWT = decltype(nt)::value;
+        auto go = [&](auto kernel, size_t lds) {
+            const int attr = mfma::set_lds_limit(kernel, lds);
+            if (attr) return attr;
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * NWT), lds, s, P, G);
+            return static_cast<int>(hipGetLastError());
+        };
+        constexpr size_t lz = LzBwdReg<T, DT, NWT, true>::kLds, ll = LzBwdReg<T, DT, NWT, false>::kLds;
+        if (z) return G.state16 ? go(lz_bwd_reg<T, DT, NWT, true, true>, lz) : go(lz_bwd_reg<T, DT, NWT, true, false>, lz);
+        return G.state16 ? go(lz_bwd_reg<T, DT, NWT, false, true>, ll) : go(lz_bwd_reg<T, DT, NWT, false, false>, ll);
+    };
+    auto by_rows = [&](auto dt) {
+        if (P.M <= 16) return launch(dt, std::integral_constant<int, 1>{});
+        if (P.M <= 32) return launch(dt, std::integral_constant<int, 2>{});
+        if (P.M <= 64) return launch(dt, std::integral_constant<int, 4>{});
+        return launch(dt, std::integral_constant<int, 8>{});
+    };
+    if (P.D <= 64) return by_rows(std::integral_constant<int, 4>{});
+    if (P.D <= 80) return by_rows(std::integral_constant<int, 5>{});
+    return by_rows(std::integral_constant<int, 8>{});
 }
 
 // The register kernel takes problems with Dv = D, D a multiple of 4 and at most 128, blocks of at
