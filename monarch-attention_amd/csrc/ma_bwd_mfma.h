@@ -1271,14 +1271,24 @@ inline int r_tile(const Problem& P, int dt_qk, bool with_v) {
     return pick_tile(P.B, bytes);
 }
 
+// Whether the register kernels (ma_bwd_reg.h) take the L / Z stages resp. the R stage of a problem.
+inline bool reg_operands_ok(const Problem& P, int dt_qk, int dt_v) {
+    return dt_qk != MA_F32 && dt_qk == dt_v && P.Dv == P.D && P.D % 4 == 0 && P.D <= 128;
+}
+
 // Whether a backward pass of this problem can keep its state gradients in the operand dtype: fp16 /
-// bf16 operands of one dtype, every stage within the 16-bit matrix-core kernels' LDS, and the L / Z
-// stages in a single tile of query blocks (gaL and gY are then written once, not accumulated).
+// bf16 operands of one dtype, every stage on a 16-bit matrix-core kernel, and gaL and gY written once,
+// not accumulated over tiles of query blocks (the register kernels always do; the LDS kernels when
+// the L / Z stages fit in a single tile).  The values are rounded to the operand dtype on their way
+// into the next stage's operand tiles either way, so the result is the same bit for bit.
 inline bool state16_ok(const Problem& P, int dt_qk, int dt_v) {
     if (dt_qk == MA_F32 || dt_qk != dt_v) return false;
+    const bool reg = reg_operands_ok(P, dt_qk, dt_v);
     const int M16 = up(P.M, 16);
-    if (lz_layout16(P.M, P.D, P.Dv, true, M16).total > kLdsBudget || lz_layout16(P.M, P.D, P.D, false, M16).total > kLdsBudget) return false;
-    return r_tile(P, dt_qk, true) > 0;
+    const bool lz_ok = (reg && P.M <= 128) || (lz_layout16(P.M, P.D, P.Dv, true, M16).total <= kLdsBudget &&
+                                               lz_layout16(P.M, P.D, P.D, false, M16).total <= kLdsBudget);
+    const bool r_ok = r_tile(P, dt_qk, true) > 0 || (reg && P.B <= 128);
+    return lz_ok && r_ok;
 }
 
 // Number of per-tile partial buffers the R stage wants for dk / dv (0: none).  Splitting a block's
