@@ -46,6 +46,47 @@ __device__ __forceinline__ void gemm2_acc(f32x4 (&O)[DT], const T* tile, const t
             O[dt] = mfma::Ops<T>::mma(mfma::lds_tr8<T, DT>(tile, 32 * g + 4 * q, 16, 2 * g + 1 < NWT, dt, r), pb[g], O[dt]);
 }
 
+// A ROWS x COLS tile of 16-bit rows in flight: issue() starts this thread's 16-byte loads into
+// registers, commit() writes them to the LDS tile (scaled and rounded again where scale != 1).  All
+// tiles of a stage are issued before the first is committed, so staging waits for ONE memory round
+// trip.  For rows of whole 16-byte pieces at 16-byte aligned addresses (the caller checks).
+template <class T, int NTH, int ROWS, int COLS, int LD>
+struct Stage16 {
+    static constexpr int CH = COLS / 8, CNT = (ROWS * CH + NTH - 1) / NTH;
+    mfma::u32x4 v[CNT];
+    template <class RowPtr>
+    __device__ __forceinline__ void issue(RowPtr&& row_ptr, int D) {
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) {
+            const int c = static_cast<int>(threadIdx.x) + i * NTH;
+            const int row = c / CH, ch = c % CH;
+            const T* p = (ROWS * CH % NTH == 0 || c < ROWS * CH) ? row_ptr(row) : nullptr;
+            v[i] = mfma::u32x4{0u, 0u, 0u, 0u};
+            if (p != nullptr && 8 * ch < D) v[i] = *reinterpret_cast<const mfma::u32x4*>(p + 8 * ch);
+        }
+    }
+    __device__ __forceinline__ void commit(T* tile, float scale) const {
+        using V8 = typename mfma::Ops<T>::v8;
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) {
+            const int c = static_cast<int>(threadIdx.x) + i * NTH;
+            if (ROWS * CH % NTH != 0 && c >= ROWS * CH) continue;
+            mfma::u32x4 x = v[i];
+            if (scale != 1.f) {
+                V8 a = __builtin_bit_cast(V8, x);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) a[u] = from_f<T>(scale * to_f(a[u]));
+                x = __builtin_bit_cast(mfma::u32x4, a);
+            }
+            *reinterpret_cast<mfma::u32x4*>(tile + (c / CH) * LD + (c % CH) * 8) = x;
+        }
+    }
+};
+// rows of a (.., t, D) tensor view start on 16-byte boundaries
+__device__ __forceinline__ bool rows16(const void* base, const long long* st) {
+    return reinterpret_cast<uintptr_t>(base) % 16 == 0 && st[0] % 8 == 0 && st[1] % 8 == 0 && st[2] % 8 == 0;
+}
+
 template <class T, int DT, int NWT, bool S16>
 __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, int first, int with_v) {
     using mfma::lds_row8;
@@ -94,12 +135,34 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
         };
         auto ga_row = [=](int j) { return j < B ? gaL + ((eh * B + j) * M + k) * D : nullptr; };
         auto gy_row = [=](int j) { return j < B ? gY + ((eh * B + j) * M + k) * D : nullptr; };
-        stage_rows<NTH, T, T>(Kt, LD, ROWS, COLS, D, 1.f, k_row);
-        stage_rows<NTH, T, T>(Xt, LD, ROWS, COLS, D, 1.f, x_row);
-        stage_rows<NTH, TG, T>(Gat, LD, ROWS, COLS, D, sm, ga_row);
-        if (with_v) {
-            stage_rows<NTH, T, T>(Vt, LD, ROWS, COLS, D, 1.f, v_row);
-            stage_rows<NTH, TG, T>(Gyt, LD, ROWS, COLS, D, 1.f, gy_row);
+        // one memory round trip for all tiles where the rows allow 16-byte loads (uniform test)
+        const bool fast = std::is_same<TG, T>::value && D % 8 == 0 && rows16(P.k, P.ks) && (!with_v || rows16(P.v, P.vs)) &&
+                          (!first || rows16(P.q, P.qs));
+        if (fast) {
+            using St = Stage16<T, NTH, ROWS, COLS, LD>;
+            St sk, sx, sa, sv, sy;
+            sk.issue(k_row, D);
+            sx.issue(x_row, D);
+            sa.issue([=](int j) { return reinterpret_cast<const T*>(ga_row(j)); }, D);
+            if (with_v) {
+                sv.issue(v_row, D);
+                sy.issue([=](int j) { return reinterpret_cast<const T*>(gy_row(j)); }, D);
+            }
+            sk.commit(Kt, 1.f);
+            sx.commit(Xt, 1.f);
+            sa.commit(Gat, sm);
+            if (with_v) {
+                sv.commit(Vt, 1.f);
+                sy.commit(Gyt, 1.f);
+            }
+        } else {
+            stage_rows<NTH, T, T>(Kt, LD, ROWS, COLS, D, 1.f, k_row);
+            stage_rows<NTH, T, T>(Xt, LD, ROWS, COLS, D, 1.f, x_row);
+            stage_rows<NTH, TG, T>(Gat, LD, ROWS, COLS, D, sm, ga_row);
+            if (with_v) {
+                stage_rows<NTH, T, T>(Vt, LD, ROWS, COLS, D, 1.f, v_row);
+                stage_rows<NTH, TG, T>(Gyt, LD, ROWS, COLS, D, 1.f, gy_row);
+            }
         }
         const float* cR = P.cR + blk;
         for (int i = threadIdx.x; i < ROWS; i += NTH) {
@@ -339,13 +402,31 @@ __global__ __launch_bounds__(64 * NWT) void lz_bwd_reg(Problem P, BwdBuffers G) 
         auto gar_row = [=](int k) { return k < M ? gaR + ((eh * M + k) * B + j) * D : nullptr; };
         auto q_row = [=](int l) { return l < M ? tok_row<T>(P.q, P.qs, e, h, l * B + j - P.pad_off, P.N) : nullptr; };
         auto do_row = [=](int l) { return l < M ? tok_row<T>(G.dout, G.dos, e, h, l * B + j - P.pad_off, P.N) : nullptr; };
-        stage_rows<NTH, T, T>(aLt, LD, ROWS, COLS, D, 1.f, aL_row);
-        stage_rows<NTH, T, T>(Qt, LD, ROWS, COLS, D, 1.f, q_row);
-        if (kZ) {
-            stage_rows<NTH, T, T>(Wt, LD, ROWS, COLS, D, 1.f, y_row);
-            stage_rows<NTH, T, T>(dOt, LD, ROWS, COLS, D, 1.f, do_row);
+        const bool fast = (kZ || std::is_same<TG, T>::value) && D % 8 == 0 && rows16(P.q, P.qs) && (!kZ || rows16(G.dout, G.dos));
+        if (fast) {
+            using St = Stage16<T, NTH, ROWS, COLS, LD>;
+            St sa, sq, sw, so;
+            sa.issue(aL_row, D);
+            sq.issue(q_row, D);
+            if (kZ) {
+                sw.issue(y_row, D);
+                so.issue(do_row, D);
+            } else {
+                sw.issue([=](int k) { return reinterpret_cast<const T*>(gar_row(k)); }, D);
+            }
+            sa.commit(aLt, 1.f);
+            sq.commit(Qt, 1.f);
+            sw.commit(Wt, 1.f);
+            if (kZ) so.commit(dOt, 1.f);
         } else {
-            stage_rows<NTH, TG, T>(Wt, LD, ROWS, COLS, D, 1.f, gar_row);
+            stage_rows<NTH, T, T>(aLt, LD, ROWS, COLS, D, 1.f, aL_row);
+            stage_rows<NTH, T, T>(Qt, LD, ROWS, COLS, D, 1.f, q_row);
+            if (kZ) {
+                stage_rows<NTH, T, T>(Wt, LD, ROWS, COLS, D, 1.f, y_row);
+                stage_rows<NTH, T, T>(dOt, LD, ROWS, COLS, D, 1.f, do_row);
+            } else {
+                stage_rows<NTH, TG, T>(Wt, LD, ROWS, COLS, D, 1.f, gar_row);
+            }
         }
         for (int i = threadIdx.x; i < ROWS; i += NTH) {
             cl[i] = i < M ? P.cL[jm + i] : 0.f;
