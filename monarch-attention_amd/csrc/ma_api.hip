@@ -229,9 +229,11 @@ bool fused_full_width(const ma_fwd_params* p) {
 //    against 55 us for T = 3),
 //  * else the chained kernel (one launch) from 32 heads on for blocks and block
 //    counts of at most 64: with many heads the wait of one head's phase is
-//    covered by other heads' problems; with 128-row problems the one kernel is
-//    held to the register / LDS needs of its largest phase, so there
-//  * one launch per half step is as fast or faster.
+//    covered by other heads' problems; and for 128-row blocks AND block counts
+//    (c5: 184 us against 213 us) when the heads divide evenly over the 8 XCDs the
+//    kernel pins them to,
+//  * else one launch per half step (few tasks per head - block counts of 4 or 8
+//    with large blocks -, blocks of 65-96 rows, uneven head counts).
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
     const bool fast32 = mfma32_supported(p);   // fp32 operands: per-stage launches only
@@ -247,7 +249,12 @@ int select_variant(const ma_fwd_params* p) {
             if (!fast) return MA_VARIANT_GENERIC;
             if (heads >= 128 && resident_fits(p)) return MA_VARIANT_RESIDENT;
             if (fused_full_width(p)) return MA_VARIANT_FUSED;
-            if (heads >= 32 && p->B <= 64 && (static_cast<long long>(p->N) + p->B - 1) / p->B <= 64 && chain_fits(p)) return MA_VARIANT_CHAINED;
+            {
+                const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+                if (heads >= 32 && p->B <= 64 && M <= 64 && chain_fits(p)) return MA_VARIANT_CHAINED;
+                // 128-row problems in both orientations (N of 10^4 and more), heads spread evenly over the XCDs
+                if (p->B > 96 && M > 96 && heads % 8 == 0 && chain_fits(p)) return MA_VARIANT_CHAINED;
+            }
             return MA_VARIANT_STAGED;
     }
 }

@@ -11,9 +11,10 @@
 // Every stage is "GEMM1 -> softmax in registers -> GEMM2":
 //   GEMM1  C[w, x] = sum_d W[w, d] X[x, d]     (both operands row-major in d,
 //          so they load as 16-byte vectors: W from its LDS tile, X from HBM)
-//   softmax over w for every x.  In the R and Z steps x is the lane's column,
-//          so the reduction is in-lane plus two cross-lane steps; the L step
-//          needs the transposed orientation and reduces across 16 lanes (DPP).
+//   softmax over w for every x.  x is the lane's column, so the reduction is
+//          in-lane plus two cross-lane steps.  The L step contracts its second
+//          product over x instead of w: it forms the logits a second time with
+//          the operand roles swapped (see LProb).
 //   GEMM2  out^T[d, x] = sum_w Wv^T[d, w] P[w, x].  P is taken straight from
 //          the C registers as the B operand: the k slots of a lane are mapped
 //          to w = 32g + 16(s/4) + 4q + s%4, exactly the rows the lane already
@@ -304,13 +305,10 @@ struct Split {
 template <class T, int DT, int NWT>
 struct Lds {
     static constexpr int ROWS = 16 * NWT;
-    static constexpr int ROWS2 = 32 * ((NWT + 1) / 2);
     static constexpr int TILE = ROWS * Geom<DT>::LD;                 // elements
-    static constexpr int TILE2 = ROWS2 * Geom<DT>::LD;
-    static constexpr int LDP = ROWS2 + 8;                            // pitch of the transposed L tile
     static constexpr size_t R = 2 * TILE * sizeof(T) + ROWS * sizeof(float);
     static constexpr size_t Z = 2 * TILE * sizeof(T) + ROWS * sizeof(float);
-    static constexpr size_t L = (TILE2 + TILE + ROWS * LDP) * sizeof(T) + (1 + Split<NWT>::WPP) * ROWS * sizeof(float);
+    static constexpr size_t L = 2 * TILE * sizeof(T) + 3 * ROWS * sizeof(float);
 };
 
 // Uniform (per problem) description of the tensors: resources and row pitches in bytes.
@@ -680,21 +678,34 @@ __device__ __forceinline__ void z_poison(const Problem& P, const Slices& S, int 
     }
 }
 
-// L step for one column problem (e,h,j).  smem: Qt tile (ROWS2 rows), aL tile,
-// transposed L tile PT[k][l], cL bias, per-wave partial cR.
-// Reference: ar_cr_ref (ma/ma_torch.py:26-35).
+// L step for one column problem (e,h,j).  smem: Q^T tile, aL tile, softmax bias of the key blocks,
+// row maximum and 1 / row sum of the query blocks.  Reference: ar_cr_ref (ma/ma_torch.py:26-35).
+//
+// The softmax runs over the key blocks k of every query block l, the product that follows
+// contracts over l - and a lane can only feed the second product from accumulators whose ROWS are
+// the contraction index, while a softmax is cheapest along the rows of the accumulators (in-lane
+// plus two lane swaps).  So the logits are formed twice:
+//   pass 1, wave = strip of query blocks l (accumulator rows = key blocks k): maximum and sum of
+//           every row l, kept in LDS;
+//   pass 2, wave = strip of key blocks k (accumulator rows = query blocks l): the logits again with
+//           the operand roles swapped, the probabilities from pass 1's statistics, straight into
+//           the B operand of aR[k] = sum_l L[l,k] Q[l]; cR[k] = sum_l L[l,k] in-lane.
+// The second evaluation costs a few instructions on idle matrix pipes and a second exp2 per entry;
+// it saves the transposed copy of the probabilities in LDS (which was as large as both operand
+// tiles together and halved the workgroups per compute unit), its write, its read and the 16-lane
+// reductions of the column-wise softmax.
 template <class T, int DT, int NWT>
 struct LProb {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
     using LS = Lds<T, DT, NWT>;
     static constexpr int WPP = Split<NWT>::WPP;
-    static constexpr int ROWS = LS::ROWS, ROWS2 = LS::ROWS2, LDP = LS::LDP, NG = (NWT + 1) / 2;
+    static constexpr int ROWS = LS::ROWS;
     static constexpr int nth = WPP * 64;
     static constexpr int SPW = NWT / WPP;   // strips per wave (2 for blocks counts above 64)
     struct Pre {
-        TileCopy<T, DT, ROWS2, nth> qc;   // Q^T tile
-        unsigned qm[4 * SPW];             // [4*i + v]: mask byte of the query token of block 16*(wig + i*WPP) + 4q + v
+        TileCopy<T, DT, ROWS, nth> qc;   // Q^T tile
+        unsigned qm[SPW];                // mask word of the query token of block 16*(wig + i*WPP) + lane % 16
     };
     struct St {
         TileCopy<T, DT, ROWS, nth> ac;    // aL tile
@@ -708,12 +719,10 @@ struct LProb {
         const int tix = wig * 64 + lane;
         pre.qc.template issue<true>(S.q, P.D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
 #pragma unroll
-        for (int i = 0; i < SPW; ++i)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int l = 16 * (wig + i * WPP) + 4 * (lane >> 4) + v;
-                pre.qm[4 * i + v] = mask_load(S, P, l * B + j - P.pad_off, l < M);
-            }
+        for (int i = 0; i < SPW; ++i) {
+            const int l = 16 * (wig + i * WPP) + (lane & 15);
+            pre.qm[i] = mask_load(S, P, l * B + j - P.pad_off, l < M);
+        }
     }
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
         if (!active) return;
@@ -727,10 +736,10 @@ struct LProb {
     static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
                                                int j, int wig, int lane) {
         T* Qt = reinterpret_cast<T*>(smem);
-        T* At = Qt + LS::TILE2;
-        T* PT = At + LS::TILE;
-        float* cb = reinterpret_cast<float*>(PT + ROWS * LDP);
-        float* crp = cb + ROWS;  // [WPP][ROWS]
+        T* At = Qt + LS::TILE;
+        float* cb = reinterpret_cast<float*>(At + LS::TILE);
+        float* mxs = cb + ROWS;
+        float* invs = mxs + ROWS;
         const int B = P.B, M = P.M, D = P.D;
         const int r = lane & 15, q = lane >> 4;
         const int tix = wig * 64 + lane;
@@ -739,103 +748,82 @@ struct LProb {
             pre.qc.commit(Qt, tix);
             st.ac.commit(At, tix);
             if (tix < ROWS) cb[tix] = st.cbv;
-            constexpr int PH = ROWS2 > ROWS ? ROWS2 - ROWS : 1;   // phantom l columns of PT that phase 2 reads
-            if (ROWS2 > ROWS)
-                for (int i = tix; i < ROWS * PH; i += nth) PT[(i / PH) * LDP + ROWS + i % PH] = from_f<T>(0.f);
         }
         problem_sync<WPP>();
         if (active) {
-            // phase 1: L[l, k] for 16-row strips of l; lane holds column k = 16kt + r, rows l0 + 4q + v
-            float crsum[NWT];
-#pragma unroll
-            for (int kt = 0; kt < NWT; ++kt) crsum[kt] = 0.f;
+            // pass 1: lane holds query block l = l0 + r, rows = key blocks 16kt + 4q + v
 #pragma unroll
             for (int si = 0; si < SPW; ++si) {
-                const int l0 = 16 * (wig + si * WPP);
-                V8 xa[G::KS];
+                const int l = 16 * (wig + si * WPP) + r;
+                V8 xq[G::KS];
 #pragma unroll
-                for (int ks = 0; ks < G::KS; ++ks) xa[ks] = lds_row8<T>(Qt + (l0 + r) * G::LD + 32 * ks + 8 * q);
+                for (int ks = 0; ks < G::KS; ++ks) xq[ks] = lds_row8<T>(Qt + l * G::LD + 32 * ks + 8 * q);
                 f32x4 C[NWT];
+                float mx = kNegBig;
 #pragma unroll
                 for (int kt = 0; kt < NWT; ++kt) {
                     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(xa[ks], lds_row8<T>(At + (16 * kt + r) * G::LD + 32 * ks + 8 * q), acc);
-                    const float b = cb[16 * kt + r];
+                    for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(lds_row8<T>(At + (16 * kt + r) * G::LD + 32 * ks + 8 * q), xq[ks], acc);
+                    const f32x4 b = *reinterpret_cast<const f32x4*>(cb + 16 * kt + 4 * q);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) acc[v] = fmaf(round_to<T>(acc[v]), kLog2e, b);
+                    for (int v = 0; v < 4; ++v) {
+                        acc[v] = fmaf(round_to<T>(acc[v]), kLog2e, b[v]);
+                        mx = fmaxf(mx, acc[v]);
+                    }
                     C[kt] = acc;
                 }
-                f32x4 mx = C[0];
-#pragma unroll
-                for (int kt = 1; kt < NWT; ++kt)
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) mx[v] = fmaxf(mx[v], C[kt][v]);
-#pragma unroll
-                for (int v = 0; v < 4; ++v) mx[v] = row16_max(mx[v]);
-                f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+                mx = quad_rows_max(mx);
+                float sum = 0.f;
 #pragma unroll
                 for (int kt = 0; kt < NWT; ++kt)
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const float p = __builtin_amdgcn_exp2f(C[kt][v] - mx[v]);
-                        sum[v] += p;
-                        C[kt][v] = p;
-                    }
-                f32x4 inv;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float sv = row16_sum(sum[v]);
+                    for (int v = 0; v < 4; ++v) sum += __builtin_amdgcn_exp2f(C[kt][v] - mx);
+                sum = quad_rows_sum(sum);
+                if (q == 0) {
+                    mxs[l] = mx;
                     // padded / masked query tokens are zeroed after the softmax (ma_torch.py:30)
-                    const int l = l0 + 4 * q + v;
-                    inv[v] = (l < M && token_kept(P, l * B + j - P.pad_off, pre.qm[4 * si + v])) ? rcp(sv) : 0.f;
+                    invs[l] = (l < M && token_kept(P, l * B + j - P.pad_off, pre.qm[si])) ? rcp(sum) : 0.f;
                 }
-#pragma unroll
-                for (int kt = 0; kt < NWT; ++kt) {
-                    typename Ops<T>::v4 o;
-                    float part = 0.f;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const float lv = C[kt][v] * inv[v];
-                        part += lv;
-                        o[v] = from_f<T>(lv);
-                    }
-                    crsum[kt] += part;
-                    *reinterpret_cast<u32x2*>(PT + (16 * kt + r) * LDP + l0 + 4 * q) = __builtin_bit_cast(u32x2, o);
-                }
-            }
-#pragma unroll
-            for (int kt = 0; kt < NWT; ++kt) {
-                const float sv = quad_rows_sum(crsum[kt]);
-                if (q == 0) crp[wig * ROWS + 16 * kt + r] = sv;
             }
         }
         problem_sync<WPP>();
         if (active) {
-            // phase 2: aR[k, :] = sum_l round(L[l,k]) Qt[l, :] for 16-wide tiles of k
-            for (int kt = wig; kt < NWT; kt += WPP) {
-                const int k = 16 * kt + r;
+            // pass 2: lane holds key block k = 16 strip + r, rows = query blocks 16lt + 4q + v
+#pragma unroll
+            for (int si = 0; si < SPW; ++si) {
+                const int k = 16 * (wig + si * WPP) + r;
                 const bool kv = k < M;
-                V8 pb[NG];
+                V8 xk[G::KS];
 #pragma unroll
-                for (int g = 0; g < NG; ++g) pb[g] = lds_row8<T>(PT + k * LDP + 32 * g + 8 * q);
-                f32x4 O[DT];
+                for (int ks = 0; ks < G::KS; ++ks) xk[ks] = lds_row8<T>(At + k * G::LD + 32 * ks + 8 * q);
+                const float cbk = cb[k];
+                f32x4 C[NWT];
+                float crs = 0.f;
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
+                for (int lt = 0; lt < NWT; ++lt) {
                     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int g = 0; g < NG; ++g)   // natural k-slot order here: slot s <-> row 32g + 8q + s
-                        acc = Ops<T>::mma(lds_tr8<T, DT>(Qt, 32 * g + 8 * q, 4, true, dt, r), pb[g], acc);
-                    O[dt] = acc;
+                    for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(lds_row8<T>(Qt + (16 * lt + r) * G::LD + 32 * ks + 8 * q), xk[ks], acc);
+                    const f32x4 mx4 = *reinterpret_cast<const f32x4*>(mxs + 16 * lt + 4 * q);
+                    const f32x4 inv4 = *reinterpret_cast<const f32x4*>(invs + 16 * lt + 4 * q);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float lv = __builtin_amdgcn_exp2f(fmaf(round_to<T>(acc[v]), kLog2e, cbk) - mx4[v]) * inv4[v];
+                        crs += lv;
+                        acc[v] = lv;
+                    }
+                    C[lt] = acc;
                 }
+                crs = quad_rows_sum(crs);
+                // aR[k, :] = sum_l round(L[l,k]) Qt[l, :]
+                V8 pb[(NWT + 1) / 2];
+                pack_p<T, NWT>(pb, C);
+                f32x4 O[DT];
+                gemm2<T, DT, NWT>(O, Qt, pb, r, q);
                 const unsigned arow = static_cast<unsigned>(k * B + j);   // row of aR / cR: (k, j)
                 store_row<T, DT>(S.aR, kv ? arow * db : kOob, D, O, q, S.stream_state);
-                if (q == 0) {
-                    float sv = 0.f;
-#pragma unroll
-                    for (int w = 0; w < WPP; ++w) sv += crp[w * ROWS + k];
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, sv), S.cR, kv ? arow * 4u : kOob, 0, 0);
-                }
+                if (q == 0) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, crs), S.cR, kv ? arow * 4u : kOob, 0, 0);
             }
         }
     }

@@ -175,11 +175,13 @@ def test_auto_variant_policy():
     assert auto(1, 16, 4096, 64, 64) == "fused"         # 16 heads x 64 workgroups: every head has a full team at once
     assert auto(2, 16, 4096, 64, 64) == "chained"
     assert auto(1, 8, 1024, 64, 32) == "fused"
-    assert auto(1, 16, 16384, 64, 128) == "staged"
+    assert auto(1, 16, 16384, 64, 128) == "chained"     # 128-row problems both ways, heads even over the XCDs
+    assert auto(1, 12, 16384, 64, 128) == "staged"      # 12 heads on 8 XCDs: uneven
+    assert auto(16, 12, 512, 64, 128) == "staged"       # 128-row blocks, but only 4 of them per head
     assert auto(64, 12, 197, 64, 16) == "resident"
     assert auto(16, 12, 512, 64, 32) == "chained"      # state of a 512-token head does not fit in LDS
     assert auto(8, 16, 1024, 72, 32) == "chained"
-    assert auto(4, 16, 16384, 64, 128) == "staged"      # many heads, but 128-row problems
+    assert auto(4, 16, 16384, 64, 128) == "chained"
     assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for
     assert auto(2, 2, 197, 64, 16) == "fused"           # few heads
     assert auto(1, 1, 16, 64, 4) == "staged"            # one workgroup per phase: nothing to fuse
