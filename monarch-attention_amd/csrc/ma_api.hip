@@ -628,8 +628,10 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
     G.dout = static_cast<const char*>(b->dout);
     for (int i = 0; i < 3; ++i) G.dos[i] = b->dout_stride[i];
     const long long rows = static_cast<long long>(P.E) * P.H * P.M * P.B;
-    st = launch_bwd_zero(G.dq, rows * (2LL * P.D + P.Dv), s);
-    if (st) return st;
+    if (fma_only || !bwd_all_reg(P, pp.dtype_qk, pp.dtype_v)) {
+        st = launch_bwd_zero(G.dq, rows * (2LL * P.D + P.Dv), s);
+        if (st) return st;
+    }
 
     at_step(T - 1);
     st = launch_bwd_z(P, G, pp.dtype_qk, pp.dtype_v, s);

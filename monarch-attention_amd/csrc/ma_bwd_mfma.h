@@ -1303,6 +1303,12 @@ inline int r_split_tiles(const Problem& P, int dt_qk, int dt_v) {
     return (tiles > 1 && blocks < 512 && (np * P.D) % 4 == 0 && (np * P.Dv) % 4 == 0) ? tiles : 0;
 }
 
+// Whether every stage of a backward pass runs a register kernel.  Those write every row of dq (Z stage)
+// and dv, and the first R stage they run starts dk's sums: the accumulators need no zeroing then.
+inline bool all_reg(const Problem& P, int dt_qk, int dt_v) {
+    return reg_operands_ok(P, dt_qk, dt_v) && P.M <= 128 && P.B <= 128 && r_split_tiles(P, dt_qk, dt_v) <= 1;
+}
+
 // The launchers return MA_ERR_UNSUPPORTED when the problem does not fit; the caller then takes the FMA kernel.
 template <class TQ>
 int launch_lz_t(const Problem& P, const BwdBuffers& G, bool z, hipStream_t s) {

@@ -22,5 +22,6 @@ int launch_bwd_r_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool fir
 
 bool bwd_state16_ok(const Problem& P, int dt_qk, int dt_v) { return state16_ok(P, dt_qk, dt_v); }
 int bwd_r_split_tiles(const Problem& P, int dt_qk, int dt_v) { return r_split_tiles(P, dt_qk, dt_v); }
+bool bwd_all_reg(const Problem& P, int dt_qk, int dt_v) { return all_reg(P, dt_qk, dt_v); }
 
 }  // namespace ma

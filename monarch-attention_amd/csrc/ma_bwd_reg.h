@@ -19,7 +19,7 @@
 //   pass 2, wave = strip of KEYS i (accumulator rows = query rows j):
 //     the same two products with the operand roles swapped, r and dDot formed
 //     again from the row statistics of pass 1;
-//     dK[i] += sum_j r[j,i] Ga[j] + dDot[j,i] X[j],  dV[i] = sum_j r[j,i] Gy[j].
+//     dK[i] (+)= sum_j r[j,i] Ga[j] + dDot[j,i] X[j],  dV[i] = sum_j r[j,i] Gy[j].
 //
 // The recomputation costs four more small products on matrix pipes that are
 // otherwise idle and the softmax arithmetic a second time; it saves three fp32
@@ -328,7 +328,8 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
                 const int d0 = 4 * DT * q + 4 * dt;
                 if (d0 >= D) continue;
                 f32x4* dst = reinterpret_cast<f32x4*>(G.dk + (blk + i) * D + d0);
-                *dst = *dst + O[dt];
+                // the stage that also forms dv is the first R stage of a backward pass: it starts dk's sums
+                *dst = with_v ? O[dt] : *dst + O[dt];
             }
         }
         if (with_v) {   // dV[i] = sum_j round(r)[j,i] gY[j]: this stage is dv's only writer

@@ -102,6 +102,8 @@ struct BwdBuffers {
 bool bwd_state16_ok(const Problem& P, int dt_qk, int dt_v);
 // partial buffers the R stage wants for this problem (0: it does not split blocks over workgroups)
 int bwd_r_split_tiles(const Problem& P, int dt_qk, int dt_v);
+// every stage on a register kernel: dq, dk, dv are written before they are added to (no zeroing needed)
+bool bwd_all_reg(const Problem& P, int dt_qk, int dt_v);
 bool bwd_fits(const Problem& P);
 // matrix-core backward stages: MA_ERR_UNSUPPORTED when the problem's tiles do not fit the LDS
 int launch_bwd_lz_mfma(const Problem& P, const BwdBuffers& G, int dt_qk, bool z, hipStream_t s);
