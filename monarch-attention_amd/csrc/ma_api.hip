@@ -625,6 +625,21 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
     G.pv = L.parts ? reinterpret_cast<float*>(ws + L.pv) : nullptr;
     G.jt_split = 0;
     G.state16 = (!fma_only && bwd_state16_ok(P, pp.dtype_qk, pp.dtype_v)) ? 1 : 0;
+    // register kernels in every stage, rows of the caller's gradients aligned for 4-element stores: the stages
+    // write dq, dk, dv themselves
+    G.direct = 0;
+    {
+        void* outp[3] = {b->dq, b->dk, b->dv};
+        const int64_t* outst[3] = {b->dq_stride, b->dk_stride, b->dv_stride};
+        bool ok = !fma_only && bwd_all_reg(P, pp.dtype_qk, pp.dtype_v);
+        for (int i = 0; i < 3; ++i) {
+            G.out[i] = static_cast<char*>(outp[i]);
+            for (int a = 0; a < 3; ++a) G.outs[i][a] = outst[i][a];
+            ok = ok && reinterpret_cast<uintptr_t>(outp[i]) % (4 * elt_size(pp.dtype_qk)) == 0 && outst[i][0] % 4 == 0 &&
+                 outst[i][1] % 4 == 0 && outst[i][2] % 4 == 0;
+        }
+        G.direct = ok ? 1 : 0;
+    }
     G.dout = static_cast<const char*>(b->dout);
     for (int i = 0; i < 3; ++i) G.dos[i] = b->dout_stride[i];
     const long long rows = static_cast<long long>(P.E) * P.H * P.M * P.B;
@@ -646,6 +661,7 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
             if (st) return st;
         }
     }
+    if (G.direct) return MA_OK;
     // fp32 accumulators -> the caller's tensors: one launch when dv has the shape and dtype of dq / dk
     long long st3[3][3];
     for (int i = 0; i < 3; ++i) { st3[0][i] = b->dq_stride[i]; st3[1][i] = b->dk_stride[i]; st3[2][i] = b->dv_stride[i]; }

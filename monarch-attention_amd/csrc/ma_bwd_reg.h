@@ -184,6 +184,14 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
         g = (key_in && ru >= kTiny) ? fmaf(gcl, d + lg1, gg) : 0.f;
     };
 
+    // four consecutive elements of a finished gradient, rounded into the caller's tensor `which` (0 dq, 1 dk,
+    // 2 dv) at token t; padding positions have no row there
+    auto emit = [&](int which, int t, int d0, const f32x4& val) {
+        if (t < 0 || t >= P.N) return;
+        T* y = reinterpret_cast<T*>(G.out[which]) + e * G.outs[which][0] + h * G.outs[which][1] + t * G.outs[which][2] + d0;
+        *reinterpret_cast<V4*>(y) = V4{from_f<T>(val[0]), from_f<T>(val[1]), from_f<T>(val[2]), from_f<T>(val[3])};
+    };
+
     // ---- pass 1: this wave's strip of query rows (accumulator rows = keys)
     {
         const int j = 16 * wave + r;
@@ -270,7 +278,9 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
                 if (d0 >= D) continue;   // D is a multiple of 4 (checked by the launcher)
                 if (first) {
                     f32x4* dst = reinterpret_cast<f32x4*>(G.dq + (blk + j) * D + d0);
-                    *dst = *dst + O[dt];
+                    const f32x4 total = *dst + O[dt];
+                    if (G.direct) emit(0, k * B + j - P.pad_off, d0, total);   // dq is complete
+                    else *dst = total;
                 } else if (S16) {
                     const V4 o = {from_f<T>(O[dt][0]), from_f<T>(O[dt][1]), from_f<T>(O[dt][2]), from_f<T>(O[dt][3])};
                     *reinterpret_cast<V4*>(reinterpret_cast<T*>(G.gaR) + (blk + j) * D + d0) = o;
@@ -329,7 +339,9 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
                 if (d0 >= D) continue;
                 f32x4* dst = reinterpret_cast<f32x4*>(G.dk + (blk + i) * D + d0);
                 // the stage that also forms dv is the first R stage of a backward pass: it starts dk's sums
-                *dst = with_v ? O[dt] : *dst + O[dt];
+                const f32x4 total = with_v ? O[dt] : *dst + O[dt];
+                if (first && G.direct) emit(1, k * B + i - P.pad_off, d0, total);   // dk is complete
+                else *dst = total;
             }
         }
         if (with_v) {   // dV[i] = sum_j round(r)[j,i] gY[j]: this stage is dv's only writer
@@ -339,7 +351,8 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
                 for (int dt = 0; dt < DT; ++dt) {
                     const int d0 = 4 * DT * q + 4 * dt;
                     if (d0 >= D) continue;
-                    *reinterpret_cast<f32x4*>(G.dv + (blk + i) * D + d0) = O[dt];
+                    if (G.direct) emit(2, k * B + i - P.pad_off, d0, O[dt]);
+                    else *reinterpret_cast<f32x4*>(G.dv + (blk + i) * D + d0) = O[dt];
                 }
             }
         }

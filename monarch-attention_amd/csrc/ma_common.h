@@ -98,6 +98,13 @@ struct BwdBuffers {
     float* pv;     //   tiles of query rows run in different workgroups; nullptr: never split
     int jt_split;  // set by the launcher: workgroups per block (0 = one workgroup walks all tiles)
     int state16;   // gaL, gY, gaR hold the operand dtype instead of fp32 (see bwd_state16_ok)
+    // direct != 0 (register kernels in every stage, see bwd_all_reg): the stage that completes a gradient
+    // rounds it into the caller's tensor itself - dv in the R stage that forms it, dq and dk in the R stage
+    // of the first step - and no conversion kernel runs.  out = {dq, dk, dv} of the caller, outs their
+    // element strides (e, h, token); rows of four elements are 8-byte aligned (checked by the host).
+    int direct;
+    char* out[3];
+    long long outs[3][3];
 };
 bool bwd_state16_ok(const Problem& P, int dt_qk, int dt_v);
 // partial buffers the R stage wants for this problem (0: it does not split blocks over workgroups)
