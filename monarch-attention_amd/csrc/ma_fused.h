@@ -208,7 +208,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, i
             const bool active = task < tasks && slot < PPW && j < P.B;
             typename ZP::Pre pre;
             typename ZP::St st;
-            if (!ts.failed) ZP::issue(P, S, pre, active, active ? j : 0, wig, lane);
+            if (!ts.failed) ZP::template issue<true>(P, S, pre, active, active ? j : 0, wig, lane);
             if (first && wait) team_wait(ts);
             first = false;
             if (ts.failed) {
@@ -233,7 +233,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, i
             const bool active = task < tasks && slot < PPW && j < P.B;
             typename LP::Pre pre;
             typename LP::St st;
-            if (!ts.failed) LP::issue(P, S, pre, active, e, active ? j : 0, wig, lane);
+            if (!ts.failed) LP::template issue<true>(P, S, pre, active, e, active ? j : 0, wig, lane);
             if (first && wait) team_wait(ts);
             first = false;
             if (ts.failed) continue;
@@ -254,7 +254,7 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, i
             const bool active = task < tasks && slot < PPW && m < P.M;
             typename RP::Pre pre;
             typename RP::St st;
-            if (!ts.failed) RP::issue(P, S, pre, active, e, active ? m : 0, first_step, with_v, wig, lane);
+            if (!ts.failed) RP::template issue<true>(P, S, pre, active, e, active ? m : 0, first_step, with_v, wig, lane);
             if (first && wait) team_wait(ts);
             first = false;
             if (ts.failed) continue;

@@ -420,6 +420,10 @@ struct RProb {
         float cr[SPW];
     };
 
+    // NT: the inputs are loaded with the streaming policy (a caller's choice: streaming inputs leave the L2 to
+    // the state, which pays where nothing re-reads them from it - few long heads in one launch; ordinary
+    // loads keep K and Q in L2 for the later steps of many-head and per-stage launches)
+    template <bool NT = false>
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int e, int m, bool first,
                                                  bool with_v, int wig, int lane) {
         if (!active) return;
@@ -427,23 +431,24 @@ struct RProb {
         const int tix = wig * 64 + lane;
         const int t0 = m * B - P.pad_off;
         // order of issue = order of arrival: what the logits need first, the V tile (needed last) last
-        pre.kc.template issue<true>(S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
+        pre.kc.template issue<NT>(S.k, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.kst) : kOob; }, tix);
         if (first) {
 #pragma unroll
             for (int i = 0; i < SPW; ++i) {
                 const int j = 16 * (wig + i * WPP) + (lane & 15);
-                load_x<T, DT, true>(pre.xq[i], S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, lane >> 4);
+                load_x<T, DT, NT>(pre.xq[i], S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, lane >> 4);
             }
         }
         pre.km = mask_load(S, P, t0 + tix, tix < B);
-        if (with_v) issue_v(P, S, pre, active, m, wig, lane);
+        if (with_v) issue_v<NT>(P, S, pre, active, m, wig, lane);
     }
     // the V tile alone (a caller that starts the state loads right away issues it after them)
+    template <bool NT = false>
     static __device__ __forceinline__ void issue_v(const Problem& P, const Slices& S, Pre& pre, bool active, int m, int wig, int lane) {
         if (!active) return;
         const int B = P.B;
         const int t0 = m * B - P.pad_off;
-        pre.vc.template issue<true>(S.v, P.D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, wig * 64 + lane);
+        pre.vc.template issue<NT>(S.v, P.D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, wig * 64 + lane);
     }
 
     static __device__ __forceinline__ void load_state_strip(const Problem& P, const Slices& S, V8 (&xa)[G::KS], float& cr, int m,
@@ -576,14 +581,16 @@ struct ZProb {
         float cbv;      // softmax bias of tile row `tix`
     };
 
+    template <bool NT>
     static __device__ __forceinline__ void load_strip(const Problem& P, const Slices& S, V8 (&xb)[G::KS], int j, int strip, int lane) {
         const int l = 16 * strip + (lane & 15);
-        load_x<T, DT, true>(xb, S.q, l < P.M ? tok_off(l * P.B + j - P.pad_off, P.N, S.qst) : kOob, P.D, lane >> 4);
+        load_x<T, DT, NT>(xb, S.q, l < P.M ? tok_off(l * P.B + j - P.pad_off, P.N, S.qst) : kOob, P.D, lane >> 4);
     }
+    template <bool NT = false>
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int j, int wig, int lane) {
         if (!active) return;
 #pragma unroll
-        for (int i = 0; i < SPW; ++i) load_strip(P, S, pre.xq[i], j, wig + i * WPP, lane);
+        for (int i = 0; i < SPW; ++i) load_strip<NT>(P, S, pre.xq[i], j, wig + i * WPP, lane);
     }
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
         if (!active) return;
@@ -712,12 +719,13 @@ struct LProb {
         float cbv;
     };
 
+    template <bool NT = false>
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int e, int j, int wig,
                                                  int lane) {
         if (!active) return;
         const int B = P.B, M = P.M;
         const int tix = wig * 64 + lane;
-        pre.qc.template issue<true>(S.q, P.D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
+        pre.qc.template issue<NT>(S.q, P.D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
 #pragma unroll
         for (int i = 0; i < SPW; ++i) {
             const int l = 16 * (wig + i * WPP) + (lane & 15);
