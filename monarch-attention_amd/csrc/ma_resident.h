@@ -84,7 +84,7 @@ struct Resident {
             const int c = tix + i * nth;
             const int row = c / CH, ch = c % CH;
             const unsigned ro = rowoff(row);
-            val[i] = bload16<true>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
+            val[i] = bload16<false>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
         }
     }
     static __device__ __forceinline__ void tile_commit(T* tile, const u32x4 (&val)[CNT], int tix, int nth) {
@@ -167,7 +167,7 @@ struct Resident {
                 tile_issue(pre.b, S.v, D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, tix, WPB * 64);
             if (rd.p == 0) {
                 const int j = 16 * wig + c.r;
-                load_x<T, DT, true>(pre.xq, S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, c.q);
+                load_x<T, DT, false>(pre.xq, S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, c.q);
             }
             pre.kb = (tix < B && token_ok(P, e, t0 + tix)) ? 0.f : kNegBig;
         } else {
@@ -176,7 +176,7 @@ struct Resident {
             if (j >= B) return;
             if (rd.p == nph - 1) {   // Z round: the strip's Q rows
                 const int l = 16 * wig + c.r;
-                load_x<T, DT, true>(pre.xq, S.q, l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob, D, c.q);
+                load_x<T, DT, false>(pre.xq, S.q, l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob, D, c.q);
             } else {                 // L round: the Q^T tile and the query mask of the strip's rows
                 tile_issue(pre.a, S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix, WPM * 64);
                 unsigned ok = 0;
