@@ -46,7 +46,7 @@ for p in (ROOT, os.path.join(ROOT, "monarch-attention_amd")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
-CONFIGS = {  # name: (E, H, N, D, B, T, dtype, scale)  - BASELINE.json configs + the metric configuration
+CONFIGS = {  # name: (E, H, N, D, B, T, dtype, scale)  - the benchmark configurations of the reference + the metric configuration
     "cM": (1, 16, 4096, 64, 64, 1, "f16", 1.0),
     "c1": (1, 1, 256, 64, 16, 1, "f32", 1.0),
     "c2": (64, 12, 197, 64, 16, 2, "f16", 0.125),
@@ -54,7 +54,7 @@ CONFIGS = {  # name: (E, H, N, D, B, T, dtype, scale)  - BASELINE.json configs +
     "c3": (16, 12, 512, 64, 32, 2, "bf16", 1.0),
     "c4": (8, 16, 1024, 72, 32, 3, "f16", 1.0),
     "c5": (1, 16, 16384, 64, 128, 3, "f16", 1.0),
-    # model shapes beyond the BASELINE configs (fp32 goes through the fp32 matrix-core stage kernels)
+    # model shapes beyond those (fp32 goes through the fp32 matrix-core stage kernels)
     "gps": (1, 2, 7600, 48, 128, 2, "f32", 1.0),
     "c3f32": (16, 12, 512, 64, 32, 2, "f32", 1.0),
     "bart": (2, 16, 8192, 64, 64, 2, "bf16", 1.0),
