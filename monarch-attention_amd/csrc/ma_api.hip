@@ -118,6 +118,7 @@ Problem make_problem(const ma_fwd_params* p, const ma_ws_layout& L) {
     P.sm_scale = static_cast<float>(1.0 / std::sqrt(static_cast<double>(p->D)));
     P.eps = p->eps;
     P.test_no_spin = (p->flags & MA_FLAG_TEST_NO_SPIN) ? 1 : 0;
+    P.pack_shift = 4;
     return P;
 }
 
@@ -319,6 +320,13 @@ int prepare(const ma_fwd_params* p, Prepared* out) {
     // with more, smaller problems or a state beyond the caches they cost 5-10 %.
     out->P.stream_stores = v == MA_VARIANT_STAGED && p->dtype_qk != MA_F32 && p->B > 32 && out->P.M > 32 &&
                            static_cast<long long>(p->E) * p->H * out->P.M * p->B <= 128 * 1024;
+    // Heads of at most 8 blocks: the per-stage L and Z kernels put 16 >> pack_shift in-block positions
+    // into one 16-row tile (2^pack_shift >= M rows each) instead of leaving most of the tile empty.
+    if (v == MA_VARIANT_STAGED && p->dtype_qk != MA_F32 && out->P.M <= 8) {
+        int sh = 0;
+        while ((1 << sh) < out->P.M) ++sh;
+        out->P.pack_shift = sh;
+    }
     return MA_OK;
 }
 

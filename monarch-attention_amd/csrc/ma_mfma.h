@@ -564,6 +564,25 @@ struct RProb {
     }
 };
 
+// Index x of a 16-row tile of an L / Z problem -> (in-block position, block).  A problem of a head with
+// more than 16 blocks, and every problem of the one-launch kernels, belongs to ONE position j: x is the
+// block.  Per-stage launches of heads with at most 8 blocks pack several positions into the tile
+// (Problem::pack_shift): x stands for block x % pack_m of position j + x / pack_m, the logits between
+// different positions are masked out (a block-diagonal problem), everything else is unchanged.
+template <int NWT>
+struct TileIndex {
+    int j, sh;
+    __device__ __forceinline__ TileIndex(const Problem& P, int j_) : j(j_), sh(NWT == 1 ? P.pack_shift : 4) {}
+    __device__ __forceinline__ int pos(int x) const { return NWT == 1 ? j + (x >> sh) : j; }
+    __device__ __forceinline__ int blk(int x) const { return NWT == 1 ? (x & ((1 << sh) - 1)) : x; }
+    __device__ __forceinline__ bool ok(const Problem& P, int x) const { return blk(x) < P.M && pos(x) < P.B; }
+    __device__ __forceinline__ bool same(int x, int y) const { return NWT != 1 || (x >> sh) == (y >> sh); }
+    // token of query block blk(x) at position pos(x)
+    __device__ __forceinline__ int token(const Problem& P, int x) const { return blk(x) * P.B + pos(x) - P.pad_off; }
+    // row of the (.., B, M, .) state arrays
+    __device__ __forceinline__ unsigned state_row(const Problem& P, int x) const { return static_cast<unsigned>(pos(x) * P.M + blk(x)); }
+};
+
 // Z step for one column problem (e,h,j).  smem: aL tile, Y tile, cL bias.
 // Reference: z_ref (ma/ma_torch.py:55-62) and the final slice (:106-108).
 template <class T, int DT, int NWT>
@@ -583,8 +602,9 @@ struct ZProb {
 
     template <bool NT>
     static __device__ __forceinline__ void load_strip(const Problem& P, const Slices& S, V8 (&xb)[G::KS], int j, int strip, int lane) {
+        const TileIndex<NWT> ti(P, j);
         const int l = 16 * strip + (lane & 15);
-        load_x<T, DT, NT>(xb, S.q, l < P.M ? tok_off(l * P.B + j - P.pad_off, P.N, S.qst) : kOob, P.D, lane >> 4);
+        load_x<T, DT, NT>(xb, S.q, ti.ok(P, l) ? tok_off(ti.token(P, l), P.N, S.qst) : kOob, P.D, lane >> 4);
     }
     template <bool NT = false>
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int j, int wig, int lane) {
@@ -594,23 +614,24 @@ struct ZProb {
     }
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
         if (!active) return;
-        const int M = P.M, D = P.D;
+        const int D = P.D;
         const int tix = wig * 64 + lane;
         const unsigned db = static_cast<unsigned>(D) * sizeof(T);
-        const unsigned row0 = static_cast<unsigned>(j * M);
+        const TileIndex<NWT> ti(P, j);
         // the Y tile (needed last) last
-        st.ac.template issue<true>(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
-        st.cbv = tix < M ? -kLog2e * bloadf<true>(S.cL, (row0 + tix) * 4u) : kNegBig;
-        st.yc.template issue<true>(S.Y, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
+        st.ac.template issue<true>(S.aL, D, [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; }, tix);
+        st.cbv = (tix < ROWS && ti.ok(P, tix)) ? -kLog2e * bloadf<true>(S.cL, ti.state_row(P, tix) * 4u) : kNegBig;
+        st.yc.template issue<true>(S.Y, D, [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; }, tix);
     }
     static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
                                                int j, int wig, int lane) {
         T* At = reinterpret_cast<T*>(smem);
         T* Yt = At + Lds<T, DT, NWT>::TILE;
         float* cb = reinterpret_cast<float*>(Yt + Lds<T, DT, NWT>::TILE);
-        const int B = P.B, M = P.M, D = P.D;
+        const int D = P.D;
         const int r = lane & 15, q = lane >> 4;
         const int tix = wig * 64 + lane;
+        const TileIndex<NWT> ti(P, j);
         if (active) {
             st.ac.commit(At, tix);
             st.yc.commit(Yt, tix);
@@ -633,7 +654,8 @@ struct ZProb {
                 for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(lds_row8<T>(At + (16 * wt + r) * G::LD + 32 * ks + 8 * q), xb[ks], acc);
                 const f32x4 b = *reinterpret_cast<const f32x4*>(cb + 16 * wt + 4 * q);
 #pragma unroll
-                for (int v = 0; v < 4; ++v) acc[v] = fmaf(round_to<T>(acc[v]), kLog2e, b[v]);
+                for (int v = 0; v < 4; ++v)   // (packed tiles: only the key blocks of the query's own position count)
+                    acc[v] = ti.same(16 * wt + 4 * q + v, 16 * strip + r) ? fmaf(round_to<T>(acc[v]), kLog2e, b[v]) : kNegBig;
                 C[wt] = acc;
             }
             float mx = C[0][0];
@@ -660,10 +682,9 @@ struct ZProb {
           }
           if (active) {
             const int l = 16 * (wig + si * WPP) + r;
-            const int t = l * B + j - P.pad_off;
             f32x4 O[DT];
             gemm2<T, DT, NWT>(O, Yt, pb, r, q);
-            store_row<T, DT>(S.out, l < M ? tok_off(t, P.N, S.ost) : kOob, D, O, q, S.stream_out);   // padded query rows are dropped (:108)
+            store_row<T, DT>(S.out, ti.ok(P, l) ? tok_off(ti.token(P, l), P.N, S.ost) : kOob, D, O, q, S.stream_out);   // padded query rows are dropped (:108)
           }
         }
     }
@@ -678,10 +699,11 @@ __device__ __forceinline__ void z_poison(const Problem& P, const Slices& S, int 
     f32x4 O[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) O[dt] = f32x4{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
+    const TileIndex<NWT> ti(P, j);
 #pragma unroll
     for (int si = 0; si < SPW; ++si) {
         const int l = 16 * (wig + si * WPP) + r;
-        store_row<T, DT>(S.out, l < P.M ? tok_off(l * P.B + j - P.pad_off, P.N, S.ost) : kOob, P.D, O, q);
+        store_row<T, DT>(S.out, ti.ok(P, l) ? tok_off(ti.token(P, l), P.N, S.ost) : kOob, P.D, O, q);
     }
 }
 
@@ -723,23 +745,23 @@ struct LProb {
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int e, int j, int wig,
                                                  int lane) {
         if (!active) return;
-        const int B = P.B, M = P.M;
         const int tix = wig * 64 + lane;
-        pre.qc.template issue<NT>(S.q, P.D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix);
+        const TileIndex<NWT> ti(P, j);
+        pre.qc.template issue<NT>(S.q, P.D, [&](int l) { return ti.ok(P, l) ? tok_off(ti.token(P, l), P.N, S.qst) : kOob; }, tix);
 #pragma unroll
         for (int i = 0; i < SPW; ++i) {
             const int l = 16 * (wig + i * WPP) + (lane & 15);
-            pre.qm[i] = mask_load(S, P, l * B + j - P.pad_off, l < M);
+            pre.qm[i] = mask_load(S, P, ti.token(P, l), ti.ok(P, l));
         }
     }
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
         if (!active) return;
-        const int M = P.M, D = P.D;
+        const int D = P.D;
         const int tix = wig * 64 + lane;
         const unsigned db = static_cast<unsigned>(D) * sizeof(T);
-        const unsigned row0 = static_cast<unsigned>(j * M);
-        st.ac.template issue<true>(S.aL, D, [&](int k) { return k < M ? (row0 + k) * db : kOob; }, tix);
-        st.cbv = tix < M ? -kLog2e * bloadf<true>(S.cL, (row0 + tix) * 4u) : kNegBig;
+        const TileIndex<NWT> ti(P, j);
+        st.ac.template issue<true>(S.aL, D, [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; }, tix);
+        st.cbv = (tix < ROWS && ti.ok(P, tix)) ? -kLog2e * bloadf<true>(S.cL, ti.state_row(P, tix) * 4u) : kNegBig;
     }
     static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
                                                int j, int wig, int lane) {
@@ -748,10 +770,11 @@ struct LProb {
         float* cb = reinterpret_cast<float*>(At + LS::TILE);
         float* mxs = cb + ROWS;
         float* invs = mxs + ROWS;
-        const int B = P.B, M = P.M, D = P.D;
+        const int B = P.B, D = P.D;
         const int r = lane & 15, q = lane >> 4;
         const int tix = wig * 64 + lane;
         const unsigned db = static_cast<unsigned>(D) * sizeof(T);
+        const TileIndex<NWT> ti(P, j);
         if (active) {
             pre.qc.commit(Qt, tix);
             st.ac.commit(At, tix);
@@ -775,8 +798,8 @@ struct LProb {
                     for (int ks = 0; ks < G::KS; ++ks) acc = Ops<T>::mma(lds_row8<T>(At + (16 * kt + r) * G::LD + 32 * ks + 8 * q), xq[ks], acc);
                     const f32x4 b = *reinterpret_cast<const f32x4*>(cb + 16 * kt + 4 * q);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        acc[v] = fmaf(round_to<T>(acc[v]), kLog2e, b[v]);
+                    for (int v = 0; v < 4; ++v) {   // (packed tiles: only the key blocks of the query's own position count)
+                        acc[v] = ti.same(16 * kt + 4 * q + v, l) ? fmaf(round_to<T>(acc[v]), kLog2e, b[v]) : kNegBig;
                         mx = fmaxf(mx, acc[v]);
                     }
                     C[kt] = acc;
@@ -791,7 +814,7 @@ struct LProb {
                 if (q == 0) {
                     mxs[l] = mx;
                     // padded / masked query tokens are zeroed after the softmax (ma_torch.py:30)
-                    invs[l] = (l < M && token_kept(P, l * B + j - P.pad_off, pre.qm[si])) ? rcp(sum) : 0.f;
+                    invs[l] = (ti.ok(P, l) && token_kept(P, ti.token(P, l), pre.qm[si])) ? rcp(sum) : 0.f;
                 }
             }
         }
@@ -801,7 +824,7 @@ struct LProb {
 #pragma unroll
             for (int si = 0; si < SPW; ++si) {
                 const int k = 16 * (wig + si * WPP) + r;
-                const bool kv = k < M;
+                const bool kv = ti.ok(P, k);
                 V8 xk[G::KS];
 #pragma unroll
                 for (int ks = 0; ks < G::KS; ++ks) xk[ks] = lds_row8<T>(At + k * G::LD + 32 * ks + 8 * q);
@@ -817,7 +840,8 @@ struct LProb {
                     const f32x4 inv4 = *reinterpret_cast<const f32x4*>(invs + 16 * lt + 4 * q);
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
-                        const float lv = __builtin_amdgcn_exp2f(fmaf(round_to<T>(acc[v]), kLog2e, cbk) - mx4[v]) * inv4[v];
+                        const float u = ti.same(16 * lt + 4 * q + v, k) ? fmaf(round_to<T>(acc[v]), kLog2e, cbk) : kNegBig;
+                        const float lv = __builtin_amdgcn_exp2f(u - mx4[v]) * inv4[v];
                         crs += lv;
                         acc[v] = lv;
                     }
@@ -829,7 +853,7 @@ struct LProb {
                 pack_p<T, NWT>(pb, C);
                 f32x4 O[DT];
                 gemm2<T, DT, NWT>(O, Qt, pb, r, q);
-                const unsigned arow = static_cast<unsigned>(k * B + j);   // row of aR / cR: (k, j)
+                const unsigned arow = static_cast<unsigned>(ti.blk(k) * B + ti.pos(k));   // row of aR / cR: (block, position)
                 store_row<T, DT>(S.aR, kv ? arow * db : kOob, D, O, q, S.stream_state);
                 if (q == 0) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, crs), S.cR, kv ? arow * 4u : kOob, 0, 0);
             }
@@ -899,12 +923,15 @@ __global__ __launch_bounds__(64 * Split<NWT>::WG) void l_step_mfma(Problem P) {
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT, Split<NWT>::WG>::PPW;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
-    const unsigned total = static_cast<unsigned>(P.E) * P.H * P.B;
+    // problems per head: one per in-block position, or per group of positions that share a tile (TileIndex)
+    const unsigned per = NWT == 1 ? static_cast<unsigned>(16 >> P.pack_shift) : 1u;
+    const unsigned groups = (static_cast<unsigned>(P.B) + per - 1) / per;
+    const unsigned total = static_cast<unsigned>(P.E) * P.H * groups;
     unsigned pid = blockIdx.x * PPW + slot;
     const bool active = pid < total;
     if (!active) pid = 0;
-    const int j = pid % static_cast<unsigned>(P.B);
-    const unsigned eh = pid / static_cast<unsigned>(P.B);
+    const int j = static_cast<int>((pid % groups) * per);
+    const unsigned eh = pid / groups;
     const int h = eh % static_cast<unsigned>(P.H);
     const int e = eh / static_cast<unsigned>(P.H);
     l_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::L, active, e, h, static_cast<long long>(eh), j, wig, lane);
@@ -916,12 +943,15 @@ __global__ __launch_bounds__(64 * Split<NWT>::WG) void z_step_mfma(Problem P) {
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT, Split<NWT>::WG>::PPW;
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
-    const unsigned total = static_cast<unsigned>(P.E) * P.H * P.B;
+    // problems per head: one per in-block position, or per group of positions that share a tile (TileIndex)
+    const unsigned per = NWT == 1 ? static_cast<unsigned>(16 >> P.pack_shift) : 1u;
+    const unsigned groups = (static_cast<unsigned>(P.B) + per - 1) / per;
+    const unsigned total = static_cast<unsigned>(P.E) * P.H * groups;
     unsigned pid = blockIdx.x * PPW + slot;
     const bool active = pid < total;
     if (!active) pid = 0;
-    const int j = pid % static_cast<unsigned>(P.B);
-    const unsigned eh = pid / static_cast<unsigned>(P.B);
+    const int j = static_cast<int>((pid % groups) * per);
+    const unsigned eh = pid / groups;
     const int h = eh % static_cast<unsigned>(P.H);
     const int e = eh / static_cast<unsigned>(P.H);
     z_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::Z, active, e, h, static_cast<long long>(eh), j, wig, lane);

@@ -111,7 +111,8 @@ int launch_l(const Problem& P, hipStream_t s) {
         constexpr size_t lds = PPW * Lds<T, DT, NWT>::L;
         const int attr = set_lds_limit(l_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
-        const long long problems = static_cast<long long>(P.E) * P.H * P.B;
+        const long long per = NWT == 1 ? (16 >> P.pack_shift) : 1;   // positions per problem (see TileIndex)
+        const long long problems = static_cast<long long>(P.E) * P.H * ((P.B + per - 1) / per);
         hipLaunchKernelGGL((l_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(64 * WG), lds, s, P);
         return static_cast<int>(hipGetLastError());
     });
@@ -125,7 +126,8 @@ int launch_z(const Problem& P, hipStream_t s) {
         constexpr size_t lds = PPW * Lds<T, DT, NWT>::Z;
         const int attr = set_lds_limit(z_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
-        const long long problems = static_cast<long long>(P.E) * P.H * P.B;
+        const long long per = NWT == 1 ? (16 >> P.pack_shift) : 1;
+        const long long problems = static_cast<long long>(P.E) * P.H * ((P.B + per - 1) / per);
         hipLaunchKernelGGL((z_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(64 * WG), lds, s, P);
         return static_cast<int>(hipGetLastError());
     });

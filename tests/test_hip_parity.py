@@ -160,6 +160,26 @@ def test_roberta_block_sizes_with_tokenizer_mask(B, variant):
     assert_parity(out.cpu(), ref, "f16", f"roberta B={B}/{variant}")
 
 
+FEW_BLOCKS = [  # E, H, N, D, B, T, pre, dt, masked: 1, 2, 3, 4, 5, 7 and 8 blocks per head, ragged last blocks
+    (2, 3, 90, 32, 90, 2, False, "f16", False), (1, 2, 100, 64, 64, 2, True, "bf16", True),
+    (2, 2, 384, 64, 128, 1, False, "f16", True), (1, 4, 512, 64, 128, 2, False, "f16", False),
+    (1, 2, 333, 40, 67, 3, True, "f16", True), (2, 1, 140, 128, 20, 2, False, "bf16", False),
+    (1, 12, 512, 64, 64, 2, False, "bf16", True), (1, 2, 17, 16, 3, 2, True, "f16", False),
+]
+
+
+@pytest.mark.parametrize("variant", ["staged", "auto"])
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", FEW_BLOCKS)
+def test_heads_of_few_blocks(E, H, N, D, B, T, pre, dt, masked, variant):
+    """At most 8 blocks per head: the per-stage L and Z kernels lay 16, 8, 4 or 2 in-block positions side by
+    side in one 16-row tile and keep them apart with a block-diagonal mask."""
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
+    mask = block_safe_mask(E, N, B, seed=B) if masked else None
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
+    out = run_hip(*to_dev(q, k, v, mask), T, B, pre, variant)
+    assert_parity(out.cpu(), ref, dt, f"few blocks {(E, H, N, D, B, T, pre, dt, masked)}/{variant}")
+
+
 def test_broadcast_over_tokens_is_accepted():
     """expand()-ed inputs (stride 0 along N) are legal for the reference (it pads, i.e. copies); the
     operator takes them too, by making the one copy the library's row-overlap check asks for."""
@@ -220,6 +240,12 @@ STAGE_CASES = [  # E,H,N,D,Dv,B,T,pre,dt,vdt,mask
     (1, 2, 256, 64, 64, 32, 2, False, "bf16", "bf16", False),
     (1, 1, 1024, 64, 64, 64, 2, False, "f16", "f16", False),
     (1, 2, 40, 32, 40, 8, 2, False, "f16", "f32", False),
+    # heads of 1..8 blocks: the 16-bit L and Z kernels put several in-block positions into one tile
+    (1, 2, 200, 64, 64, 64, 2, True, "f16", "f16", True),
+    (2, 2, 250, 32, 32, 96, 3, False, "bf16", "bf16", True),
+    (1, 2, 100, 64, 64, 100, 2, False, "f16", "f16", False),
+    (1, 3, 130, 40, 40, 20, 2, True, "f16", "f16", False),
+    (1, 2, 45, 72, 72, 27, 2, False, "bf16", "bf16", False),
 ]
 
 
