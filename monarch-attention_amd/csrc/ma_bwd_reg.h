@@ -274,7 +274,7 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
         if (jv) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const int d0 = 4 * DT * q + 4 * dt;
+                const int d0 = mfma::chunk_col<DT>(q, dt);
                 if (d0 >= D) continue;   // D is a multiple of 4 (checked by the launcher)
                 if (first) {
                     f32x4* dst = reinterpret_cast<f32x4*>(G.dq + (blk + j) * D + d0);
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
         if (key_in) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const int d0 = 4 * DT * q + 4 * dt;
+                const int d0 = mfma::chunk_col<DT>(q, dt);
                 if (d0 >= D) continue;
                 f32x4* dst = reinterpret_cast<f32x4*>(G.dk + (blk + i) * D + d0);
                 // the stage that also forms dv is the first R stage of a backward pass: it starts dk's sums
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
             if (key_in) {
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const int d0 = 4 * DT * q + 4 * dt;
+                    const int d0 = mfma::chunk_col<DT>(q, dt);
                     if (d0 >= D) continue;
                     if (G.direct) emit(2, k * B + i - P.pad_off, d0, O[dt]);
                     else *reinterpret_cast<f32x4*>(G.dv + (blk + i) * D + d0) = O[dt];
@@ -526,7 +526,7 @@ __global__ __launch_bounds__(64 * NWT) void lz_bwd_reg(Problem P, BwdBuffers G) 
             float* row = G.dq + ((eh * M + l) * B + j) * D;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const int d0 = 4 * DT * q + 4 * dt;
+                const int d0 = mfma::chunk_col<DT>(q, dt);
                 if (d0 >= D) continue;
                 f32x4* dst = reinterpret_cast<f32x4*>(row + d0);
                 // the Z stage runs first and every dq row belongs to one workgroup: it is written, not added to
@@ -582,7 +582,7 @@ __global__ __launch_bounds__(64 * NWT) void lz_bwd_reg(Problem P, BwdBuffers G) 
             if (!kin) return;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const int d0 = 4 * DT * q + 4 * dt;
+                const int d0 = mfma::chunk_col<DT>(q, dt);
                 if (d0 >= D) continue;
                 if (S16) {
                     const V4 o = {from_f<T>(O[dt][0]), from_f<T>(O[dt][1]), from_f<T>(O[dt][2]), from_f<T>(O[dt][3])};

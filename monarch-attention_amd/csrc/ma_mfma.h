@@ -205,18 +205,29 @@ __device__ __forceinline__ typename Ops<T>::v8 lds_row8(const T* tile_elem) {
     return __builtin_bit_cast(typename Ops<T>::v8, *reinterpret_cast<const u32x4*>(tile_elem));
 }
 
+// Which tile columns a lane ends up with after GEMM2: the first of the four consecutive columns
+// that lane group g (r/4 of an MFMA row on the operand side, q of a lane on the result side) has in
+// output tile dt.  Even DT: tiles 2p and 2p+1 give a lane the 8 columns 8*(g + 4p) .., a 16-byte
+// piece, and the four lane groups of a row write 64 contiguous bytes with each store instruction.
+// Odd DT, or RUN (the kernel that keeps its state in LDS and writes little to memory asks for it:
+// it is at its register limit and this form costs it three registers fewer): a lane's 4*DT columns
+// are one consecutive run, 4*DT*g ...
+template <int DT, bool RUN = false>
+__host__ __device__ constexpr int chunk_col(int g, int dt) {
+    return (DT % 2 == 0 && !RUN) ? 8 * g + 32 * (dt >> 1) + 4 * (dt & 1) : 4 * DT * g + 4 * dt;
+}
+
 // Transposed A operand of GEMM2 from a row-major LDS tile via ds_read_b64_tr_b16.
 // Output tile dt, lane (r, q) = MFMA row r: the row is mapped to the tile column
-// d = 4*DT*(r/4) + 4*dt + r%4, so that after all DT tiles a lane of the C layout
-// (rows 4q..4q+3) owns the 4*DT CONSECUTIVE columns 4*DT*q .. 4*DT*(q+1)-1 and
-// can store them as one contiguous run.  row0 is the tile row of k slot 0,
-// hi_rows the distance to the row of k slot 4.
-template <class T, int DT>
+// d = chunk_col(r/4, dt) + r%4, so that a lane of the C layout (rows 4q..4q+3) owns the columns
+// chunk_col(q, dt) .. +3.  row0 is the tile row of k slot 0, hi_rows the distance to the row of
+// k slot 4.
+template <class T, int DT, bool RUN = false>
 __device__ __forceinline__ typename Ops<T>::v8 lds_tr8(const T* tile, int row0, int hi_rows, bool with_hi, int dt, int r) {
     typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
     constexpr int LD = Geom<DT>::LD;
     const int e = r >> 2, c = r & 3;
-    const T* p0 = tile + (row0 + e) * LD + 4 * DT * c + 4 * dt;
+    const T* p0 = tile + (row0 + e) * LD + chunk_col<DT, RUN>(c, dt);
     i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
     i16x4 hi = {0, 0, 0, 0};
     if (with_hi) hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + hi_rows * LD));
@@ -241,8 +252,8 @@ __device__ __forceinline__ void pack_p(typename Ops<T>::v8 (&pb)[(NWT + 1) / 2],
     }
 }
 
-// GEMM2: O[dt][v] = sum_w tile[w][4*DT*q + 4*dt + v] * P[w][x = lane column]
-template <class T, int DT, int NWT>
+// GEMM2: O[dt][v] = sum_w tile[w][chunk_col(q, dt) + v] * P[w][x = lane column]
+template <class T, int DT, int NWT, bool RUN = false>
 __device__ __forceinline__ void gemm2(f32x4 (&O)[DT], const T* tile, const typename Ops<T>::v8 (&pb)[(NWT + 1) / 2],
                                       int r, int q) {
 #pragma unroll
@@ -250,12 +261,12 @@ __device__ __forceinline__ void gemm2(f32x4 (&O)[DT], const T* tile, const typen
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int g = 0; g < (NWT + 1) / 2; ++g)
-            acc = Ops<T>::mma(lds_tr8<T, DT>(tile, 32 * g + 4 * q, 16, 2 * g + 1 < NWT, dt, r), pb[g], acc);
+            acc = Ops<T>::mma(lds_tr8<T, DT, RUN>(tile, 32 * g + 4 * q, 16, 2 * g + 1 < NWT, dt, r), pb[g], acc);
         O[dt] = acc;
     }
 }
 
-// Store a lane's 4*DT consecutive output elements (columns 4*DT*q ..) of the row at
+// Store a lane's 4*DT output elements (columns chunk_col(q, dt) ..) of the row at
 // byte offset ro (kOob drops the store): 16-byte pieces when the head dim fills the
 // tiles exactly, else 8-byte pieces so that a piece never straddles D.
 // stream: the rows are whole 128-byte lines (see Slices::stream_*): they are written with
@@ -264,10 +275,10 @@ __device__ __forceinline__ void gemm2(f32x4 (&O)[DT], const T* tile, const typen
 // (measured: 5 us after an R step that wrote 17 MB, against 2 us with streaming stores).
 // Rows that share lines with other writers keep the plain policy (partial streaming
 // writes are several times slower).
-template <class T, int DT>
+template <class T, int DT, bool RUN = false>
 __device__ __forceinline__ void store_row(rsrc_t dst, unsigned ro, int D, const f32x4 (&O)[DT], int q, bool stream = false) {
     typedef typename Ops<T>::v4 V4;
-    const unsigned base = ro + 8 * DT * q;  // bytes
+    const unsigned base = ro + 2 * chunk_col<DT, RUN>(q, 0);  // bytes; the pieces sit at fixed distances from it
     if (DT % 2 == 0 && D == 16 * DT) {
 #pragma unroll
         for (int p = 0; p < DT / 2; ++p) {
@@ -275,15 +286,15 @@ __device__ __forceinline__ void store_row(rsrc_t dst, unsigned ro, int D, const 
             V4 b = {from_f<T>(O[2 * p + 1][0]), from_f<T>(O[2 * p + 1][1]), from_f<T>(O[2 * p + 1][2]), from_f<T>(O[2 * p + 1][3])};
             const u32x2 lo = __builtin_bit_cast(u32x2, a), hi = __builtin_bit_cast(u32x2, b);
             const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
-            if (stream) __builtin_amdgcn_raw_buffer_store_b128(v, dst, base + 16 * p, 0, 2);
-            else __builtin_amdgcn_raw_buffer_store_b128(v, dst, base + 16 * p, 0, 0);
+            if (stream) __builtin_amdgcn_raw_buffer_store_b128(v, dst, base + 2 * (chunk_col<DT, RUN>(0, 2 * p) - chunk_col<DT, RUN>(0, 0)), 0, 2);
+            else __builtin_amdgcn_raw_buffer_store_b128(v, dst, base + 2 * (chunk_col<DT, RUN>(0, 2 * p) - chunk_col<DT, RUN>(0, 0)), 0, 0);
         }
     } else {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             V4 a = {from_f<T>(O[dt][0]), from_f<T>(O[dt][1]), from_f<T>(O[dt][2]), from_f<T>(O[dt][3])};
-            const int d0 = 4 * DT * q + 4 * dt;
-            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, a), dst, d0 < D ? base + 8 * dt : kOob, 0, 0);
+            const int d0 = chunk_col<DT, RUN>(q, dt);
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, a), dst, d0 < D ? base + 2 * chunk_col<DT, RUN>(0, dt) : kOob, 0, 0);
         }
     }
 }

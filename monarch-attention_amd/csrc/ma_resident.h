@@ -120,7 +120,7 @@ struct Resident {
         return rd.head < heads;
     }
 
-    // lane's 4*DT consecutive elements (columns 4*DT*q ..) of an LDS row
+    // lane's 4*DT consecutive elements (columns 4*DT*q ..: chunk_col's RUN form, used throughout this kernel) of an LDS row
     static __device__ __forceinline__ void lds_store_row(T* row, const f32x4 (&O)[DT], int q) {
         T* dst = row + 4 * DT * q;
         if (DT % 2 == 0) {
@@ -141,7 +141,7 @@ struct Resident {
     }
 
     // transposed A operand from arbitrary LDS rows: p_lo / p_hi point at this lane's source row
-    // (k slot e resp. 4 + e of its 16-lane group) at column 4*DT*c + 4*dt
+    // (k slot e resp. 4 + e of its 16-lane group) at column chunk_col(c, dt)
     static __device__ __forceinline__ V8 tr8(const T* p_lo, const T* p_hi) {
         typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
         typedef short i16x8 __attribute__((ext_vector_type(8)));
@@ -279,7 +279,7 @@ struct Resident {
             pack_p<T, NTB>(pb, C);
             {
                 f32x4 O[DT];
-                gemm2<T, DT, NTB>(O, Kt, pb, r, q);
+                gemm2<T, DT, NTB, true>(O, Kt, pb, r, q);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -288,7 +288,7 @@ struct Resident {
             }
             if (with_v) {
                 f32x4 O[DT];
-                gemm2<T, DT, NTB>(O, Vt, pb, r, q);
+                gemm2<T, DT, NTB, true>(O, Vt, pb, r, q);
                 if (jv) lds_store_row(c.SY + lrow * LD, O, q);
             }
         }
@@ -385,8 +385,8 @@ struct Resident {
 #pragma unroll
                 for (int g = 0; g < NG; ++g) {   // natural k-slot order: slot s <-> query block 32g + 8q + s
                     const int lo = 32 * g + 8 * q + e4, hi = lo + 4;
-                    const T* p_lo = (lo < ROWSM ? Qt + lo * LD : c.ZR) + 4 * DT * c4 + 4 * dt;
-                    const T* p_hi = (hi < ROWSM ? Qt + hi * LD : c.ZR) + 4 * DT * c4 + 4 * dt;
+                    const T* p_lo = (lo < ROWSM ? Qt + lo * LD : c.ZR) + chunk_col<DT, true>(c4, dt);
+                    const T* p_hi = (hi < ROWSM ? Qt + hi * LD : c.ZR) + chunk_col<DT, true>(c4, dt);
                     acc = Ops<T>::mma(tr8(p_lo, p_hi), pb[g], acc);
                 }
                 O[dt] = acc;
@@ -462,13 +462,13 @@ struct Resident {
 #pragma unroll
                 for (int g = 0; g < (NTM + 1) / 2; ++g) {   // k slot s <-> key block 32g + 16(s/4) + 4q + s%4
                     const int lo = 32 * g + 4 * q + e4, hi = lo + 16;
-                    const T* p_lo = (lo < M ? c.SY + (j * M + lo) * LD : c.ZR) + 4 * DT * c4 + 4 * dt;
-                    const T* p_hi = (hi < M ? c.SY + (j * M + hi) * LD : c.ZR) + 4 * DT * c4 + 4 * dt;
+                    const T* p_lo = (lo < M ? c.SY + (j * M + lo) * LD : c.ZR) + chunk_col<DT, true>(c4, dt);
+                    const T* p_hi = (hi < M ? c.SY + (j * M + hi) * LD : c.ZR) + chunk_col<DT, true>(c4, dt);
                     acc = Ops<T>::mma(tr8(p_lo, p_hi), pb[g], acc);
                 }
                 O[dt] = acc;
             }
-            store_row<T, DT>(S.out, l < M ? tok_off(t, P.N, S.ost) : kOob, D, O, q, S.stream_out);   // padded query rows are dropped
+            store_row<T, DT, true>(S.out, l < M ? tok_off(t, P.N, S.ost) : kOob, D, O, q, S.stream_out);   // padded query rows are dropped
         }
         round_end<WPM>(P, rd);
     }
