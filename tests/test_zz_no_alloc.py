@@ -43,6 +43,7 @@ CASES = [  # two calls in a row per case: (E, H, N, D, B, T, pre, dtype, masked)
     ((1, 16, 4096, 64, 64, 1, False, "f16", False), (1, 4, 1000, 64, 32, 2, True, "f16", True)),      # the metric workload first
     ((2, 3, 512, 64, 32, 3, False, "bf16", True), (1, 2, 197, 64, 16, 2, True, "bf16", False)),
     ((1, 2, 300, 48, 16, 2, False, "f32", True), (1, 1, 64, 48, 16, 1, False, "f32", False)),
+    ((2, 12, 512, 64, 128, 2, False, "f16", True), (1, 3, 200, 64, 96, 2, True, "f16", False)),          # heads of 4 and 3 blocks
 ]
 
 
