@@ -62,7 +62,7 @@ CONFIGS = {  # name: (E, H, N, D, B, T, dtype, scale)  - the benchmark configura
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
 MFMA_PEAK_TFLOPS_F32 = 157.3   # dense fp32
-FETCH_SIZE_FACTOR = 2.00       # FETCH_SIZE under-reports a plain copy of known size by this factor (profiles/traffic_cM_T1.md)
+FETCH_SIZE_FACTOR = 2.00       # FETCH_SIZE under-reports a plain copy of known size by this factor (profiles/traffic_forward_kernels.md)
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
 KERNEL_DIR = os.path.join(ROOT, "monarch-attention_amd", "csrc")
 ONE_LAUNCH = {"fused": "fused_fwd_mfma", "resident": "resident_fwd_mfma", "chained": "chain_fwd_mfma"}

@@ -305,6 +305,15 @@ int run_z(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
     return p->dtype_qk == MA_F16 ? launch_mfma_z_f16(pr.P, s) : launch_mfma_z_bf16(pr.P, s);
 }
 
+// Heads of at most 8 blocks: the 16-bit per-stage L and Z kernels put 16 >> pack_shift in-block positions
+// into one 16-row tile (2^pack_shift >= M rows each) instead of leaving most of the tile empty.
+int pack_shift_of(int variant, const ma_fwd_params* p, int M) {
+    if (variant != MA_VARIANT_STAGED || p->dtype_qk == MA_F32 || M > 8) return 4;
+    int sh = 0;
+    while ((1 << sh) < M) ++sh;
+    return sh;
+}
+
 int prepare(const ma_fwd_params* p, Prepared* out) {
     ma_ws_layout L;
     int st = layout_of(p, &L);
@@ -320,13 +329,7 @@ int prepare(const ma_fwd_params* p, Prepared* out) {
     // with more, smaller problems or a state beyond the caches they cost 5-10 %.
     out->P.stream_stores = v == MA_VARIANT_STAGED && p->dtype_qk != MA_F32 && p->B > 32 && out->P.M > 32 &&
                            static_cast<long long>(p->E) * p->H * out->P.M * p->B <= 128 * 1024;
-    // Heads of at most 8 blocks: the per-stage L and Z kernels put 16 >> pack_shift in-block positions
-    // into one 16-row tile (2^pack_shift >= M rows each) instead of leaving most of the tile empty.
-    if (v == MA_VARIANT_STAGED && p->dtype_qk != MA_F32 && out->P.M <= 8) {
-        int sh = 0;
-        while ((1 << sh) < out->P.M) ++sh;
-        out->P.pack_shift = sh;
-    }
+    out->P.pack_shift = pack_shift_of(v, p, out->P.M);
     return MA_OK;
 }
 
@@ -596,6 +599,7 @@ int ma_bwd(const ma_bwd_params* b, void* stream) {
     pr.P = make_problem(&pp, none);
     pr.variant = v;
     Problem& P = pr.P;
+    P.pack_shift = pack_shift_of(v, &pp, P.M);   // the forward steps run again as per-stage launches
     if (!bwd_fits(P)) return MA_ERR_UNSUPPORTED;
     P.Y = ws + L.Y;
     P.stats = reinterpret_cast<float*>(ws + L.stats);
