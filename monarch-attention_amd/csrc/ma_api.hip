@@ -231,8 +231,10 @@ bool fused_full_width(const ma_fwd_params* p) {
 //  * else the chained kernel (one launch) from 32 heads on for blocks and block
 //    counts of at most 64: with many heads the wait of one head's phase is
 //    covered by other heads' problems; and for 128-row blocks AND block counts
-//    (c5: 184 us against 213 us) when the heads divide evenly over the 8 XCDs the
-//    kernel pins them to,
+//    (c5: 157 us against 203 us) when the heads divide evenly over the 8 XCDs the
+//    kernel pins them to; and for 97 .. 128 blocks of at most 96 rows with head
+//    dims up to 64 from 16 heads on (N = 8192 in 64-row blocks, 32 heads, T = 2:
+//    117 us against 127 us),
 //  * else one launch per half step (few tasks per head - block counts of 4 or 8
 //    with large blocks -, blocks of 65-96 rows, uneven head counts).
 int select_variant(const ma_fwd_params* p) {
@@ -255,6 +257,11 @@ int select_variant(const ma_fwd_params* p) {
                 if (heads >= 32 && p->B <= 64 && M <= 64 && chain_fits(p)) return MA_VARIANT_CHAINED;
                 // 128-row problems in both orientations (N of 10^4 and more), heads spread evenly over the XCDs
                 if (p->B > 96 && M > 96 && heads % 8 == 0 && chain_fits(p)) return MA_VARIANT_CHAINED;
+                // 97 .. 128 blocks of up to 96 rows, head dims up to 64 (long documents: N = 8192 in 64-row blocks):
+                // 0.83 - 0.96 of the per-stage time from 16 heads on (one step: from 32 heads on); wider heads,
+                // fewer heads and 65 .. 96 blocks (which the one-launch kernels run as 128) stay per stage
+                if (M > 96 && p->B <= 96 && p->D <= 64 && heads >= 16 && (p->T >= 2 || heads >= 32) && chain_fits(p))
+                    return MA_VARIANT_CHAINED;
             }
             return MA_VARIANT_STAGED;
     }

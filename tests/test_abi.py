@@ -183,6 +183,10 @@ def test_auto_variant_policy():
     assert auto(8, 16, 1024, 72, 32) == "chained"
     assert auto(4, 16, 16384, 64, 128) == "chained"
     assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for
+    assert auto(2, 16, 8192, 64, 64) == "chained"       # 128 blocks of 64 rows (long documents), head dim 64
+    assert auto(1, 12, 8192, 64, 64) == "staged"        # ... but not for fewer than 16 heads,
+    assert auto(2, 16, 8192, 128, 64) == "staged"       # wider heads,
+    assert auto(2, 16, 5000, 64, 64) == "staged"        # or 65 .. 96 blocks, which the one-launch kernels would run as 128
     assert auto(2, 2, 197, 64, 16) == "fused"           # few heads
     assert auto(1, 1, 16, 64, 4) == "staged"            # one workgroup per phase: nothing to fuse
     assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "staged"       # fp32 MFMA stage kernels
