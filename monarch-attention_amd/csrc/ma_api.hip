@@ -176,12 +176,14 @@ int run_resident(const Problem& P, int dtype_qk, bool dry_run, hipStream_t s) {
     return h ? launch_resident_f16_d8(P, dry_run, s) : launch_resident_bf16_d8(P, dry_run, s);
 }
 
-// Does a head's state fit in LDS (the resident kernel's condition)?
-bool resident_fits(const ma_fwd_params* p) {
+// Does a head's state fit in LDS (the resident kernel's condition)?  one_tile: also count the form that
+// keeps aL and aR in one tile and passes Y through the workspace.
+bool resident_fits(const ma_fwd_params* p, bool one_tile) {
     Problem P;
     std::memset(&P, 0, sizeof(P));
     P.E = p->E; P.H = p->H; P.N = p->N; P.D = p->D; P.Dv = p->Dv; P.B = p->B; P.T = p->T;
     P.M = (p->N + p->B - 1) / p->B;
+    P.one_tile_ok = one_tile ? 1 : 0;
     return run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
 }
 
@@ -223,7 +225,8 @@ bool fused_full_width(const ma_fwd_params* p) {
 // The variant a problem resolves to.  AUTO: the MFMA kernels when the problem
 // qualifies; among them (measured on MI355X)
 //  * the resident kernel when a head's state fits in LDS and there are enough
-//    heads to occupy the device with one workgroup per head,
+//    heads to occupy the device with one workgroup per head (its one-tile form,
+//    for heads of up to ~512 tokens, only for problems of one or two strips),
 //  * else the fused kernel (one launch, one team of workgroups per head) for fewer
 //    than 32 heads of problems of up to 64 rows when every head gets a full-width
 //    team at once (the metric workload: 18 us against 19.4 us for T = 1, 42 us
@@ -246,14 +249,20 @@ int select_variant(const ma_fwd_params* p) {
         case MA_VARIANT_STAGED: return fast || fast32 ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_FUSED: return fast ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_CHAINED: return fast && chain_fits(p) ? MA_VARIANT_CHAINED : MA_ERR_UNSUPPORTED;
-        case MA_VARIANT_RESIDENT: return fast && resident_fits(p) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_RESIDENT: return fast && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
         default:
             if (fast32) return MA_VARIANT_STAGED;
             if (!fast) return MA_VARIANT_GENERIC;
-            if (heads >= 128 && resident_fits(p)) return MA_VARIANT_RESIDENT;
+            if (heads >= 128 && resident_fits(p, false)) return MA_VARIANT_RESIDENT;
             if (fused_full_width(p)) return MA_VARIANT_FUSED;
             {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+                // one-tile form of the resident kernel: heads of up to ~512 tokens whose problems are one or two
+                // strips in one orientation and one in the other (16 waves per workgroup, every R phase in one or
+                // two rounds): 0.94 - 1.0 of the chained kernel's time at 192 heads, 0.84 at 768, with 0.6 of its
+                // traffic; larger problems run on 8 waves there and lose 15 - 40 %
+                if (heads >= 128 && ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && resident_fits(p, true))
+                    return MA_VARIANT_RESIDENT;
                 if (heads >= 32 && p->B <= 64 && M <= 64 && chain_fits(p)) return MA_VARIANT_CHAINED;
                 // 128-row problems in both orientations (N of 10^4 and more), heads spread evenly over the XCDs
                 if (p->B > 96 && M > 96 && heads % 8 == 0 && chain_fits(p)) return MA_VARIANT_CHAINED;
@@ -337,6 +346,7 @@ int prepare(const ma_fwd_params* p, Prepared* out) {
     out->P.stream_stores = v == MA_VARIANT_STAGED && p->dtype_qk != MA_F32 && p->B > 32 && out->P.M > 32 &&
                            static_cast<long long>(p->E) * p->H * out->P.M * p->B <= 128 * 1024;
     out->P.pack_shift = pack_shift_of(v, p, out->P.M);
+    out->P.one_tile_ok = 1;   // a problem that resolves to the resident kernel may use any of its forms
     return MA_OK;
 }
 

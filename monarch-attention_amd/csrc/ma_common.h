@@ -36,6 +36,9 @@ struct Problem {
     // Per-stage launches of heads with few blocks (M <= 8): a 16-row tile of an L / Z problem holds 16 >> pack_shift
     // in-block positions of pack_m = 1 << pack_shift rows each (4: one position per tile, as everywhere else).
     int pack_shift;
+    // The resident kernel may keep aL and aR in ONE LDS tile and pass Y through the workspace where two or
+    // three tiles do not fit (heads of up to ~512 tokens at d = 64).
+    int one_tile_ok;
     int test_no_spin;    // waits between workgroups give up at once (failure-path tests)
 };
 

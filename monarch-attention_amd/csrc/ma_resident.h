@@ -7,6 +7,11 @@
 // It applies when the state fits: two or three Np x D tiles (aL, aR, Y) plus the
 // operand staging of the problems in flight within the 160 KB of LDS, i.e. heads
 // of up to ~256 padded tokens at D = 64, and blocks / block counts of at most 64.
+// Heads of up to ~512 tokens run with ONE tile (kOneTile): aL and aR share it in
+// place - the R problem of block m reads the rows aR(m, .) and writes aL(., m)
+// over them, the L problem of position j reads aL(j, .) and writes aR(., j) over
+// those - and Y, which is written once and read once, goes through the caller's
+// workspace (the workgroup that wrote a head's Y is the one that reads it back).
 //
 // The head is processed as a sequence of ROUNDS; a round runs up to PPW block
 // problems of one phase concurrently on the workgroup's W waves (R phase: key
@@ -23,6 +28,7 @@
 //   SX  aR rows (m, j) -> m*B + j      read as the "aR[m]" rows of the R problems
 //   SY  Y  rows (j, m) -> j*M + m      read (transposed) by the Z problems; in aR's place when
 //       the last R phase is a single round (see y_on_x), else a tile of its own
+//   kOneTile: SA = SX, aL(j, m) and aR(m, j) both live in row m*B + j; no SY
 //   cLs[j*M + m], cRs[m*B + j] (fp32), ZR: one row of zeros that stands in for
 //   rows beyond the tile tails (k >= M, j >= B).
 #pragma once
@@ -32,7 +38,7 @@
 namespace ma {
 namespace mfma {
 
-template <class T, int DT, int NTB, int NTM, int W>
+template <class T, int DT, int NTB, int NTM, int W, bool ONE = false>
 struct Resident {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
@@ -52,14 +58,17 @@ struct Resident {
     // at a barrier, and only then write Y - so Y can take aR's place and the state is two tiles.
     // It costs that barrier, so it is only used where three tiles do not fit (the launcher decides).
     static __host__ __device__ bool y_on_x_possible(int M) { return M <= PPB; }
-    static __host__ __device__ size_t state_bytes(int Np, bool y_on_x) {   // SA, SX, (SY,) ZR, cLs, cRs
+    // how the state is kept: three tiles, two (Y in aR's place), or one (aL and aR in place, Y through memory)
+    enum { kThreeTiles = 0, kYOnX = 1, kOneTile = 2 };
+    static __host__ __device__ int tiles_of(int mode) { return mode == kOneTile ? 1 : mode == kYOnX ? 2 : 3; }
+    static __host__ __device__ size_t state_bytes(int Np, int mode) {   // SA, (SX,) (SY,) ZR, cLs, cRs
         const size_t np4 = (static_cast<size_t>(Np) + 3) / 4 * 4;
-        return ((y_on_x ? 2 : 3) * static_cast<size_t>(Np) + 1) * LD * sizeof(T) + 2 * np4 * sizeof(float);
+        return (tiles_of(mode) * static_cast<size_t>(Np) + 1) * LD * sizeof(T) + 2 * np4 * sizeof(float);
     }
     // staging is only needed for the problems a round can actually hold
-    static __host__ __device__ size_t lds_bytes(int Np, int M, int B, bool y_on_x) {
+    static __host__ __device__ size_t lds_bytes(int Np, int M, int B, int mode) {
         const size_t sr = static_cast<size_t>(M < PPB ? M : PPB) * kSlotR, sl = static_cast<size_t>(B < PPM ? B : PPM) * kSlotL;
-        return state_bytes(Np, y_on_x) + (sr > sl ? sr : sl);
+        return state_bytes(Np, mode) + (sr > sl ? sr : sl);
     }
 
     // registers that carry one round's global loads from issue to execute
@@ -77,14 +86,14 @@ struct Resident {
     };
     // start the loads of this thread's chunks of a tile of a problem with `nth` threads: rowoff(row)
     // is the row's byte offset in `src` or kOob; columns at or beyond D read as zero
-    template <class RowOff>
+    template <bool SHARED = false, class RowOff>
     static __device__ __forceinline__ void tile_issue(u32x4 (&val)[CNT], rsrc_t src, int D, RowOff rowoff, int tix, int nth) {
 #pragma unroll
         for (int i = 0; i < CNT; ++i) {
             const int c = tix + i * nth;
             const int row = c / CH, ch = c % CH;
             const unsigned ro = rowoff(row);
-            val[i] = bload16<false>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
+            val[i] = bload16<SHARED>(src, (ch * 8 < D) ? ro + ch * 16 : kOob);
         }
     }
     static __device__ __forceinline__ void tile_commit(T* tile, const u32x4 (&val)[CNT], int tix, int nth) {
@@ -106,7 +115,20 @@ struct Resident {
         char* stage;
         int wave, lane, r, q;
         bool y_on_x;   // Y shares the LDS of aR
+        // row of aL(j, m) (m < M, j < B); ONE (kOneTile): SA == SX, aL(j, m) and aR(m, j) share row m*B + j, Y is in the workspace
+        __device__ __forceinline__ T* al_row(int j, int m, int B, int M) const { return SA + (ONE ? m * B + j : j * M + m) * LD; }
     };
+    // the head's Y rows (j, m) -> j*M + m in the workspace (kOneTile)
+    static __device__ __forceinline__ rsrc_t y_slice(const Problem& P, int head) {
+        const long long bytes = static_cast<long long>(P.M) * P.B * P.D * static_cast<long long>(sizeof(T));
+        return make_rsrc(P.Y + head * bytes, static_cast<unsigned>(bytes));
+    }
+    // start the loads of the Y tile of position j of a Z problem (kOneTile)
+    static __device__ __forceinline__ void y_issue(const Problem& P, int head, u32x4 (&val)[CNT], int j, int tix) {
+        const unsigned db = static_cast<unsigned>(P.D) * sizeof(T);
+        const int M = P.M;
+        tile_issue<true>(val, y_slice(P, head), P.D, [&](int k) { return k < M ? static_cast<unsigned>(j * M + k) * db : kOob; }, tix, WPM * 64);
+    }
 
     static __device__ __forceinline__ int rounds_of(const Problem& P, int p) {
         return (p & 1) ? (P.B + PPM - 1) / PPM : (P.M + PPB - 1) / PPB;   // p odd: L or Z (positions j), p even: R (blocks m)
@@ -177,6 +199,9 @@ struct Resident {
             if (rd.p == nph - 1) {   // Z round: the strip's Q rows
                 const int l = 16 * wig + c.r;
                 load_x<T, DT, false>(pre.xq, S.q, l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob, D, c.q);
+                // Y from the workspace: complete once the last R phase has ended, i.e. for every Z round
+                // but the first, whose loads would start while that phase still runs (round_z loads them itself)
+                if constexpr (ONE) if (rd.rnd > 0) y_issue(P, rd.head, pre.a, j, tix);
             } else {                 // L round: the Q^T tile and the query mask of the strip's rows
                 tile_issue(pre.a, S.q, D, [&](int l) { return l < M ? tok_off(l * B + j - P.pad_off, P.N, S.qst) : kOob; }, tix, WPM * 64);
                 unsigned ok = 0;
@@ -284,14 +309,17 @@ struct Resident {
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                     for (int v = 0; v < 4; ++v) O[dt][v] = P.sm_scale * round_to<T>(O[dt][v]);
-                if (jv) lds_store_row(c.SA + lrow * LD, O, q);
+                if (jv) lds_store_row(c.al_row(j, m, B, M), O, q);
             }
             if (with_v) {
                 f32x4 O[DT];
                 gemm2<T, DT, NTB, true>(O, Vt, pb, r, q);
-                if (jv) lds_store_row(c.SY + lrow * LD, O, q);
+                if (ONE) store_row<T, DT, true>(y_slice(P, rd.head), jv ? static_cast<unsigned>(lrow) * (static_cast<unsigned>(P.D) * sizeof(T)) : kOob, P.D, O, q);
+                else if (jv) lds_store_row(c.SY + lrow * LD, O, q);
             }
         }
+        // Y rows in the workspace: written (acknowledged) before the barrier that ends the phase lets the Z rounds load them
+        if (ONE && with_v && rd.rnd + 1 == rounds_of(P, rd.p)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         round_end<WPB>(P, rd);
     }
 
@@ -324,7 +352,7 @@ struct Resident {
 #pragma unroll
             for (int kt = 0; kt < NTM; ++kt) {
                 const int k = 16 * kt + r;
-                const T* brow = k < M ? c.SA + (j * M + k) * LD : c.ZR;
+                const T* brow = k < M ? c.al_row(j, k, B, M) : c.ZR;
                 f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) acc = Ops<T>::mma(xa[ks], lds_row8<T>(brow + 32 * ks + 8 * q), acc);
@@ -411,8 +439,19 @@ struct Resident {
         const int j = rd.rnd * PPM + slot;
         const bool active = j < B;
         const int r = c.r, q = c.q;
-        float* cb = reinterpret_cast<float*>(c.stage + slot * kSlotL);
+        // staging as in an L round: the Y tile (kOneTile) where that has its Q^T tile, the bias behind the P^T tile
+        T* Yt = reinterpret_cast<T*>(c.stage + slot * kSlotL);
+        float* cb = reinterpret_cast<float*>(Yt + ROWSM * LD + ROWSM * LDP);
         if (active && tix < ROWSM) cb[tix] = tix < M ? -kLog2e * c.cLs[j * M + tix] : kNegBig;
+        if (ONE && active) {
+            if (rd.rnd == 0) {   // uniform: the first Z round loads its Y tile here, after the barrier that ended the last R phase
+                u32x4 ya[CNT];
+                y_issue(P, rd.head, ya, j, tix);
+                tile_commit(Yt, ya, tix, WPM * 64);
+            } else {
+                tile_commit(Yt, pre.a, tix, WPM * 64);
+            }
+        }
         problem_sync<WPM>();
         if (active) {
             const int e = rd.head / P.H, h = rd.head % P.H;
@@ -423,7 +462,7 @@ struct Resident {
 #pragma unroll
             for (int wt = 0; wt < NTM; ++wt) {
                 const int k = 16 * wt + r;
-                const T* arow = k < M ? c.SA + (j * M + k) * LD : c.ZR;
+                const T* arow = k < M ? c.al_row(j, k, B, M) : c.ZR;
                 f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) acc = Ops<T>::mma(lds_row8<T>(arow + 32 * ks + 8 * q), pre.xq[ks], acc);
@@ -462,8 +501,10 @@ struct Resident {
 #pragma unroll
                 for (int g = 0; g < (NTM + 1) / 2; ++g) {   // k slot s <-> key block 32g + 16(s/4) + 4q + s%4
                     const int lo = 32 * g + 4 * q + e4, hi = lo + 16;
-                    const T* p_lo = (lo < M ? c.SY + (j * M + lo) * LD : c.ZR) + chunk_col<DT, true>(c4, dt);
-                    const T* p_hi = (hi < M ? c.SY + (j * M + hi) * LD : c.ZR) + chunk_col<DT, true>(c4, dt);
+                    const T* ylo = ONE ? Yt + lo * LD : c.SY + (j * M + lo) * LD;
+                    const T* yhi = ONE ? Yt + hi * LD : c.SY + (j * M + hi) * LD;
+                    const T* p_lo = (lo < M ? ylo : c.ZR) + chunk_col<DT, true>(c4, dt);
+                    const T* p_hi = (hi < M ? yhi : c.ZR) + chunk_col<DT, true>(c4, dt);
                     acc = Ops<T>::mma(tr8(p_lo, p_hi), pb[g], acc);
                 }
                 O[dt] = acc;
@@ -480,21 +521,21 @@ struct Resident {
     }
 };
 
-template <class T, int DT, int NTB, int NTM, int W>
-__global__ __launch_bounds__(64 * W) void resident_fwd_mfma(Problem P, int y_on_x) {
-    using RS = Resident<T, DT, NTB, NTM, W>;
+template <class T, int DT, int NTB, int NTM, int W, bool ONE>
+__global__ __launch_bounds__(64 * W) void resident_fwd_mfma(Problem P, int mode) {
+    using RS = Resident<T, DT, NTB, NTM, W, ONE>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int Np = P.M * P.B;
     typename RS::Ctx c;
     c.SA = reinterpret_cast<T*>(smem);
-    c.y_on_x = y_on_x != 0;
-    const int tiles = c.y_on_x ? 2 : 3;
-    c.SX = c.SA + Np * RS::LD;
-    c.SY = c.y_on_x ? c.SX : c.SX + Np * RS::LD;
+    c.y_on_x = mode == RS::kYOnX;
+    const int tiles = RS::tiles_of(mode);
+    c.SX = ONE ? c.SA : c.SA + Np * RS::LD;
+    c.SY = c.y_on_x ? c.SX : c.SX + Np * RS::LD;   // unused with one tile
     c.ZR = c.SA + tiles * Np * RS::LD;
     c.cLs = reinterpret_cast<float*>(c.ZR + RS::LD);
     c.cRs = c.cLs + (Np + 3) / 4 * 4;
-    c.stage = smem + RS::state_bytes(Np, c.y_on_x);
+    c.stage = smem + RS::state_bytes(Np, mode);
     c.wave = wave_id();
     c.lane = threadIdx.x & 63;
     c.r = c.lane & 15;

@@ -14,20 +14,9 @@ constexpr size_t kLdsPerCu = 160 * 1024;
 constexpr int kResidentWaves = 8;       // workgroup size in waves ...
 constexpr int kResidentWavesWide = 16;  // ... and for blocks of up to 32 rows when the staging of 16 waves still fits
 
-template <class T, int DT, int NTB, int NTM, int W>
-int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
-    using RS = Resident<T, DT, NTB, NTM, W>;
-    const int Np = P.M * P.B;
-    // Y in a tile of its own if that fits, else in aR's place where the kernel allows it
-    bool y_on_x = false;
-    size_t lds = RS::lds_bytes(Np, P.M, P.B, false);
-    if (lds > kLdsPerCu && RS::y_on_x_possible(P.M)) {
-        y_on_x = true;
-        lds = RS::lds_bytes(Np, P.M, P.B, true);
-    }
-    if (lds > kLdsPerCu) return MA_ERR_UNSUPPORTED;   // the head's state does not fit in LDS
-    if (dry_run) return MA_OK;
-    auto kernel = resident_fwd_mfma<T, DT, NTB, NTM, W>;
+template <class T, int DT, int NTB, int NTM, int W, bool ONE>
+int launch_resident_mode(const Problem& P, int mode, size_t lds, hipStream_t s) {
+    auto kernel = resident_fwd_mfma<T, DT, NTB, NTM, W, ONE>;
     const int lds_err = set_lds_limit(kernel, kLdsPerCu);
     if (lds_err) return lds_err;
     const DeviceCaps caps = device_caps(kernel, 0, 0);
@@ -39,8 +28,30 @@ int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
     const long long per_cu = lds * 2 <= kLdsPerCu ? 2 : 1;
     long long grid = caps.cus * per_cu;
     if (grid > heads) grid = heads;
-    hipLaunchKernelGGL((resident_fwd_mfma<T, DT, NTB, NTM, W>), dim3(grid), dim3(64 * W), lds, s, P, y_on_x ? 1 : 0);
+    hipLaunchKernelGGL((resident_fwd_mfma<T, DT, NTB, NTM, W, ONE>), dim3(grid), dim3(64 * W), lds, s, P, mode);
     return static_cast<int>(hipGetLastError());
+}
+
+template <class T, int DT, int NTB, int NTM, int W>
+int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
+    using RS = Resident<T, DT, NTB, NTM, W>;
+    const int Np = P.M * P.B;
+    // Y in a tile of its own if that fits, else in aR's place where the kernel allows it, else
+    // aL and aR in one tile and Y through the workspace
+    int mode = RS::kThreeTiles;
+    size_t lds = RS::lds_bytes(Np, P.M, P.B, mode);
+    if (lds > kLdsPerCu && RS::y_on_x_possible(P.M)) {
+        mode = RS::kYOnX;
+        lds = RS::lds_bytes(Np, P.M, P.B, mode);
+    }
+    if (lds > kLdsPerCu && P.one_tile_ok) {
+        mode = RS::kOneTile;
+        lds = RS::lds_bytes(Np, P.M, P.B, mode);
+    }
+    if (lds > kLdsPerCu) return MA_ERR_UNSUPPORTED;   // the head's state does not fit in LDS
+    if (dry_run) return MA_OK;
+    return mode == RS::kOneTile ? launch_resident_mode<T, DT, NTB, NTM, W, true>(P, mode, lds, s)
+                                : launch_resident_mode<T, DT, NTB, NTM, W, false>(P, mode, lds, s);
 }
 
 // The problems of a head are small and latency-bound: more waves per workgroup run more of

@@ -179,7 +179,9 @@ def test_auto_variant_policy():
     assert auto(1, 12, 16384, 64, 128) == "staged"      # 12 heads on 8 XCDs: uneven
     assert auto(16, 12, 512, 64, 128) == "staged"       # 128-row blocks, but only 4 of them per head
     assert auto(64, 12, 197, 64, 16) == "resident"
-    assert auto(16, 12, 512, 64, 32) == "chained"      # state of a 512-token head does not fit in LDS
+    assert auto(16, 12, 512, 64, 32) == "resident"     # 512-token heads: aL / aR in one LDS tile, Y through the workspace
+    assert auto(8, 12, 512, 64, 32) == "chained"       # ... from 128 heads on
+    assert auto(16, 12, 512, 64, 64) == "chained"      # ... and for problems of one or two strips
     assert auto(8, 16, 1024, 72, 32) == "chained"
     assert auto(4, 16, 16384, 64, 128) == "chained"
     assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for

@@ -180,6 +180,29 @@ def test_heads_of_few_blocks(E, H, N, D, B, T, pre, dt, masked, variant):
     assert_parity(out.cpu(), ref, dt, f"few blocks {(E, H, N, D, B, T, pre, dt, masked)}/{variant}")
 
 
+ONE_TILE = [  # E, H, N, D, B, T, pre, dt, masked: heads whose aL / aR / Y do not fit in LDS as three (or two) tiles
+    (2, 3, 512, 64, 32, 2, False, "bf16", False), (1, 4, 500, 64, 32, 3, True, "f16", True),
+    (1, 2, 384, 64, 24, 1, False, "f16", True), (2, 2, 448, 64, 16, 2, True, "bf16", False),
+    (1, 3, 300, 72, 20, 2, False, "f16", True), (1, 2, 1000, 32, 32, 2, False, "f16", False),
+    (1, 2, 512, 64, 64, 2, False, "f16", True), (1, 2, 470, 64, 48, 2, True, "bf16", False),
+    (30, 12, 400, 64, 25, 2, False, "f16", True),   # more heads than workgroups: a workgroup walks several heads
+]
+
+
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", ONE_TILE)
+def test_resident_kernel_with_one_state_tile(E, H, N, D, B, T, pre, dt, masked):
+    """Heads of ~300 .. 1000 tokens in the resident kernel: aL and aR share one LDS tile in place and Y goes
+    through the workspace."""
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
+    mask = block_safe_mask(E, N, B, seed=B) if masked else None
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
+    dev = to_dev(q, k, v, mask)
+    out = monarch_attention_hip(*dev, T, B, pre, variant="resident")   # the variant must take these shapes
+    assert_parity(out.cpu(), ref, dt, f"one-tile resident {(E, H, N, D, B, T, pre, dt, masked)}")
+    again = monarch_attention_hip(*dev, T, B, pre, variant="resident")
+    assert torch.equal(out, again)
+
+
 def test_broadcast_over_tokens_is_accepted():
     """expand()-ed inputs (stride 0 along N) are legal for the reference (it pads, i.e. copies); the
     operator takes them too, by making the one copy the library's row-overlap check asks for."""
