@@ -67,7 +67,9 @@ typedef enum ma_variant {
                             /* longer than the bounded waits (about a millisecond)   */
                             /* makes the call fail loudly (NaN rows + error word)    */
     MA_VARIANT_RESIDENT = 4,/* MFMA, ONE launch, one workgroup per head with the     */
-                            /* whole per-head state resident in LDS (small heads)    */
+                            /* per-head state resident in LDS (heads of up to ~256   */
+                            /* tokens at d = 64; up to ~512 with Y passed through    */
+                            /* the workspace)                                        */
     MA_VARIANT_CHAINED = 5  /* MFMA, ONE launch, one workgroup per block problem of  */
                             /* every phase; a problem starts when its head's         */
                             /* previous phase has released it through the workspace. */
