@@ -207,14 +207,16 @@ __device__ __forceinline__ typename Ops<T>::v8 lds_row8(const T* tile_elem) {
 
 // Which tile columns a lane ends up with after GEMM2: the first of the four consecutive columns
 // that lane group g (r/4 of an MFMA row on the operand side, q of a lane on the result side) has in
-// output tile dt.  Even DT: tiles 2p and 2p+1 give a lane the 8 columns 8*(g + 4p) .., a 16-byte
-// piece, and the four lane groups of a row write 64 contiguous bytes with each store instruction.
-// Odd DT, or RUN (the kernel that keeps its state in LDS and writes little to memory asks for it:
-// it is at its register limit and this form costs it three registers fewer): a lane's 4*DT columns
-// are one consecutive run, 4*DT*g ...
+// output tile dt.  Tiles 2p and 2p+1 give a lane the 8 columns 8*(g + 4p) .., a 16-byte piece, and
+// the four lane groups of a row write 64 contiguous bytes with each store instruction; the last
+// tile of an odd DT gives the lane groups the 4-column pieces behind those, 32 contiguous bytes.
+// RUN (the kernel that keeps its state in LDS and writes little to memory asks for it: it is at
+// its register limit and this form costs it three registers fewer): a lane's 4*DT columns are one
+// consecutive run, 4*DT*g ...
 template <int DT, bool RUN = false>
 __host__ __device__ constexpr int chunk_col(int g, int dt) {
-    return (DT % 2 == 0 && !RUN) ? 8 * g + 32 * (dt >> 1) + 4 * (dt & 1) : 4 * DT * g + 4 * dt;
+    return RUN ? 4 * DT * g + 4 * dt
+               : (DT % 2 == 1 && dt == DT - 1) ? 16 * (DT - 1) + 4 * g : 8 * g + 32 * (dt >> 1) + 4 * (dt & 1);
 }
 
 // Transposed A operand of GEMM2 from a row-major LDS tile via ds_read_b64_tr_b16.
@@ -266,9 +268,11 @@ __device__ __forceinline__ void gemm2(f32x4 (&O)[DT], const T* tile, const typen
     }
 }
 
-// Store a lane's 4*DT output elements (columns chunk_col(q, dt) ..) of the row at
-// byte offset ro (kOob drops the store): 16-byte pieces when the head dim fills the
-// tiles exactly, else 8-byte pieces so that a piece never straddles D.
+// Store a lane's 4*DT output elements (columns chunk_col(q, dt) ..) of the row at byte offset ro
+// (kOob drops the store) in 16-byte pieces - 8 columns at a multiple of 8, so with D a multiple of
+// 8 (a condition of these kernels) a piece lies wholly inside or wholly beyond the row - plus one
+// 8-byte piece per lane for the last tile of an odd DT.  (RUN: 16-byte pieces when the head dim
+// fills the tiles exactly, else 8-byte pieces.)
 // stream: the rows are whole 128-byte lines (see Slices::stream_*): they are written with
 // streaming ("nt") stores, which leave for memory while the kernel still runs.  Plain stores
 // are acknowledged early and the launch then ends with a long drain of its written lines
@@ -279,15 +283,23 @@ template <class T, int DT, bool RUN = false>
 __device__ __forceinline__ void store_row(rsrc_t dst, unsigned ro, int D, const f32x4 (&O)[DT], int q, bool stream = false) {
     typedef typename Ops<T>::v4 V4;
     const unsigned base = ro + 2 * chunk_col<DT, RUN>(q, 0);  // bytes; the pieces sit at fixed distances from it
-    if (DT % 2 == 0 && D == 16 * DT) {
+    const bool whole = D == 16 * DT;   // no piece lies beyond the row
+    if (!RUN || (DT % 2 == 0 && whole)) {
 #pragma unroll
         for (int p = 0; p < DT / 2; ++p) {
             V4 a = {from_f<T>(O[2 * p][0]), from_f<T>(O[2 * p][1]), from_f<T>(O[2 * p][2]), from_f<T>(O[2 * p][3])};
             V4 b = {from_f<T>(O[2 * p + 1][0]), from_f<T>(O[2 * p + 1][1]), from_f<T>(O[2 * p + 1][2]), from_f<T>(O[2 * p + 1][3])};
             const u32x2 lo = __builtin_bit_cast(u32x2, a), hi = __builtin_bit_cast(u32x2, b);
             const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
-            if (stream) __builtin_amdgcn_raw_buffer_store_b128(v, dst, base + 2 * (chunk_col<DT, RUN>(0, 2 * p) - chunk_col<DT, RUN>(0, 0)), 0, 2);
-            else __builtin_amdgcn_raw_buffer_store_b128(v, dst, base + 2 * (chunk_col<DT, RUN>(0, 2 * p) - chunk_col<DT, RUN>(0, 0)), 0, 0);
+            unsigned off = base + 2 * (chunk_col<DT, RUN>(0, 2 * p) - chunk_col<DT, RUN>(0, 0));
+            if (!whole) off = chunk_col<DT, RUN>(q, 2 * p) < D ? off : kOob;
+            if (stream) __builtin_amdgcn_raw_buffer_store_b128(v, dst, off, 0, 2);
+            else __builtin_amdgcn_raw_buffer_store_b128(v, dst, off, 0, 0);
+        }
+        if (DT % 2 == 1) {
+            V4 a = {from_f<T>(O[DT - 1][0]), from_f<T>(O[DT - 1][1]), from_f<T>(O[DT - 1][2]), from_f<T>(O[DT - 1][3])};
+            const int d0 = chunk_col<DT, RUN>(q, DT - 1);
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, a), dst, d0 < D ? ro + 2 * d0 : kOob, 0, 0);
         }
     } else {
 #pragma unroll
