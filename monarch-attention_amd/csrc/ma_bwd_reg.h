@@ -36,6 +36,37 @@ struct RBwdReg {
     static constexpr size_t kLds = 5 * static_cast<size_t>(TILE) * sizeof(T) + kStats * ROWS * sizeof(float);
 };
 
+
+// A lane's 4*DT results of one row as 16-bit elements at dst (the row's first element).  Tiles 2p and 2p+1
+// hold 8 consecutive columns (mfma::chunk_col): they go out as ONE 16-byte piece where the row allows it (D a
+// multiple of 8, the piece 16-byte aligned), so that the four lane groups of a row write 64 contiguous bytes
+// with one instruction; else, and for the last tile of an odd DT, as 8-byte pieces.
+template <class T, int DT>
+__device__ __forceinline__ void store_row16(T* dst, int D, const f32x4 (&O)[DT], int q) {
+    typedef typename mfma::Ops<T>::v4 V4;
+    const bool wide = D % 8 == 0 && (reinterpret_cast<unsigned long long>(dst) & 15ull) == 0;
+#pragma unroll
+    for (int p = 0; p < DT / 2; ++p) {
+        const int d0 = mfma::chunk_col<DT>(q, 2 * p);   // d0 + 4 == chunk_col(q, 2 * p + 1)
+        const V4 a = {from_f<T>(O[2 * p][0]), from_f<T>(O[2 * p][1]), from_f<T>(O[2 * p][2]), from_f<T>(O[2 * p][3])};
+        const V4 b = {from_f<T>(O[2 * p + 1][0]), from_f<T>(O[2 * p + 1][1]), from_f<T>(O[2 * p + 1][2]), from_f<T>(O[2 * p + 1][3])};
+        if (wide) {
+            if (d0 < D) {
+                const mfma::u32x2 lo = __builtin_bit_cast(mfma::u32x2, a), hi = __builtin_bit_cast(mfma::u32x2, b);
+                *reinterpret_cast<mfma::u32x4*>(dst + d0) = mfma::u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+        } else {
+            if (d0 < D) *reinterpret_cast<V4*>(dst + d0) = a;
+            if (d0 + 4 < D) *reinterpret_cast<V4*>(dst + d0 + 4) = b;
+        }
+    }
+    if (DT % 2 == 1) {
+        const int d0 = mfma::chunk_col<DT>(q, DT - 1);
+        const V4 a = {from_f<T>(O[DT - 1][0]), from_f<T>(O[DT - 1][1]), from_f<T>(O[DT - 1][2]), from_f<T>(O[DT - 1][3])};
+        if (d0 < D) *reinterpret_cast<V4*>(dst + d0) = a;
+    }
+}
+
 // O[dt] += sum_w tile[w][4*DT*q + 4*dt + v] * P[w][lane column]   (gemm2 of ma_mfma.h, accumulating)
 template <class T, int DT, int NWT>
 __device__ __forceinline__ void gemm2_acc(f32x4 (&O)[DT], const T* tile, const typename mfma::Ops<T>::v8 (&pb)[(NWT + 1) / 2], int r, int q) {
@@ -184,12 +215,12 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
         g = (key_in && ru >= kTiny) ? fmaf(gcl, d + lg1, gg) : 0.f;
     };
 
-    // four consecutive elements of a finished gradient, rounded into the caller's tensor `which` (0 dq, 1 dk,
-    // 2 dv) at token t; padding positions have no row there
-    auto emit = [&](int which, int t, int d0, const f32x4& val) {
+    // a finished gradient row is rounded straight into the caller's tensor `which` (0 dq, 1 dk, 2 dv) at token t;
+    // padding positions have no row there
+    auto emit = [&](int which, int t, const f32x4 (&val)[DT]) {
         if (t < 0 || t >= P.N) return;
-        T* y = reinterpret_cast<T*>(G.out[which]) + e * G.outs[which][0] + h * G.outs[which][1] + t * G.outs[which][2] + d0;
-        *reinterpret_cast<V4*>(y) = V4{from_f<T>(val[0]), from_f<T>(val[1]), from_f<T>(val[2]), from_f<T>(val[3])};
+        T* y = reinterpret_cast<T*>(G.out[which]) + e * G.outs[which][0] + h * G.outs[which][1] + t * G.outs[which][2];
+        store_row16<T, DT>(y, D, val, q);
     };
 
     // ---- pass 1: this wave's strip of query rows (accumulator rows = keys)
@@ -272,20 +303,23 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
         f32x4 O[DT];
         mfma::gemm2<T, DT, NWT>(O, Kt, pb, r, q);
         if (jv) {
+            if (first) {   // dq is complete with this stage's part
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const int d0 = mfma::chunk_col<DT>(q, dt);
-                if (d0 >= D) continue;   // D is a multiple of 4 (checked by the launcher)
-                if (first) {
+                for (int dt = 0; dt < DT; ++dt) {
+                    const int d0 = mfma::chunk_col<DT>(q, dt);
+                    if (d0 >= D) continue;   // D is a multiple of 4 (checked by the launcher)
                     f32x4* dst = reinterpret_cast<f32x4*>(G.dq + (blk + j) * D + d0);
-                    const f32x4 total = *dst + O[dt];
-                    if (G.direct) emit(0, k * B + j - P.pad_off, d0, total);   // dq is complete
-                    else *dst = total;
-                } else if (S16) {
-                    const V4 o = {from_f<T>(O[dt][0]), from_f<T>(O[dt][1]), from_f<T>(O[dt][2]), from_f<T>(O[dt][3])};
-                    *reinterpret_cast<V4*>(reinterpret_cast<T*>(G.gaR) + (blk + j) * D + d0) = o;
-                } else {
-                    *reinterpret_cast<f32x4*>(G.gaR + (blk + j) * D + d0) = O[dt];
+                    O[dt] += *dst;
+                    if (!G.direct) *dst = O[dt];
+                }
+                if (G.direct) emit(0, k * B + j - P.pad_off, O);
+            } else if (S16) {
+                store_row16<T, DT>(reinterpret_cast<T*>(G.gaR) + (blk + j) * D, D, O, q);
+            } else {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const int d0 = mfma::chunk_col<DT>(q, dt);
+                    if (d0 < D) *reinterpret_cast<f32x4*>(G.gaR + (blk + j) * D + d0) = O[dt];
                 }
             }
         }
@@ -333,26 +367,29 @@ __global__ __launch_bounds__(64 * NWT) void r_bwd_reg(Problem P, BwdBuffers G, i
         mfma::gemm2<T, DT, NWT>(O, Gat, pr, r, q);
         gemm2_acc<T, DT, NWT>(O, Xt, pd, r, q);
         if (key_in) {
+            const bool done = first && G.direct;   // dk is complete: it goes to the caller's tensor
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const int d0 = mfma::chunk_col<DT>(q, dt);
                 if (d0 >= D) continue;
                 f32x4* dst = reinterpret_cast<f32x4*>(G.dk + (blk + i) * D + d0);
                 // the stage that also forms dv is the first R stage of a backward pass: it starts dk's sums
-                const f32x4 total = with_v ? O[dt] : *dst + O[dt];
-                if (first && G.direct) emit(1, k * B + i - P.pad_off, d0, total);   // dk is complete
-                else *dst = total;
+                if (!with_v) O[dt] += *dst;
+                if (!done) *dst = O[dt];
             }
+            if (done) emit(1, k * B + i - P.pad_off, O);
         }
         if (with_v) {   // dV[i] = sum_j round(r)[j,i] gY[j]: this stage is dv's only writer
             mfma::gemm2<T, DT, NWT>(O, Gyt, pr, r, q);
             if (key_in) {
+                if (G.direct) {
+                    emit(2, k * B + i - P.pad_off, O);
+                } else {
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const int d0 = mfma::chunk_col<DT>(q, dt);
-                    if (d0 >= D) continue;
-                    if (G.direct) emit(2, k * B + i - P.pad_off, d0, O[dt]);
-                    else *reinterpret_cast<f32x4*>(G.dv + (blk + i) * D + d0) = O[dt];
+                    for (int dt = 0; dt < DT; ++dt) {
+                        const int d0 = mfma::chunk_col<DT>(q, dt);
+                        if (d0 < D) *reinterpret_cast<f32x4*>(G.dv + (blk + i) * D + d0) = O[dt];
+                    }
                 }
             }
         }
@@ -580,16 +617,14 @@ __global__ __launch_bounds__(64 * NWT) void lz_bwd_reg(Problem P, BwdBuffers G) 
         f32x4 O[DT];
         auto store_state = [&](float* base32) {   // row (j, k) of gaL / gY, in the operand dtype or fp32
             if (!kin) return;
+            if (S16) {
+                store_row16<T, DT>(reinterpret_cast<T*>(base32) + (jm + k) * D, D, O, q);
+                return;
+            }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const int d0 = mfma::chunk_col<DT>(q, dt);
-                if (d0 >= D) continue;
-                if (S16) {
-                    const V4 o = {from_f<T>(O[dt][0]), from_f<T>(O[dt][1]), from_f<T>(O[dt][2]), from_f<T>(O[dt][3])};
-                    *reinterpret_cast<V4*>(reinterpret_cast<T*>(base32) + (jm + k) * D + d0) = o;
-                } else {
-                    *reinterpret_cast<f32x4*>(base32 + (jm + k) * D + d0) = O[dt];
-                }
+                if (d0 < D) *reinterpret_cast<f32x4*>(base32 + (jm + k) * D + d0) = O[dt];
             }
         };
         mfma::gemm2<T, DT, NWT>(O, Qt, pd, r, q);   // gaL[j,k] = sum_l dU[l,k] Q[l]
