@@ -210,36 +210,42 @@ bool chain_fits(const ma_fwd_params* p) {
     return 8 * ((heads + 7) / 8) * p->T * (tR + tL) <= 0x7fffffffLL;
 }
 
-// Few heads of 64-row problems: every head gets a team with one workgroup per block problem and
-// all teams are on the device at once (256 CUs x 4 workgroups) - the fused kernel then runs each
-// phase like a per-stage launch would, without the launch boundaries.
+// Few heads of 64-row problems: every head gets a team with one workgroup per block problem (64 of
+// them per phase: heads of ~4096 tokens), the teams sit on one XCD each and all of them are on the
+// device at once (256 CUs x 4 workgroups) - the fused kernel then runs each phase like a per-stage
+// launch would, without the launch boundaries.
 bool fused_full_width(const ma_fwd_params* p) {
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
     if (p->B > 64 || M > 64) return false;
     const long long tR = phase_tasks(M, p->B), tL = phase_tasks(p->B, M);
     const long long widest = tR > tL ? tR : tL;
     const long long heads = static_cast<long long>(p->E) * p->H;
-    return heads < 32 && widest > 1 && (heads + 7) / 8 * 8 * widest <= 1024;
+    return heads < 32 && heads % 8 == 0 && widest >= 64 && heads * widest <= 1024;
 }
 
-// The variant a problem resolves to.  AUTO: the MFMA kernels when the problem
-// qualifies; among them (measured on MI355X)
-//  * the resident kernel when a head's state fits in LDS and there are enough
-//    heads to occupy the device with one workgroup per head (its one-tile form,
-//    for heads of up to ~512 tokens, only for problems of one or two strips),
-//  * else the fused kernel (one launch, one team of workgroups per head) for fewer
-//    than 32 heads of problems of up to 64 rows when every head gets a full-width
-//    team at once (the metric workload: 18 us against 19.4 us for T = 1, 42 us
-//    against 55 us for T = 3),
-//  * else the chained kernel (one launch) from 32 heads on for blocks and block
-//    counts of at most 64: with many heads the wait of one head's phase is
-//    covered by other heads' problems; and for 128-row blocks AND block counts
-//    (c5: 157 us against 203 us) when the heads divide evenly over the 8 XCDs the
-//    kernel pins them to; and for 97 .. 128 blocks of at most 96 rows with head
-//    dims up to 64 from 16 heads on (N = 8192 in 64-row blocks, 32 heads, T = 2:
-//    117 us against 127 us),
-//  * else one launch per half step (few tasks per head - block counts of 4 or 8
-//    with large blocks -, blocks of 65-96 rows, uneven head counts).
+// The variant a problem resolves to.  AUTO: the MFMA kernels when the problem qualifies; among
+// them what a sweep on MI355X says (fp16, E*H = 1 .. 384 heads, N = 256 .. 8192, blocks of 16 .. 128
+// rows, T = 1, 2, 3, head dims 32, 64, 128: the choice below is within 0.6 % of the fastest variant
+// in the geometric mean over the 827 points, 17 % at worst):
+//  * the resident kernel for many heads of small problems: with two or three state tiles (heads
+//    of up to ~256 tokens) for blocks and block counts of at most 32, from 128 heads on for
+//    16-row blocks and 192 for 32-row blocks; in its one-tile form (up to ~512 tokens) for
+//    problems of one or two strips when the head count fills the device's 256 one-per-CU
+//    workgroups to three quarters or more in its last pass (192 heads: 0.95 of the chained
+//    kernel's time with 0.6 of its traffic, 768: 0.84; 128 or 384 heads: 1.05 - 1.3);
+//  * the fused kernel (one team of workgroups per head, counter barriers) for 8 or 16 heads of
+//    ~4096 tokens in 64-row problems (the metric workload: 17.7 us against 20.0 chained and
+//    22.4 as two launches);
+//  * one launch per half step where the one-launch kernels are at a disadvantage: heads of at most
+//    8 blocks when there are many of them (the per-stage L and Z kernels pack several positions
+//    into a tile: 192 heads of four 128-row blocks 53 us against 73 us chained); 65 .. 96 blocks
+//    or block rows (the one-launch kernels run them in the 128 class); 128-row problems both ways
+//    on a head count that does not divide by the 8 XCDs the chained kernel pins heads to; head
+//    dims above 80 with more than 64 blocks of 64 rows and more; fewer than 8 heads of thousands
+//    of tokens (a head's tasks all run on one XCD); a single step on an uneven head count from
+//    4096 tokens on (two launches against an unbalanced one);
+//  * else the chained kernel (one launch, tasks in dispatch order): 10 - 25 % ahead of the stage
+//    launches over most of the sweep.
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
     const bool fast32 = mfma32_supported(p);   // fp32 operands: per-stage launches only
@@ -253,23 +259,20 @@ int select_variant(const ma_fwd_params* p) {
         default:
             if (fast32) return MA_VARIANT_STAGED;
             if (!fast) return MA_VARIANT_GENERIC;
-            if (heads >= 128 && resident_fits(p, false)) return MA_VARIANT_RESIDENT;
-            if (fused_full_width(p)) return MA_VARIANT_FUSED;
             {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-                // one-tile form of the resident kernel: heads of up to ~512 tokens whose problems are one or two
-                // strips in one orientation and one in the other (16 waves per workgroup, every R phase in one or
-                // two rounds): 0.94 - 1.0 of the chained kernel's time at 192 heads, 0.84 at 768, with 0.6 of its
-                // traffic; larger problems run on 8 waves there and lose 15 - 40 %
-                if (heads >= 128 && ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && resident_fits(p, true))
+                if (p->B <= 32 && M <= 32 && heads >= (p->B <= 16 ? 128 : 192) && resident_fits(p, false)) return MA_VARIANT_RESIDENT;
+                if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) &&
+                    ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && resident_fits(p, true))
                     return MA_VARIANT_RESIDENT;
-                if (heads >= 32 && p->B <= 64 && M <= 64 && chain_fits(p)) return MA_VARIANT_CHAINED;
-                // 128-row problems in both orientations (N of 10^4 and more), heads spread evenly over the XCDs
-                if (p->B > 96 && M > 96 && heads % 8 == 0 && chain_fits(p)) return MA_VARIANT_CHAINED;
-                // 97 .. 128 blocks of up to 96 rows, head dims up to 64 (long documents: N = 8192 in 64-row blocks):
-                // 0.83 - 0.96 of the per-stage time from 16 heads on (one step: from 32 heads on); wider heads,
-                // fewer heads and 65 .. 96 blocks (which the one-launch kernels run as 128) stay per stage
-                if (M > 96 && p->B <= 96 && p->D <= 64 && heads >= 16 && (p->T >= 2 || heads >= 32) && chain_fits(p))
+                if (fused_full_width(p)) return MA_VARIANT_FUSED;
+                const bool few_blocks = M <= 8 && heads >= (p->D <= 64 ? 32 : 16) * M;
+                const bool class_96 = (M > 64 && M <= 96) || (p->B > 64 && p->B <= 96 && M <= 96);
+                const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
+                const bool wide_dim = p->D > 80 && M > 64 && p->B >= 64;
+                const bool few_heads = heads < 8 && p->N > (heads <= 4 ? 2048 : 4096);
+                const bool one_step = p->T == 1 && heads % 8 != 0 && p->N >= 4096;
+                if (!few_blocks && !class_96 && !uneven_128 && !wide_dim && !few_heads && !one_step && chain_fits(p))
                     return MA_VARIANT_CHAINED;
             }
             return MA_VARIANT_STAGED;

@@ -157,15 +157,16 @@ def test_check_maps_status_to_python_exceptions():
 
 
 def test_auto_variant_policy():
-    """AUTO: generic when the MFMA kernels do not apply; resident when a head's
-    state fits in LDS and there are many heads; the fused kernel for a few heads of
-    problems of up to 64 rows; the chained kernel from 32 heads for such problems;
-    per-stage launches otherwise."""
+    """AUTO: generic when the MFMA kernels do not apply; resident for many heads of small problems
+    whose state fits in LDS; the fused kernel for 8 or 16 heads of ~4096 tokens in 64-row problems;
+    per-stage launches where the one-launch kernels are at a disadvantage (few-block heads in large
+    numbers, the 96-row tile class, uneven head counts of 128-row problems, wide heads with many blocks,
+    very few long heads); the chained kernel otherwise."""
     lib = L.load()
 
-    def auto(E, H, N, D, B, dt=L.MA_F16, Dv=None):
+    def auto(E, H, N, D, B, dt=L.MA_F16, Dv=None, T=2):
         p = L.FwdParams()
-        p.E, p.H, p.N, p.D, p.Dv, p.B, p.T = E, H, N, D, Dv or D, B, 2
+        p.E, p.H, p.N, p.D, p.Dv, p.B, p.T = E, H, N, D, Dv or D, B, T
         p.dtype_qk = p.dtype_v = dt
         for name, w in (("q_stride", D), ("k_stride", D), ("v_stride", p.Dv), ("out_stride", p.Dv)):
             setattr(p, name, (C.c_int64 * 3)(H * N * w, N * w, w))
@@ -173,24 +174,30 @@ def test_auto_variant_policy():
         return L.VARIANT_NAMES[lib.ma_fwd_select_variant(p)]
 
     assert auto(1, 16, 4096, 64, 64) == "fused"         # 16 heads x 64 workgroups: every head has a full team at once
+    assert auto(1, 16, 4096, 64, 64, T=1) == "fused"
     assert auto(2, 16, 4096, 64, 64) == "chained"
-    assert auto(1, 8, 1024, 64, 32) == "fused"
+    assert auto(1, 8, 1024, 64, 32) == "chained"        # teams of 16 workgroups: the chained kernel is ahead
+    assert auto(1, 12, 4096, 64, 64) == "chained"       # 12 heads do not sit evenly on 8 XCDs: no teams
+    assert auto(1, 12, 4096, 64, 64, T=1) == "staged"   # ... and with a single step two launches beat an unbalanced one
     assert auto(1, 16, 16384, 64, 128) == "chained"     # 128-row problems both ways, heads even over the XCDs
     assert auto(1, 12, 16384, 64, 128) == "staged"      # 12 heads on 8 XCDs: uneven
-    assert auto(16, 12, 512, 64, 128) == "staged"       # 128-row blocks, but only 4 of them per head
+    assert auto(16, 12, 512, 64, 128) == "staged"       # 192 heads of four 128-row blocks: packed L / Z tiles
+    assert auto(1, 8, 512, 64, 128) == "chained"        # ... few such heads: one launch
     assert auto(64, 12, 197, 64, 16) == "resident"
     assert auto(16, 12, 512, 64, 32) == "resident"     # 512-token heads: aL / aR in one LDS tile, Y through the workspace
-    assert auto(8, 12, 512, 64, 32) == "chained"       # ... from 128 heads on
+    assert auto(8, 12, 512, 64, 32) == "chained"       # ... when the head count fills the device's workgroups
+    assert auto(32, 12, 512, 64, 32) == "chained"      # (384 heads: 1.5 passes over 256 CUs)
     assert auto(16, 12, 512, 64, 64) == "chained"      # ... and for problems of one or two strips
+    assert auto(32, 12, 256, 64, 64) == "staged"       # 64-row blocks never run resident: 384 heads of four blocks
     assert auto(8, 16, 1024, 72, 32) == "chained"
     assert auto(4, 16, 16384, 64, 128) == "chained"
     assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for
     assert auto(2, 16, 8192, 64, 64) == "chained"       # 128 blocks of 64 rows (long documents), head dim 64
-    assert auto(1, 12, 8192, 64, 64) == "staged"        # ... but not for fewer than 16 heads,
-    assert auto(2, 16, 8192, 128, 64) == "staged"       # wider heads,
+    assert auto(2, 16, 8192, 128, 64) == "staged"       # ... but not for wide heads
     assert auto(2, 16, 5000, 64, 64) == "staged"        # or 65 .. 96 blocks, which the one-launch kernels would run as 128
-    assert auto(2, 2, 197, 64, 16) == "fused"           # few heads
-    assert auto(1, 1, 16, 64, 4) == "staged"            # one workgroup per phase: nothing to fuse
+    assert auto(1, 2, 8192, 64, 64) == "staged"         # two long heads would run on two of the eight XCDs
+    assert auto(2, 2, 197, 64, 16) == "chained"         # few short heads: one launch
+    assert auto(1, 1, 16, 64, 4) == "chained"
     assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "staged"       # fp32 MFMA stage kernels
     assert auto(1, 2, 7600, 48, 128, dt=L.MA_F32) == "staged"
     assert auto(1, 16, 16384, 128, 128, dt=L.MA_F32) == "generic"   # 128 x 128 fp32 tiles do not fit the LDS
