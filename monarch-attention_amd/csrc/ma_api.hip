@@ -228,7 +228,7 @@ bool fused_full_width(const ma_fwd_params* p) {
 // rows, T = 1, 2, 3, head dims 32, 64, 128: the choice below is within 0.6 % of the fastest variant
 // in the geometric mean over the 827 points, 17 % at worst):
 //  * the resident kernel for many heads of small problems: with two or three state tiles (heads
-//    of up to ~256 tokens) for blocks and block counts of at most 32, from 128 heads on for
+//    of up to ~256 tokens, whatever the head dim) for blocks and block counts of at most 32, from 128 heads on for
 //    16-row blocks and 192 for 32-row blocks; in its one-tile form (up to ~512 tokens) for
 //    problems of one or two strips when the head count fills the device's 256 one-per-CU
 //    workgroups to three quarters or more in its last pass (192 heads: 0.95 of the chained
@@ -243,7 +243,7 @@ bool fused_full_width(const ma_fwd_params* p) {
 //    on a head count that does not divide by the 8 XCDs the chained kernel pins heads to; head
 //    dims above 80 with more than 64 blocks of 64 rows and more; fewer than 8 heads of thousands
 //    of tokens (a head's tasks all run on one XCD); a single step on an uneven head count from
-//    4096 tokens on (two launches against an unbalanced one);
+//    4096 tokens on, or on 8 heads from 8192 on (two launches against an unbalanced one);
 //  * else the chained kernel (one launch, tasks in dispatch order): 10 - 25 % ahead of the stage
 //    launches over most of the sweep.
 int select_variant(const ma_fwd_params* p) {
@@ -261,7 +261,8 @@ int select_variant(const ma_fwd_params* p) {
             if (!fast) return MA_VARIANT_GENERIC;
             {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-                if (p->B <= 32 && M <= 32 && heads >= (p->B <= 16 ? 128 : 192) && resident_fits(p, false)) return MA_VARIANT_RESIDENT;
+                if (p->B <= 32 && M <= 32 && M * p->B <= 288 && heads >= (p->B <= 16 ? 128 : 192) && resident_fits(p, false))
+                    return MA_VARIANT_RESIDENT;
                 if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) &&
                     ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && resident_fits(p, true))
                     return MA_VARIANT_RESIDENT;
@@ -270,8 +271,8 @@ int select_variant(const ma_fwd_params* p) {
                 const bool class_96 = (M > 64 && M <= 96) || (p->B > 64 && p->B <= 96 && M <= 96);
                 const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
                 const bool wide_dim = p->D > 80 && M > 64 && p->B >= 64;
-                const bool few_heads = heads < 8 && p->N > (heads <= 4 ? 2048 : 4096);
-                const bool one_step = p->T == 1 && heads % 8 != 0 && p->N >= 4096;
+                const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
+                const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 8192));
                 if (!few_blocks && !class_96 && !uneven_128 && !wide_dim && !few_heads && !one_step && chain_fits(p))
                     return MA_VARIANT_CHAINED;
             }
