@@ -228,18 +228,17 @@ bool fused_full_width(const ma_fwd_params* p) {
 // rows, T = 1, 2, 3, head dims 32, 64, 128: the choice below is within 0.6 % of the fastest variant
 // in the geometric mean over the 827 points, 17 % at worst):
 //  * the resident kernel for many heads of small problems: with two or three state tiles (heads
-//    of up to ~256 tokens, whatever the head dim) for blocks and block counts of at most 32, from 128 heads on for
-//    16-row blocks and 192 for 32-row blocks; in its one-tile form (up to ~512 tokens) for
+//    of up to ~256 tokens, whatever the head dim) for blocks of at most 16 rows from 128 heads
+//    on; in its one-tile form (up to ~512 tokens) for
 //    problems of one or two strips when the head count fills the device's 256 one-per-CU
 //    workgroups to three quarters or more in its last pass (192 heads: 0.95 of the chained
 //    kernel's time with 0.6 of its traffic, 768: 0.84; 128 or 384 heads: 1.05 - 1.3);
 //  * the fused kernel (one team of workgroups per head, counter barriers) for 8 or 16 heads of
 //    ~4096 tokens in 64-row problems (the metric workload: 17.7 us against 20.0 chained and
 //    22.4 as two launches);
-//  * one launch per half step where the one-launch kernels are at a disadvantage: heads of at most
-//    8 blocks when there are many of them (the per-stage L and Z kernels pack several positions
-//    into a tile: 192 heads of four 128-row blocks 53 us against 73 us chained); 65 .. 96 blocks
-//    or block rows (the one-launch kernels run them in the 128 class); 128-row problems both ways
+//  * one launch per half step where the one-launch kernels are at a disadvantage: 65 .. 96 blocks,
+//    or blocks of 65 .. 96 rows in more than 8 of them (the one-launch kernels run these in the
+//    128 class); 128-row problems both ways
 //    on a head count that does not divide by the 8 XCDs the chained kernel pins heads to; head
 //    dims above 80 with more than 64 blocks of 64 rows and more; fewer than 8 heads of thousands
 //    of tokens (a head's tasks all run on one XCD); a single step on an uneven head count from
@@ -261,19 +260,18 @@ int select_variant(const ma_fwd_params* p) {
             if (!fast) return MA_VARIANT_GENERIC;
             {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-                if (p->B <= 32 && M <= 32 && M * p->B <= 288 && heads >= (p->B <= 16 ? 128 : 192) && resident_fits(p, false))
+                if (p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= 128 && resident_fits(p, false))
                     return MA_VARIANT_RESIDENT;
                 if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) &&
-                    ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && resident_fits(p, true))
+                    ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))
                     return MA_VARIANT_RESIDENT;
                 if (fused_full_width(p)) return MA_VARIANT_FUSED;
-                const bool few_blocks = M <= 8 && heads >= (p->D <= 64 ? 32 : 16) * M;
-                const bool class_96 = (M > 64 && M <= 96) || (p->B > 64 && p->B <= 96 && M <= 96);
+                const bool class_96 = (M > 64 && M <= 96) || (p->B > 64 && p->B <= 96 && M > 8 && M <= 96);
                 const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
                 const bool wide_dim = p->D > 80 && M > 64 && p->B >= 64;
                 const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
                 const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 8192));
-                if (!few_blocks && !class_96 && !uneven_128 && !wide_dim && !few_heads && !one_step && chain_fits(p))
+                if (!class_96 && !uneven_128 && !wide_dim && !few_heads && !one_step && chain_fits(p))
                     return MA_VARIANT_CHAINED;
             }
             return MA_VARIANT_STAGED;
@@ -325,10 +323,10 @@ int run_z(const Prepared& pr, const ma_fwd_params* p, hipStream_t s) {
     return p->dtype_qk == MA_F16 ? launch_mfma_z_f16(pr.P, s) : launch_mfma_z_bf16(pr.P, s);
 }
 
-// Heads of at most 8 blocks: the 16-bit per-stage L and Z kernels put 16 >> pack_shift in-block positions
-// into one 16-row tile (2^pack_shift >= M rows each) instead of leaving most of the tile empty.
+// Heads of at most 8 blocks: the 16-bit per-stage and chained L and Z problems put 16 >> pack_shift in-block
+// positions into one 16-row tile (2^pack_shift >= M rows each) instead of leaving most of the tile empty.
 int pack_shift_of(int variant, const ma_fwd_params* p, int M) {
-    if (variant != MA_VARIANT_STAGED || p->dtype_qk == MA_F32 || M > 8) return 4;
+    if ((variant != MA_VARIANT_STAGED && variant != MA_VARIANT_CHAINED) || p->dtype_qk == MA_F32 || M > 8) return 4;
     int sh = 0;
     while ((1 << sh) < M) ++sh;
     return sh;

@@ -151,7 +151,7 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
     if (p == nph - 1) {
         constexpr int WPP = Split<NTM, W>::WPP, PPW = Split<NTM, W>::PPW;
         const int sub = wave / WPP, wig = wave % WPP;
-        const int j = task * PPW + sub;
+        const int j = (task * PPW + sub) * (NTM == 1 ? 16 >> P.pack_shift : 1);   // heads of few blocks: several positions per tile (TileIndex)
         const bool active = sub < PPW && j < P.B;
         char* sm = smem + sub * Lds<T, DT, NTM>::Z;
         typename ZP::Pre pre;
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
     } else if (odd) {
         constexpr int WPP = Split<NTM, W>::WPP, PPW = Split<NTM, W>::PPW;
         const int sub = wave / WPP, wig = wave % WPP;
-        const int j = task * PPW + sub;
+        const int j = (task * PPW + sub) * (NTM == 1 ? 16 >> P.pack_shift : 1);
         const bool active = sub < PPW && j < P.B;
         char* sm = smem + sub * Lds<T, DT, NTM>::L;
         typename LP::Pre pre;

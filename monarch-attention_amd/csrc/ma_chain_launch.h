@@ -22,7 +22,8 @@ int launch_chain_one(const Problem& P, bool sync_ready, hipStream_t s) {
     ChainPlan pl;
     pl.hx = static_cast<int>((heads + 7) / 8);
     pl.tR = (P.M + Split<NTB, W>::PPW - 1) / Split<NTB, W>::PPW;
-    pl.tL = (P.B + Split<NTM, W>::PPW - 1) / Split<NTM, W>::PPW;
+    const int per = NTM == 1 ? 16 >> P.pack_shift : 1;   // in-block positions per L / Z problem (heads of few blocks share tiles)
+    pl.tL = ((P.B + per - 1) / per + Split<NTM, W>::PPW - 1) / Split<NTM, W>::PPW;
     pl.stride = chain_stride(P.T);
     pl.go_off = chain_go_offset(P.T);
     pl.spin_limit = P.test_no_spin ? 0u : 1u << 18;   // a legitimate wait lasts one phase of one head (well under a millisecond)

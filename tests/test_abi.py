@@ -159,8 +159,7 @@ def test_check_maps_status_to_python_exceptions():
 def test_auto_variant_policy():
     """AUTO: generic when the MFMA kernels do not apply; resident for many heads of small problems
     whose state fits in LDS; the fused kernel for 8 or 16 heads of ~4096 tokens in 64-row problems;
-    per-stage launches where the one-launch kernels are at a disadvantage (few-block heads in large
-    numbers, the 96-row tile class, uneven head counts of 128-row problems, wide heads with many blocks,
+    per-stage launches where the one-launch kernels are at a disadvantage (the 96-row tile class, uneven head counts of 128-row problems, wide heads with many blocks,
     very few long heads); the chained kernel otherwise."""
     lib = L.load()
 
@@ -181,14 +180,16 @@ def test_auto_variant_policy():
     assert auto(1, 12, 4096, 64, 64, T=1) == "staged"   # ... and with a single step two launches beat an unbalanced one
     assert auto(1, 16, 16384, 64, 128) == "chained"     # 128-row problems both ways, heads even over the XCDs
     assert auto(1, 12, 16384, 64, 128) == "staged"      # 12 heads on 8 XCDs: uneven
-    assert auto(16, 12, 512, 64, 128) == "staged"       # 192 heads of four 128-row blocks: packed L / Z tiles
-    assert auto(1, 8, 512, 64, 128) == "chained"        # ... few such heads: one launch
+    assert auto(16, 12, 512, 64, 128) == "chained"      # 192 heads of four 128-row blocks: several positions per L / Z tile
+    assert auto(16, 12, 384, 64, 96) == "chained"       # ... also for 96-row blocks, which otherwise stay per stage:
+    assert auto(1, 16, 8192, 64, 90) == "staged"        # 92 blocks of 90 rows run in the stage kernels' 96-row class
     assert auto(64, 12, 197, 64, 16) == "resident"
     assert auto(16, 12, 512, 64, 32) == "resident"     # 512-token heads: aL / aR in one LDS tile, Y through the workspace
     assert auto(8, 12, 512, 64, 32) == "chained"       # ... when the head count fills the device's workgroups
     assert auto(32, 12, 512, 64, 32) == "chained"      # (384 heads: 1.5 passes over 256 CUs)
     assert auto(16, 12, 512, 64, 64) == "chained"      # ... and for problems of one or two strips
-    assert auto(32, 12, 256, 64, 64) == "staged"       # 64-row blocks never run resident: 384 heads of four blocks
+    assert auto(32, 12, 256, 64, 64) == "chained"      # 64-row blocks never run resident
+    assert auto(16, 12, 256, 64, 32) == "chained"      # nor do 32-row blocks in 8 blocks (the chained kernel packs them)
     assert auto(8, 16, 1024, 72, 32) == "chained"
     assert auto(4, 16, 16384, 64, 128) == "chained"
     assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for
