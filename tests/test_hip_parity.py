@@ -168,11 +168,11 @@ FEW_BLOCKS = [  # E, H, N, D, B, T, pre, dt, masked: 1, 2, 3, 4, 5, 7 and 8 bloc
 ]
 
 
-@pytest.mark.parametrize("variant", ["staged", "auto"])
+@pytest.mark.parametrize("variant", ["staged", "chained", "auto"])
 @pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", FEW_BLOCKS)
 def test_heads_of_few_blocks(E, H, N, D, B, T, pre, dt, masked, variant):
-    """At most 8 blocks per head: the per-stage L and Z kernels lay 16, 8, 4 or 2 in-block positions side by
-    side in one 16-row tile and keep them apart with a block-diagonal mask."""
+    """At most 8 blocks per head: the per-stage and chained L and Z problems lay 16, 8, 4 or 2 in-block
+    positions side by side in one 16-row tile and keep them apart with a block-diagonal mask."""
     q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
     mask = block_safe_mask(E, N, B, seed=B) if masked else None
     ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
