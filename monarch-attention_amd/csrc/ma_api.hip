@@ -216,7 +216,7 @@ bool chain_fits(const ma_fwd_params* p) {
 // launch would, without the launch boundaries.
 bool fused_full_width(const ma_fwd_params* p) {
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-    if (p->B > 64 || M > 64) return false;
+    if (p->B > 64 || M > 64 || p->D > 64) return false;   // (head dims of 128: 4 - 50 % behind the chained kernel)
     const long long tR = phase_tasks(M, p->B), tL = phase_tasks(p->B, M);
     const long long widest = tR > tL ? tR : tL;
     const long long heads = static_cast<long long>(p->E) * p->H;
