@@ -225,26 +225,28 @@ bool fused_full_width(const ma_fwd_params* p) {
 
 // The variant a problem resolves to.  AUTO: the MFMA kernels when the problem qualifies; among
 // them what a sweep on MI355X says (fp16, E*H = 1 .. 384 heads, N = 256 .. 8192, blocks of 16 .. 128
-// rows, T = 1, 2, 3, head dims 32, 64, 128: the choice below is within 0.6 % of the fastest variant
-// in the geometric mean over the 827 points, 17 % at worst):
+// rows, T = 1, 2, 3, head dims 32, 64, 128; every variant that takes a shape timed: the choice
+// below is within 0.1 - 0.5 % of the fastest variant in the geometric mean of each sweep and 15 %
+// at worst):
 //  * the resident kernel for many heads of small problems: with two or three state tiles (heads
-//    of up to ~256 tokens, whatever the head dim) for blocks of at most 16 rows from 128 heads
-//    on; in its one-tile form (up to ~512 tokens) for
-//    problems of one or two strips when the head count fills the device's 256 one-per-CU
-//    workgroups to three quarters or more in its last pass (192 heads: 0.95 of the chained
-//    kernel's time with 0.6 of its traffic, 768: 0.84; 128 or 384 heads: 1.05 - 1.3);
+//    of up to ~256 tokens) for blocks of at most 16 rows from 128 heads on; in its one-tile form
+//    (up to ~512 tokens) for problems of one or two strips when the head count fills the
+//    device's 256 one-per-CU workgroups to three quarters or more in its last pass (192 heads:
+//    0.95 of the chained kernel's time with 0.6 of its traffic, 768: 0.84; 128 or 384 heads:
+//    1.05 - 1.3);
 //  * the fused kernel (one team of workgroups per head, counter barriers) for 8 or 16 heads of
-//    ~4096 tokens in 64-row problems (the metric workload: 17.7 us against 20.0 chained and
-//    22.4 as two launches);
-//  * one launch per half step where the one-launch kernels are at a disadvantage: 65 .. 96 blocks,
-//    or blocks of 65 .. 96 rows in more than 8 of them (the one-launch kernels run these in the
-//    128 class); 128-row problems both ways
-//    on a head count that does not divide by the 8 XCDs the chained kernel pins heads to; head
-//    dims above 80 with more than 64 blocks of 64 rows and more; fewer than 8 heads of thousands
-//    of tokens (a head's tasks all run on one XCD); a single step on an uneven head count from
-//    4096 tokens on, or on 8 heads from 8192 on (two launches against an unbalanced one);
+//    ~4096 tokens in 64-row problems with head dims up to 64 (the metric workload: 17.7 us
+//    against 20.0 chained and 22.4 as two launches);
+//  * one launch per half step where the one-launch kernels are at a disadvantage: 65 .. 96
+//    blocks, or blocks of 65 .. 96 rows in more than 8 of them (the one-launch kernels run these
+//    in the 128 class); 128-row problems both ways on a head count that does not divide by the
+//    8 XCDs the chained kernel pins heads to; head dims above 80 with more than 64 blocks of 64
+//    rows and more; fewer than 8 heads of thousands of tokens (a head's tasks all run on one
+//    XCD); a single step on an uneven head count from 4096 tokens on, or on 8 heads from 8192
+//    on (two launches against an unbalanced one);
 //  * else the chained kernel (one launch, tasks in dispatch order): 10 - 25 % ahead of the stage
-//    launches over most of the sweep.
+//    launches over most of the sweep, heads of 2 .. 8 blocks included (their L / Z problems share
+//    tiles, see pack_shift_of).
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
     const bool fast32 = mfma32_supported(p);   // fp32 operands: per-stage launches only
@@ -262,7 +264,7 @@ int select_variant(const ma_fwd_params* p) {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
                 if (p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= 128 && resident_fits(p, false))
                     return MA_VARIANT_RESIDENT;
-                if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) &&
+                if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D <= 64 &&
                     ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))
                     return MA_VARIANT_RESIDENT;
                 if (fused_full_width(p)) return MA_VARIANT_FUSED;
