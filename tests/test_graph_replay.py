@@ -17,8 +17,11 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 CASES = [  # E, H, N, D, B, T, dtype, variant
-    (1, 16, 1024, 64, 32, 1, "f16", "auto"),      # few heads of small blocks: the team kernel
+    (1, 16, 1024, 64, 32, 1, "f16", "auto"),      # few heads of small blocks: the chained kernel
     (1, 16, 1024, 64, 32, 2, "f16", "fused"),
+    (1, 8, 4096, 64, 64, 1, "f16", "auto"),       # teams that fill the device: the team kernel
+    (2, 4, 512, 64, 32, 2, "f16", "resident"),    # one state tile in LDS, Y through the workspace
+    (2, 6, 384, 64, 128, 2, "bf16", "chained"),   # heads of three blocks: several positions per tile
     (4, 12, 512, 64, 32, 2, "bf16", "chained"),
     (8, 16, 197, 64, 16, 2, "f16", "resident"),
     (1, 4, 2048, 64, 128, 2, "f16", "staged"),
