@@ -154,7 +154,7 @@ def main():
     ap.add_argument("--no-sdpa", action="store_true", help="skip the dense SDPA comparison")
     ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep over the variants")
     ap.add_argument("--sweep-n", action="store_true",
-                    help="the reference's sequence-length sweep (perfbench/bench.py:87-127): fp16 E=1 H=12 D=64, N = 2^10..2^14, "
+                    help="the reference's sequence-length sweep (perfbench/bench.py:87-127): fp16 E=1 H=12 D=64, N = 2^10..2^14 (and on to 2^16), "
                          "block floor(sqrt(N)), T=1, against dense SDPA")
     ap.add_argument("--sweep-e", action="store_true",
                     help="the reference's batch sweep (perfbench/bench.py:42-85): fp16 N=256 H=12 D=64 block 16, E = 2^3..2^13, T=1")
@@ -227,8 +227,9 @@ def main():
     if args.sweep_n or args.sweep_e:
         rows = []
         if args.sweep_n:
-            shapes = [(1, 12, 2 ** k, 64, int((2 ** k) ** 0.5)) for k in range(10, 15)]
-            name = "sweep_n: fp16 E1 H12 D64, block floor(sqrt(N)), T=1 (perfbench/bench.py:87-127)"
+            # the reference's sweep ends at 2^14; 2^15 and 2^16 (blocks of 181 and 256 rows) are added here
+            shapes = [(1, 12, 2 ** k, 64, int((2 ** k) ** 0.5)) for k in range(10, 17)]
+            name = "sweep_n: fp16 E1 H12 D64, block floor(sqrt(N)), T=1 (perfbench/bench.py:87-127, extended to N = 2^16)"
         else:
             shapes = [(2 ** k, 12, 256, 64, 16) for k in range(3, 14)]
             name = "sweep_e: fp16 N256 H12 D64 block 16, T=1 (perfbench/bench.py:42-85)"

@@ -58,7 +58,10 @@ typedef enum ma_mask_dtype {
 typedef enum ma_variant {
     MA_VARIANT_AUTO = 0,    /* fastest variant that supports the problem            */
     MA_VARIANT_GENERIC = 1, /* FMA kernels, 2T(+T-1) launches: any dtype/shape/stride */
-    MA_VARIANT_STAGED = 2,  /* MFMA kernels, one launch per half step (2T launches)  */
+    MA_VARIANT_STAGED = 2,  /* MFMA kernels, one launch per half step (2T launches); */
+                            /* 16-bit: blocks and block counts of up to 256 rows     */
+                            /* (heads of up to 65536 tokens), the one-launch         */
+                            /* variants below stop at 128                            */
     MA_VARIANT_FUSED = 3,   /* MFMA, all T steps in ONE launch, teams of workgroups  */
                             /* per head, state exchanged through the workspace.  Its */
                             /* workgroups wait for each other, so the grid is sized  */

@@ -124,13 +124,14 @@ Problem make_problem(const ma_fwd_params* p, const ma_ws_layout& L) {
 
 // What the MFMA kernels need: 16-bit operands of one dtype, Dv == D, 16-byte
 // row chunks (D % 8 == 0 and every row start 16-byte aligned), and block
-// problems that fit the register / LDS tiles (B, M <= 128, D <= 128).
+// problems that fit the register / LDS tiles (B, M <= 256, D <= 128: heads of up
+// to 65536 tokens; the one-launch kernels stop at 128, see one_launch_tiles).
 // Pointers may be NULL in a layout query; they are then not checked.
 bool mfma_supported(const ma_fwd_params* p) {
     if (p->dtype_qk == MA_F32 || p->dtype_v != p->dtype_qk) return false;
     if (p->Dv != p->D || p->D % 8 != 0 || p->D > 128) return false;
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-    if (p->B > 128 || M > 128) return false;
+    if (p->B > 256 || M > 256) return false;
     for (int i = 0; i < 3; ++i)
         if (p->q_stride[i] % 8 || p->k_stride[i] % 8 || p->v_stride[i] % 8 || p->out_stride[i] % 8) return false;
     if (reinterpret_cast<uintptr_t>(p->q) % 16 || reinterpret_cast<uintptr_t>(p->k) % 16 ||
@@ -187,6 +188,12 @@ bool resident_fits(const ma_fwd_params* p, bool one_tile) {
     return run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
 }
 
+// The fused, chained and resident kernels are built for block problems of at most 128 rows.
+bool one_launch_tiles(const ma_fwd_params* p) {
+    const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+    return p->B <= 128 && M <= 128;
+}
+
 // Tasks (workgroups) of one phase of one head in the one-launch kernels: four waves per workgroup; a
 // block problem of n rows takes min(ceil(n / 16), 4) waves, rounded up to a power of two.
 long long phase_tasks(long long count, long long rows) {
@@ -205,7 +212,7 @@ bool chain_fits(const ma_fwd_params* p) {
     const long long heads = static_cast<long long>(p->E) * p->H;
     const long long nph1 = 2ll * p->T - 1;
     const long long stride = (2 * nph1 + 2 + 31) / 32 * 32 + (nph1 + 31) / 32 * 32;
-    if (tR > 128 || tL > 128) return false;
+    if (!one_launch_tiles(p) || tR > 128 || tL > 128) return false;
     if (heads * stride > static_cast<long long>(kChainSyncBytes / 4)) return false;
     return 8 * ((heads + 7) / 8) * p->T * (tR + tL) <= 0x7fffffffLL;
 }
@@ -243,7 +250,8 @@ bool fused_full_width(const ma_fwd_params* p) {
 //    8 XCDs the chained kernel pins heads to; head dims above 80 with more than 64 blocks of 64
 //    rows and more; fewer than 8 heads of thousands of tokens (a head's tasks all run on one
 //    XCD); a single step on an uneven head count from 4096 tokens on, or on 8 heads from 8192
-//    on (two launches against an unbalanced one);
+//    on (two launches against an unbalanced one); blocks or block counts of 129 .. 256 rows
+//    (heads of up to 65536 tokens), which only the stage kernels have tile classes for;
 //  * else the chained kernel (one launch, tasks in dispatch order): 10 - 25 % ahead of the stage
 //    launches over most of the sweep, heads of 2 .. 8 blocks included (their L / Z problems share
 //    tiles, see pack_shift_of).
@@ -254,7 +262,7 @@ int select_variant(const ma_fwd_params* p) {
     switch (p->variant) {
         case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
         case MA_VARIANT_STAGED: return fast || fast32 ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
-        case MA_VARIANT_FUSED: return fast ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_FUSED: return fast && one_launch_tiles(p) ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_CHAINED: return fast && chain_fits(p) ? MA_VARIANT_CHAINED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_RESIDENT: return fast && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
         default:

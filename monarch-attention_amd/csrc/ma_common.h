@@ -134,7 +134,7 @@ int launch_bwd_r(const Problem& P, const BwdBuffers& G, int dt_qk, int dt_v, boo
 int launch_bwd_out(int n, const float* const* src, void* const* dst, const long long (*st)[3], int dt, const Problem& P, int W,
                    hipStream_t s);
 
-// MFMA stage kernels (fp16 / bf16, Dv == D <= 128, D % 8 == 0, B, M <= 128,
+// MFMA stage kernels (fp16 / bf16, Dv == D <= 128, D % 8 == 0, B, M <= 256,
 // 16-byte aligned rows).
 int launch_mfma_r_f16(const Problem& P, bool first, bool with_v, hipStream_t s);
 int launch_mfma_l_f16(const Problem& P, hipStream_t s);

@@ -312,13 +312,15 @@ __device__ __forceinline__ void store_row(rsrc_t dst, unsigned ro, int D, const 
 }
 
 // How a workgroup's W waves are shared among block problems with NT strips:
-// WPP waves per problem (at most four), PPW problems per workgroup.  Problems of 3 or 6 strips
+// WPP waves per problem (at most four: a wave of a 128-row problem walks two strips, one after
+// the other, a wave of a 192- / 256-row problem three / four), PPW problems per workgroup.  Problems of 3 or 6 strips
 // (blocks and block counts of 33-48 / 81-96, e.g. the 48- and 96-token blocks of the reference's
 // RoBERTa sweep, experiments/roberta/benchmark.py:78) run on three waves: a per-stage launch uses
 // workgroups of three waves (WG), a one-launch kernel leaves its fourth wave idle in such a phase.
 template <int NT, int W = kWaves>
 struct Split {
-    static_assert(NT == 1 || NT == 2 || NT == 3 || NT == 4 || NT == 6 || NT == 8, "strip counts are 1, 2, 3, 4, 6 or 8");
+    static_assert(NT == 1 || NT == 2 || NT == 3 || NT == 4 || NT == 6 || NT == 8 || NT == 12 || NT == 16,
+                  "strip counts are 1, 2, 3, 4, 6, 8, 12 or 16");
     static constexpr int WPP = (NT == 3 || NT == 6) ? 3 : (NT < kWaves ? NT : kWaves);
     static constexpr int PPW = W / WPP;
     static constexpr int WG = (NT == 3 || NT == 6) ? 3 : kWaves;   // waves of a per-stage launch's workgroup

@@ -18,9 +18,11 @@ inline int nt_class_one_launch(int n) {
     const int t = (n + 15) / 16;
     return t <= 4 ? (t < 1 ? 1 : t) : 8;
 }
+// (129 .. 256 rows: classes of 12 and 16 strips, per-stage launches only; a head of 32768 tokens in
+// blocks of floor(sqrt(N)) = 181 rows runs in the 12-strip class both ways)
 inline int nt_class(int n) {
     const int t = (n + 15) / 16;
-    return t <= 4 ? (t < 1 ? 1 : t) : t <= 6 ? 6 : 8;
+    return t <= 4 ? (t < 1 ? 1 : t) : t <= 6 ? 6 : t <= 8 ? 8 : t <= 12 ? 12 : 16;
 }
 
 // Raises a kernel's dynamic-LDS limit to `bytes`, once per (kernel, device): the attribute belongs
@@ -77,7 +79,9 @@ int for_classes(int dt, int nt, F&& f) {
         case 3: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 3>{}); \
         case 4: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 4>{}); \
         case 6: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 6>{}); \
-        default: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 8>{}); \
+        case 8: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 8>{}); \
+        case 12: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 12>{}); \
+        default: return f(std::integral_constant<int, DTV>{}, std::integral_constant<int, 16>{}); \
     }
     switch (dt) {
         case 2: MA_NT(2)

@@ -205,7 +205,20 @@ def test_auto_variant_policy():
     assert auto(1, 16, 4096, 62, 64, dt=L.MA_F32) == "generic"      # D % 4 != 0
     assert auto(1, 16, 4096, 64, 64, Dv=128) == "generic"
     assert auto(1, 16, 4096, 60, 64) == "generic"       # D % 8 != 0
-    assert auto(1, 16, 4096, 64, 256) == "generic"      # B > 128
+    assert auto(1, 16, 4096, 64, 256) == "staged"       # blocks of 129 .. 256 rows: per-stage launches only
+    assert auto(1, 16, 32768, 64, 128) == "staged"      # 129 .. 256 blocks likewise (heads of up to 65536 tokens)
+    assert auto(1, 16, 65536, 64, 256) == "staged"
+    assert auto(1, 16, 4096, 64, 257) == "generic"      # B > 256
+    for name in ("fused", "chained", "resident"):       # the one-launch kernels stop at 128 rows
+        p = L.FwdParams()
+        p.E, p.H, p.N, p.D, p.Dv, p.B, p.T = 1, 16, 4096, 64, 64, 256, 2
+        p.dtype_qk = p.dtype_v = L.MA_F16
+        for field in ("q_stride", "k_stride", "v_stride", "out_stride"):
+            setattr(p, field, (C.c_int64 * 3)(4096 * 64, 4096 * 64, 64))
+        p.eps = 1e-12
+        p.variant = L.VARIANTS[name]
+        assert lib.ma_fwd_select_variant(p) == L.MA_ERR_UNSUPPORTED
+    assert auto(1, 16, 65537, 64, 256) == "generic"     # more than 256 blocks
 
 
 def good_bwd_params(**kw):

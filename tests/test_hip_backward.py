@@ -69,6 +69,9 @@ CASES = [  # E, H, N, D, Dv, B, T, pre, dt, masked
     # 128-row blocks in enough blocks (512) that they are not split over workgroups
     (1, 2, 224, 72, 72, 32, 3, True, "f16", True), (1, 2, 512, 128, 128, 64, 2, False, "bf16", False),
     (2, 2, 512, 64, 64, 64, 2, False, "f16", True), (1, 8, 8192, 32, 32, 128, 2, False, "bf16", False),
+    # 129 .. 256 blocks / rows per block: the forward steps run in the stage kernels' 16-strip class, the
+    # derivative stages in the LDS kernels (row tiles)
+    (1, 2, 1600, 64, 64, 10, 2, False, "f16", True), (1, 1, 1500, 32, 32, 150, 2, True, "bf16", False),
 ]
 
 

@@ -180,6 +180,31 @@ def test_heads_of_few_blocks(E, H, N, D, B, T, pre, dt, masked, variant):
     assert_parity(out.cpu(), ref, dt, f"few blocks {(E, H, N, D, B, T, pre, dt, masked)}/{variant}")
 
 
+LARGE_TILES = [  # E, H, N, D, B, T, pre, dt, masked: blocks and / or block counts of 129 .. 256 rows
+    (1, 2, 4096, 64, 256, 2, False, "f16", False), (2, 1, 3000, 64, 20, 2, True, "bf16", True),       # one side only
+    (1, 2, 2100, 72, 130, 3, False, "f16", True), (1, 3, 2571, 32, 150, 1, True, "f16", False),
+    (1, 1, 32768, 64, 181, 2, False, "f16", False), (1, 1, 40000, 128, 200, 2, True, "bf16", True),   # both sides
+    (1, 1, 65536, 64, 256, 1, False, "bf16", False), (1, 2, 20000, 40, 129, 3, False, "f16", True),
+]
+
+
+@pytest.mark.parametrize("variant", ["staged", "auto"])
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", LARGE_TILES)
+def test_blocks_and_block_counts_up_to_256(E, H, N, D, B, T, pre, dt, masked, variant):
+    """Heads of up to 65536 tokens: block problems of 129 .. 256 rows run in the stage kernels' 16-strip
+    class; AUTO must pick those kernels (not the FMA path), the one-launch variants must refuse."""
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
+    mask = block_safe_mask(E, N, B, seed=B) if masked else None
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
+    dev = to_dev(q, k, v, mask)
+    out = run_hip(*dev, T, B, pre, variant)
+    assert_parity(out.cpu(), ref, dt, f"large tiles {(E, H, N, D, B, T, pre, dt, masked)}/{variant}")
+    if variant == "auto":
+        for other in ("fused", "chained", "resident"):
+            with pytest.raises(NotImplementedError):
+                monarch_attention_hip(*dev, T, B, pre, variant=other)
+
+
 ONE_TILE = [  # E, H, N, D, B, T, pre, dt, masked: heads whose aL / aR / Y do not fit in LDS as three (or two) tiles
     (2, 3, 512, 64, 32, 2, False, "bf16", False), (1, 4, 500, 64, 32, 3, True, "f16", True),
     (1, 2, 384, 64, 24, 1, False, "f16", True), (2, 2, 448, 64, 16, 2, True, "bf16", False),
@@ -269,6 +294,10 @@ STAGE_CASES = [  # E,H,N,D,Dv,B,T,pre,dt,vdt,mask
     (1, 2, 100, 64, 64, 100, 2, False, "f16", "f16", False),
     (1, 3, 130, 40, 40, 20, 2, True, "f16", "f16", False),
     (1, 2, 45, 72, 72, 27, 2, False, "bf16", "bf16", False),
+    # blocks / block counts of 129 .. 256 rows: the 16-strip tile class (four strips per wave)
+    (1, 2, 3000, 64, 64, 200, 2, True, "f16", "f16", True),
+    (1, 1, 2600, 32, 32, 20, 2, False, "bf16", "bf16", False),
+    (1, 1, 33000, 64, 64, 180, 2, False, "f16", "f16", True),
 ]
 
 
