@@ -447,7 +447,9 @@ struct RProb {
 
     // NT: the inputs are loaded with the streaming policy (a caller's choice: streaming inputs leave the L2 to
     // the state, which pays where nothing re-reads them from it - few long heads in one launch; ordinary
-    // loads keep K and Q in L2 for the later steps of many-head and per-stage launches)
+    // loads keep K and Q in L2 for the later steps of many-head and per-stage launches).  Q is the
+    // exception when there are L steps to come (T > 1): they and the Z step read it again, and the
+    // caller that streams everything else measured 3 - 5 % faster at T = 2, 3 with Q kept (T = 1: no gain).
     template <bool NT = false>
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int e, int m, bool first,
                                                  bool with_v, int wig, int lane) {
@@ -461,7 +463,9 @@ struct RProb {
 #pragma unroll
             for (int i = 0; i < SPW; ++i) {
                 const int j = 16 * (wig + i * WPP) + (lane & 15);
-                load_x<T, DT, NT>(pre.xq[i], S.q, j < B ? tok_off(t0 + j, P.N, S.qst) : kOob, D, lane >> 4);
+                const unsigned ro = j < B ? tok_off(t0 + j, P.N, S.qst) : kOob;
+                if (NT && P.T == 1) load_x<T, DT, true>(pre.xq[i], S.q, ro, D, lane >> 4);
+                else load_x<T, DT, false>(pre.xq[i], S.q, ro, D, lane >> 4);
             }
         }
         pre.km = mask_load(S, P, t0 + tix, tix < B);
@@ -772,7 +776,8 @@ struct LProb {
         if (!active) return;
         const int tix = wig * 64 + lane;
         const TileIndex<NWT> ti(P, j);
-        pre.qc.template issue<NT>(S.q, P.D, [&](int l) { return ti.ok(P, l) ? tok_off(ti.token(P, l), P.N, S.qst) : kOob; }, tix);
+        // (never streamed: an L step is followed by at least the Z step, which reads Q again)
+        pre.qc.template issue<false>(S.q, P.D, [&](int l) { return ti.ok(P, l) ? tok_off(ti.token(P, l), P.N, S.qst) : kOob; }, tix);
 #pragma unroll
         for (int i = 0; i < SPW; ++i) {
             const int l = 16 * (wig + i * WPP) + (lane & 15);
