@@ -646,6 +646,37 @@ def test_random_shapes_every_variant(idx, E, H, N, D, B, T, pre, dt, masked):
     assert sync_status() == 0
 
 
+def _random_large_cases(n, seed):
+    import random
+    rng = random.Random(seed)
+    cases = []
+    for i in range(n):
+        side = rng.choice(["blocks", "rows", "both"])
+        B = rng.randint(129, 256) if side != "blocks" else rng.choice([1, 7, 16, 24, 33, 64])
+        M = rng.randint(129, 256) if side != "rows" else rng.choice([1, 2, 5, 16, 40])
+        N = max(1, M * B - rng.randrange(0, B))
+        dt = rng.choice(["f16", "bf16"])
+        D = rng.choice([8, 16, 32, 40, 64, 72, 96, 128])
+        H = 1 if side == "both" else rng.choice([1, 2, 3])
+        cases.append((i, 1, H, N, D, B, rng.choice([1, 2, 3]), rng.random() < 0.5, dt, rng.random() < 0.4))
+    return cases
+
+
+@pytest.mark.parametrize("idx,E,H,N,D,B,T,pre,dt,masked", _random_large_cases(24, seed=65536))
+def test_random_shapes_in_the_192_and_256_row_classes(idx, E, H, N, D, B, T, pre, dt, masked):
+    """Seeded random problems whose blocks and / or block counts lie in 129 .. 256 (heads of up to 65536
+    tokens): AUTO must run them on the MFMA stage kernels and meet the parity gate."""
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt], scale=0.7, seed=300 + idx)
+    mask = block_safe_mask(E, N, B, seed=idx) if masked else None
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
+    dev = to_dev(q, k, v, mask)
+    out = torch.empty_like(dev[2])
+    assert L.VARIANT_NAMES[L.load().ma_fwd_select_variant(make_params(*dev[:3], None, out, T, B, pre, "auto"))] == "staged"
+    got = monarch_attention_hip(*dev, T, B, pre, variant="auto")
+    torch.cuda.synchronize()
+    assert_parity(got.cpu(), ref, dt, f"large case {idx} {(E, H, N, D, B, T, pre, dt, masked)}")
+
+
 # ---------------------------------------------------------------- a wait between workgroups that runs out is loud
 @pytest.mark.parametrize("shape", [(1, 2, 1024, 64, 32, 2), (3, 8, 512, 64, 32, 3), (1, 16, 2048, 64, 64, 1)])
 @pytest.mark.parametrize("variant", ["fused", "chained"])
