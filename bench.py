@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cM] [--T 1]
                     [--variant auto|generic|staged|fused|resident|chained] [--no-cpu] [--no-sdpa] [--no-sweep]
     python bench.py --sweep-n | --sweep-e        # the reference's own sweep protocol, against dense SDPA
-    python bench.py --sweep-variants [--T 2] [--head-dim 64]   # every variant over a grid of shapes: AUTO's choice vs the fastest
+    python bench.py --sweep-variants [--T 2] [--head-dim 64] [--sweep-grid class96]   # every variant over a grid of shapes: AUTO's choice vs the fastest
     python bench.py --record-traffic FETCH.csv WRITE.csv [--config cM --T 1 --variant auto]
 
 A step is ONE forward call of the hot path (monarch_attention, all T steps)
@@ -163,6 +163,8 @@ def main():
                          "N = 256 .. 8192, blocks of 16 .. 128 rows (T from --T, default 2; head dim from --head-dim); prints the rows "
                          "and how far AUTO's choice is from the fastest variant")
     ap.add_argument("--head-dim", type=int, default=64, help="head dim of --sweep-variants")
+    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96"],
+                    help="shapes of --sweep-variants: power-of-two lengths and blocks, or blocks / block counts in the 96-row tile class")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="fold two rocprofv3 --pmc counter_collection.csv files into profiles/traffic.json (no GPU needed)")
     ap.add_argument("--matrix", action="store_true",
@@ -269,49 +271,54 @@ def main():
         T_, D = args.T or 2, args.head_dim
         names = ("staged", "chained", "fused", "resident")
         rows, logsum, worst = [], 0.0, None
-        for heads in (1, 2, 4, 6, 8, 12, 16, 32, 64, 128, 192, 384):
-            for N in (256, 512, 1024, 2048, 4096, 8192):
-                for B in (16, 32, 64, 128):
-                    M = -(-N // B)
-                    set_bytes = 4 * heads * N * D * 2
-                    if M > 128 or M < 2 or set_bytes > 1.2e9:
-                        continue
-                    E, H = (heads // 4, 4) if heads % 4 == 0 else (1, heads)
-                    gen = torch.Generator().manual_seed(0)
-                    nbuf = max(2, min(8, -(-400 * 2 ** 20 // set_bytes)))
-                    base = [torch.randn(E, H, N, D, generator=gen).to(torch.float16) for _ in range(3)]
-                    sets = []
-                    for i in range(nbuf):
-                        q, k, v = (t.to(dev).roll(i, dims=2).contiguous() for t in base)
-                        sets.append((q, k, v, torch.empty_like(q)))
-                    row = {"heads": heads, "N": N, "block": B}
-                    for variant in ("auto",) + names:
-                        ps = [make_params(q, k, v, None, o, T_, B, False, variant) for (q, k, v, o) in sets]
-                        sel = lib.ma_fwd_select_variant(ps[0])
-                        if variant == "auto":
-                            row["auto"] = L.VARIANT_NAMES[sel]
-                            continue
-                        if sel < 0:
-                            continue
-                        nbytes = lib.ma_fwd_workspace_bytes(ps[0])
-                        ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
-                        for p in ps:
-                            p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), nbytes, L.MA_FLAG_SYNC_READY
-                        if any(lib.ma_fwd(ps[i % nbuf], sp) for i in range(4)):
-                            continue   # e.g. a team grid that does not fit the device
-                        row[variant] = round(batch_stats(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), 100)["median_ms"] * 1e3, 2)
-                        del ws
-                    best = min(names, key=lambda v: row.get(v, float("inf")))
-                    row["best"] = best
-                    row["auto_over_best"] = round(row[row["auto"]] / row[best], 3)
-                    logsum += math.log(row["auto_over_best"])
-                    if worst is None or row["auto_over_best"] > worst["auto_over_best"]:
-                        worst = row
-                    rows.append(row)
-                    del sets
-                    torch.cuda.empty_cache()
+        if args.sweep_grid == "pow2":
+            grid = [(h, N, B) for h in (1, 2, 4, 6, 8, 12, 16, 32, 64, 128, 192, 384) for N in (256, 512, 1024, 2048, 4096, 8192)
+                    for B in (16, 32, 64, 128)]
+        else:   # blocks and / or block counts of 65 .. 96 rows (and two 128-row shapes with ragged block counts)
+            grid = [(h, N, B) for h in (4, 8, 12, 16, 24, 32, 64, 192)
+                    for (N, B) in ((8192, 96), (6000, 64), (4096, 48), (2048, 24), (1000, 80), (512, 96), (9000, 96), (5500, 80),
+                                   (7000, 128), (12000, 128), (768, 96))]
+        for (heads, N, B) in grid:
+            M = -(-N // B)
+            set_bytes = 4 * heads * N * D * 2
+            if M > 128 or M < 2 or set_bytes > (1.2e9 if args.sweep_grid == "pow2" else 0.6e9):
+                continue
+            E, H = (heads // 4, 4) if heads % 4 == 0 else (1, heads)
+            gen = torch.Generator().manual_seed(0)
+            nbuf = max(2, min(8, -(-400 * 2 ** 20 // set_bytes)))
+            base = [torch.randn(E, H, N, D, generator=gen).to(torch.float16) for _ in range(3)]
+            sets = []
+            for i in range(nbuf):
+                q, k, v = (t.to(dev).roll(i, dims=2).contiguous() for t in base)
+                sets.append((q, k, v, torch.empty_like(q)))
+            row = {"heads": heads, "N": N, "block": B}
+            for variant in ("auto",) + names:
+                ps = [make_params(q, k, v, None, o, T_, B, False, variant) for (q, k, v, o) in sets]
+                sel = lib.ma_fwd_select_variant(ps[0])
+                if variant == "auto":
+                    row["auto"] = L.VARIANT_NAMES[sel]
+                    continue
+                if sel < 0:
+                    continue
+                nbytes = lib.ma_fwd_workspace_bytes(ps[0])
+                ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+                for p in ps:
+                    p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), nbytes, L.MA_FLAG_SYNC_READY
+                if any(lib.ma_fwd(ps[i % nbuf], sp) for i in range(4)):
+                    continue   # e.g. a team grid that does not fit the device
+                row[variant] = round(batch_stats(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), 100)["median_ms"] * 1e3, 2)
+                del ws
+            best = min(names, key=lambda v: row.get(v, float("inf")))
+            row["best"] = best
+            row["auto_over_best"] = round(row[row["auto"]] / row[best], 3)
+            logsum += math.log(row["auto_over_best"])
+            if worst is None or row["auto_over_best"] > worst["auto_over_best"]:
+                worst = row
+            rows.append(row)
+            del sets
+            torch.cuda.empty_cache()
         print(json.dumps({"metric": "AUTO's choice against the fastest variant", "unit": "us (median)", "n_gpus": 1, "dtype": "f16",
-                          "data": "synthetic", "T": T_, "D": D, "points": len(rows),
+                          "data": "synthetic", "T": T_, "D": D, "grid": args.sweep_grid, "points": len(rows),
                           "geomean_auto_over_best": round(math.exp(logsum / max(len(rows), 1)), 4), "worst": worst, "rows": rows}))
         return
 

@@ -244,10 +244,9 @@ bool fused_full_width(const ma_fwd_params* p) {
 //  * the fused kernel (one team of workgroups per head, counter barriers) for 8 or 16 heads of
 //    ~4096 tokens in 64-row problems with head dims up to 64 (the metric workload: 17.7 us
 //    against 20.0 chained and 22.4 as two launches);
-//  * one launch per half step where the one-launch kernels are at a disadvantage: 65 .. 96
-//    blocks, or blocks of 65 .. 96 rows in more than 8 of them (the one-launch kernels run these
-//    in the 128 class); 128-row problems both ways on a head count that does not divide by the
-//    8 XCDs the chained kernel pins heads to; head dims above 80 with more than 64 blocks of 64
+//  * one launch per half step where the one-launch kernels are at a disadvantage: 128-row
+//    problems both ways on a head count that does not divide by the 8 XCDs the chained kernel
+//    pins heads to; head dims above 80 with more than 64 blocks of 64
 //    rows and more; fewer than 8 heads of thousands of tokens (a head's tasks all run on one
 //    XCD); a single step on an uneven head count from 4096 tokens on, or on 8 heads from 8192
 //    on (two launches against an unbalanced one); blocks or block counts of 129 .. 256 rows
@@ -276,12 +275,11 @@ int select_variant(const ma_fwd_params* p) {
                     ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))
                     return MA_VARIANT_RESIDENT;
                 if (fused_full_width(p)) return MA_VARIANT_FUSED;
-                const bool class_96 = (M > 64 && M <= 96) || (p->B > 64 && p->B <= 96 && M > 8 && M <= 96);
                 const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
                 const bool wide_dim = p->D > 80 && M > 64 && p->B >= 64;
                 const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
                 const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 8192));
-                if (!class_96 && !uneven_128 && !wide_dim && !few_heads && !one_step && chain_fits(p))
+                if (!uneven_128 && !wide_dim && !few_heads && !one_step && chain_fits(p))
                     return MA_VARIANT_CHAINED;
             }
             return MA_VARIANT_STAGED;

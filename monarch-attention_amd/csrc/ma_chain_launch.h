@@ -44,13 +44,14 @@ int launch_chain_one(const Problem& P, bool sync_ready, hipStream_t s) {
 
 template <class T, int DT>
 int launch_chain(const Problem& P, bool sync_ready, hipStream_t s) {
-    const int ntb = nt_class_one_launch(P.B), ntm = nt_class_one_launch(P.M);
+    const int ntb = nt_class_chain(P.B), ntm = nt_class_chain(P.M);
 #define MA_NTM(NB)                                                              \
     switch (ntm) {                                                              \
         case 1: return launch_chain_one<T, DT, NB, 1>(P, sync_ready, s);        \
         case 2: return launch_chain_one<T, DT, NB, 2>(P, sync_ready, s);        \
         case 3: return launch_chain_one<T, DT, NB, 3>(P, sync_ready, s);        \
         case 4: return launch_chain_one<T, DT, NB, 4>(P, sync_ready, s);        \
+        case 6: return launch_chain_one<T, DT, NB, 6>(P, sync_ready, s);        \
         default: return launch_chain_one<T, DT, NB, 8>(P, sync_ready, s);       \
     }
     switch (ntb) {
@@ -58,6 +59,7 @@ int launch_chain(const Problem& P, bool sync_ready, hipStream_t s) {
         case 2: MA_NTM(2)
         case 3: MA_NTM(3)
         case 4: MA_NTM(4)
+        case 6: MA_NTM(6)
         default: MA_NTM(8)
     }
 #undef MA_NTM

@@ -13,10 +13,15 @@ namespace ma {
 namespace mfma {
 
 inline int dt_class(int D) { return D <= 32 ? 2 : D <= 64 ? 4 : D <= 80 ? 5 : 8; }
-// the one-launch kernels are built for fewer classes: 96-row problems run as 128-row ones there
+// the team kernel is built for fewer classes: 96-row problems run as 128-row ones there
 inline int nt_class_one_launch(int n) {
     const int t = (n + 15) / 16;
     return t <= 4 ? (t < 1 ? 1 : t) : 8;
+}
+// the chained kernel has the 96-row class as well
+inline int nt_class_chain(int n) {
+    const int t = (n + 15) / 16;
+    return t <= 4 ? (t < 1 ? 1 : t) : t <= 6 ? 6 : 8;
 }
 // (129 .. 256 rows: classes of 12 and 16 strips, per-stage launches only; a head of 32768 tokens in
 // blocks of floor(sqrt(N)) = 181 rows runs in the 12-strip class both ways)

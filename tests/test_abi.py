@@ -159,7 +159,7 @@ def test_check_maps_status_to_python_exceptions():
 def test_auto_variant_policy():
     """AUTO: generic when the MFMA kernels do not apply; resident for many heads of small problems
     whose state fits in LDS; the fused kernel for 8 or 16 heads of ~4096 tokens in 64-row problems;
-    per-stage launches where the one-launch kernels are at a disadvantage (the 96-row tile class, uneven head counts of 128-row problems, wide heads with many blocks,
+    per-stage launches where the one-launch kernels are at a disadvantage (uneven head counts of 128-row problems, wide heads with many blocks,
     very few long heads); the chained kernel otherwise."""
     lib = L.load()
 
@@ -181,8 +181,8 @@ def test_auto_variant_policy():
     assert auto(1, 16, 16384, 64, 128) == "chained"     # 128-row problems both ways, heads even over the XCDs
     assert auto(1, 12, 16384, 64, 128) == "staged"      # 12 heads on 8 XCDs: uneven
     assert auto(16, 12, 512, 64, 128) == "chained"      # 192 heads of four 128-row blocks: several positions per L / Z tile
-    assert auto(16, 12, 384, 64, 96) == "chained"       # ... also for 96-row blocks, which otherwise stay per stage:
-    assert auto(1, 16, 8192, 64, 90) == "staged"        # 92 blocks of 90 rows run in the stage kernels' 96-row class
+    assert auto(16, 12, 384, 64, 96) == "chained"       # ... also for 96-row blocks
+    assert auto(1, 16, 8192, 64, 90) == "chained"       # 92 blocks of 90 rows: the chained kernel has the 96-row class too
     assert auto(64, 12, 197, 64, 16) == "resident"
     assert auto(16, 12, 512, 64, 32) == "resident"     # 512-token heads: aL / aR in one LDS tile, Y through the workspace
     assert auto(8, 12, 512, 64, 32) == "chained"       # ... when the head count fills the device's workgroups
@@ -195,7 +195,7 @@ def test_auto_variant_policy():
     assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for
     assert auto(2, 16, 8192, 64, 64) == "chained"       # 128 blocks of 64 rows (long documents), head dim 64
     assert auto(2, 16, 8192, 128, 64) == "staged"       # ... but not for wide heads
-    assert auto(2, 16, 5000, 64, 64) == "staged"        # or 65 .. 96 blocks, which the one-launch kernels would run as 128
+    assert auto(2, 16, 5000, 64, 64) == "chained"       # 79 blocks: the 96-row class
     assert auto(1, 2, 8192, 64, 64) == "staged"         # two long heads would run on two of the eight XCDs
     assert auto(2, 2, 197, 64, 16) == "chained"         # few short heads: one launch
     assert auto(1, 1, 16, 64, 4) == "chained"
