@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cM] [--T 1]
                     [--variant auto|generic|staged|fused|resident|chained] [--no-cpu] [--no-sdpa] [--no-sweep]
     python bench.py --sweep-n | --sweep-e        # the reference's own sweep protocol, against dense SDPA
-    python bench.py --sweep-variants [--T 2] [--head-dim 64] [--sweep-grid class96]   # every variant over a grid of shapes: AUTO's choice vs the fastest
+    python bench.py --sweep-variants [--T 2] [--head-dim 64] [--sweep-grid class96|fewheads]   # every variant over a grid of shapes: AUTO's choice vs the fastest
     python bench.py --record-traffic FETCH.csv WRITE.csv [--config cM --T 1 --variant auto]
 
 A step is ONE forward call of the hot path (monarch_attention, all T steps)
@@ -163,8 +163,9 @@ def main():
                          "N = 256 .. 8192, blocks of 16 .. 128 rows (T from --T, default 2; head dim from --head-dim); prints the rows "
                          "and how far AUTO's choice is from the fastest variant")
     ap.add_argument("--head-dim", type=int, default=64, help="head dim of --sweep-variants")
-    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96"],
-                    help="shapes of --sweep-variants: power-of-two lengths and blocks, or blocks / block counts in the 96-row tile class")
+    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96", "fewheads"],
+                    help="shapes of --sweep-variants: power-of-two lengths and blocks, blocks / block counts in the 96-row tile class, "
+                         "or few heads of thousands of tokens")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="fold two rocprofv3 --pmc counter_collection.csv files into profiles/traffic.json (no GPU needed)")
     ap.add_argument("--matrix", action="store_true",
@@ -274,6 +275,8 @@ def main():
         if args.sweep_grid == "pow2":
             grid = [(h, N, B) for h in (1, 2, 4, 6, 8, 12, 16, 32, 64, 128, 192, 384) for N in (256, 512, 1024, 2048, 4096, 8192)
                     for B in (16, 32, 64, 128)]
+        elif args.sweep_grid == "fewheads":   # 8, 16, 24 heads of thousands of tokens: where the team kernel competes
+            grid = [(h, N, B) for h in (8, 16, 24) for N in (2048, 4096, 5000, 6144, 8000, 8192) for B in (32, 64, 128)]
         else:   # blocks and / or block counts of 65 .. 96 rows (and two 128-row shapes with ragged block counts)
             grid = [(h, N, B) for h in (4, 8, 12, 16, 24, 32, 64, 192)
                     for (N, B) in ((8192, 96), (6000, 64), (4096, 48), (2048, 24), (1000, 80), (512, 96), (9000, 96), (5500, 80),

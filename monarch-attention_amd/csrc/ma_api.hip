@@ -217,23 +217,32 @@ bool chain_fits(const ma_fwd_params* p) {
     return 8 * ((heads + 7) / 8) * p->T * (tR + tL) <= 0x7fffffffLL;
 }
 
-// Few heads of 64-row problems: every head gets a team with one workgroup per block problem (64 of
-// them per phase: heads of ~4096 tokens), the teams sit on one XCD each and all of them are on the
-// device at once (256 CUs x 4 workgroups) - the fused kernel then runs each phase like a per-stage
-// launch would, without the launch boundaries.
+// Few heads whose phases fill the device: every head gets a team with one workgroup per task (64
+// or 128 of them per phase), the teams sit on one XCD each and all of them are on the device at
+// once (256 CUs x 4 workgroups) - the fused kernel then runs each phase like a per-stage launch
+// would, without the launch boundaries.  With a single step that pays for 16 heads of 64-row
+// problems only (~4096 tokens: the metric workload); with more steps - the later exchanges of a team stay in its XCD's L2 -
+// also for 128 blocks or 128-row blocks (8 heads of ~8192 tokens, 16 of ~4096 in 32- or 128-row
+// blocks: 3 - 17 % ahead of the chained kernel), and for 8 heads also with head dims up to 80.
+// Blocks or block counts of 65 .. 96 rows stay away: the team kernel runs them as 128-row problems.
 bool fused_full_width(const ma_fwd_params* p) {
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-    if (p->B > 64 || M > 64 || p->D > 64) return false;   // (head dims of 128: 4 - 50 % behind the chained kernel)
+    const long long heads = static_cast<long long>(p->E) * p->H;
+    const bool steps = p->T > 1;
+    const int rows = steps ? 128 : 64;
+    if (p->B > rows || M > rows) return false;
+    if ((M > 64 && M <= 96) || (p->B > 64 && p->B <= 96)) return false;
+    if (p->D > (steps && heads == 8 ? 80 : 64)) return false;   // (head dims of 128: 4 - 50 % behind the chained kernel)
     const long long tR = phase_tasks(M, p->B), tL = phase_tasks(p->B, M);
     const long long widest = tR > tL ? tR : tL;
-    const long long heads = static_cast<long long>(p->E) * p->H;
+    if (!steps && heads * widest != 1024) return false;   // a single step: only with every workgroup slot of the device taken
     return heads < 32 && heads % 8 == 0 && widest >= 64 && heads * widest <= 1024;
 }
 
 // The variant a problem resolves to.  AUTO: the MFMA kernels when the problem qualifies; among
 // them what a sweep on MI355X says (fp16, E*H = 1 .. 384 heads, N = 256 .. 8192, blocks of 16 .. 128
 // rows, T = 1, 2, 3, head dims 32, 64, 128; every variant that takes a shape timed: the choice
-// below is within 0.1 - 0.5 % of the fastest variant in the geometric mean of each sweep and 15 %
+// below is within 0.0 - 0.7 % of the fastest variant in the geometric mean of each sweep and 18 %
 // at worst):
 //  * the resident kernel for many heads of small problems: with two or three state tiles (heads
 //    of up to ~256 tokens) for blocks of at most 16 rows from 128 heads on; in its one-tile form
@@ -241,14 +250,14 @@ bool fused_full_width(const ma_fwd_params* p) {
 //    device's 256 one-per-CU workgroups to three quarters or more in its last pass (192 heads:
 //    0.95 of the chained kernel's time with 0.6 of its traffic, 768: 0.84; 128 or 384 heads:
 //    1.05 - 1.3);
-//  * the fused kernel (one team of workgroups per head, counter barriers) for 8 or 16 heads of
-//    ~4096 tokens in 64-row problems with head dims up to 64 (the metric workload: 17.7 us
-//    against 20.0 chained and 22.4 as two launches);
+//  * the fused kernel (one team of workgroups per head, counter barriers) for 8 or 16 heads whose
+//    phases fill the device (fused_full_width; the metric workload: 17.7 us against 20.0 chained
+//    and 22.4 as two launches);
 //  * one launch per half step where the one-launch kernels are at a disadvantage: 128-row
 //    problems both ways on a head count that does not divide by the 8 XCDs the chained kernel
 //    pins heads to; head dims above 80 with more than 64 blocks of 64
 //    rows and more; fewer than 8 heads of thousands of tokens (a head's tasks all run on one
-//    XCD); a single step on an uneven head count from 4096 tokens on, or on 8 heads from 8192
+//    XCD); a single step on an uneven head count from 4096 tokens on, or on 8 heads from ~7000
 //    on (two launches against an unbalanced one); blocks or block counts of 129 .. 256 rows
 //    (heads of up to 65536 tokens), which only the stage kernels have tile classes for;
 //  * else the chained kernel (one launch, tasks in dispatch order): 10 - 25 % ahead of the stage
@@ -278,7 +287,7 @@ int select_variant(const ma_fwd_params* p) {
                 const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
                 const bool wide_dim = p->D > 80 && M > 64 && p->B >= 64;
                 const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
-                const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 8192));
+                const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 7168));
                 if (!uneven_128 && !wide_dim && !few_heads && !one_step && chain_fits(p))
                     return MA_VARIANT_CHAINED;
             }

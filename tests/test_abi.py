@@ -175,6 +175,13 @@ def test_auto_variant_policy():
     assert auto(1, 16, 4096, 64, 64) == "fused"         # 16 heads x 64 workgroups: every head has a full team at once
     assert auto(1, 16, 4096, 64, 64, T=1) == "fused"
     assert auto(2, 16, 4096, 64, 64) == "chained"
+    assert auto(1, 8, 8192, 64, 64) == "fused"          # with more than one step also 128 tasks per phase: 8 heads of 8192 tokens,
+    assert auto(1, 16, 4096, 64, 128) == "fused"        # 16 heads of 4096 in 128-row blocks (two positions per workgroup)
+    assert auto(1, 8, 8192, 72, 128) == "fused"         # 8 heads also with head dims up to 80
+    assert auto(1, 16, 4096, 72, 64) == "chained"       # ... 16 heads not
+    assert auto(1, 8, 6144, 64, 64) == "chained"        # 96 blocks: the team kernel would run them as 128
+    assert auto(1, 8, 8192, 64, 64, T=1) == "staged"    # a single step: two launches
+    assert auto(1, 8, 4096, 64, 64, T=1) == "chained"   # ... and teams only when they fill every workgroup slot (16 heads)
     assert auto(1, 8, 1024, 64, 32) == "chained"        # teams of 16 workgroups: the chained kernel is ahead
     assert auto(1, 12, 4096, 64, 64) == "chained"       # 12 heads do not sit evenly on 8 XCDs: no teams
     assert auto(1, 12, 4096, 64, 64, T=1) == "staged"   # ... and with a single step two launches beat an unbalanced one
