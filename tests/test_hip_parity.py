@@ -205,6 +205,29 @@ def test_blocks_and_block_counts_up_to_256(E, H, N, D, B, T, pre, dt, masked, va
                 monarch_attention_hip(*dev, T, B, pre, variant=other)
 
 
+TEAM_SHAPES = [  # E, H, N, D, B, T, pre, dt, masked: 8 or 16 heads whose phases fill the device, more than one step
+    (1, 8, 8000, 64, 64, 2, True, "f16", True), (1, 8, 8192, 72, 128, 3, False, "f16", False),
+    (1, 16, 4096, 64, 32, 2, False, "bf16", True), (2, 4, 5000, 32, 128, 3, True, "f16", True),
+    (1, 16, 4000, 64, 128, 2, True, "bf16", False), (1, 8, 4096, 80, 64, 2, False, "f16", True),
+]
+
+
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", TEAM_SHAPES)
+def test_few_long_heads_run_in_the_team_kernel(E, H, N, D, B, T, pre, dt, masked):
+    """AUTO sends 8 or 16 heads of 64 .. 128 tasks per phase to the team kernel when T > 1 (teams larger than
+    the workgroups the device holds per head loop over their tasks): parity, and the bounded waits all met."""
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
+    mask = block_safe_mask(E, N, B, seed=B) if masked else None
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
+    dev = to_dev(q, k, v, mask)
+    out = torch.empty_like(dev[2])
+    assert L.VARIANT_NAMES[L.load().ma_fwd_select_variant(make_params(*dev[:3], None, out, T, B, pre, "auto"))] == "fused"
+    got = monarch_attention_hip(*dev, T, B, pre, variant="auto")
+    torch.cuda.synchronize()
+    assert_parity(got.cpu(), ref, dt, f"team shapes {(E, H, N, D, B, T, pre, dt, masked)}")
+    assert sync_status() == 0
+
+
 ONE_TILE = [  # E, H, N, D, B, T, pre, dt, masked: heads whose aL / aR / Y do not fit in LDS as three (or two) tiles
     (2, 3, 512, 64, 32, 2, False, "bf16", False), (1, 4, 500, 64, 32, 3, True, "f16", True),
     (1, 2, 384, 64, 24, 1, False, "f16", True), (2, 2, 448, 64, 16, 2, True, "bf16", False),
