@@ -428,13 +428,17 @@ __device__ __forceinline__ void problem_sync() {
 // R step for one block problem (e,h,m), run by WPP waves (wig = wave in group).
 // smem: K tile, V tile, key bias.   Reference: al_cl_ref / al_y_cl_ref
 // (ma/ma_torch.py:10-23, :38-52).
-template <class T, int DT, int NWT>
+// HV = 2: the problem is run as two halves of NWT / 2 query strips by two workgroups, `half` = 0, 1 (both
+// stage the whole key / value tiles); a per-stage launch asks for it when it would not fill the device.
+template <class T, int DT, int NWT, int HV = 1>
 struct RProb {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
     static constexpr int WPP = Split<NWT>::WPP;
-    static constexpr int SPW = NWT / WPP;   // strips per wave: 2 for blocks of more than 64 rows (strip = wig + i * WPP)
+    static_assert(NWT % (WPP * HV) == 0, "a half must be whole strips per wave");
+    static constexpr int SPW = NWT / WPP / HV;   // strips per wave: 2 for blocks of more than 64 rows
     static constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
+    static __device__ __forceinline__ int strip_of(int wig, int i, int half) { return half * (NWT / HV) + wig + i * WPP; }
     struct Pre {
         TileCopy<T, DT, ROWS, WPP * 64> kc, vc;
         V8 xq[SPW][G::KS];   // first step: the Q rows of this wave's strips
@@ -452,7 +456,7 @@ struct RProb {
     // caller that streams everything else measured 3 - 5 % faster at T = 2, 3 with Q kept (T = 1: no gain).
     template <bool NT = false>
     static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int e, int m, bool first,
-                                                 bool with_v, int wig, int lane) {
+                                                 bool with_v, int wig, int lane, int half = 0) {
         if (!active) return;
         const int B = P.B, D = P.D;
         const int tix = wig * 64 + lane;
@@ -462,7 +466,7 @@ struct RProb {
         if (first) {
 #pragma unroll
             for (int i = 0; i < SPW; ++i) {
-                const int j = 16 * (wig + i * WPP) + (lane & 15);
+                const int j = 16 * strip_of(wig, i, half) + (lane & 15);
                 const unsigned ro = j < B ? tok_off(t0 + j, P.N, S.qst) : kOob;
                 if (NT && P.T == 1) load_x<T, DT, true>(pre.xq[i], S.q, ro, D, lane >> 4);
                 else load_x<T, DT, false>(pre.xq[i], S.q, ro, D, lane >> 4);
@@ -490,16 +494,16 @@ struct RProb {
     }
 
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int m, bool first, int wig,
-                                                 int lane) {
+                                                 int lane, int half = 0) {
 #pragma unroll
         for (int i = 0; i < SPW; ++i) {
             st.cr[i] = 1.0f;
-            if (active && !first) load_state_strip(P, S, st.xa[i], st.cr[i], m, wig + i * WPP, lane);
+            if (active && !first) load_state_strip(P, S, st.xa[i], st.cr[i], m, strip_of(wig, i, half), lane);
         }
     }
 
     static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
-                                               int m, bool first, bool with_v, int wig, int lane) {
+                                               int m, bool first, bool with_v, int wig, int lane, int half = 0) {
         T* Kt = reinterpret_cast<T*>(smem);
         T* Vt = Kt + Lds<T, DT, NWT>::TILE;
         float* kbias = reinterpret_cast<float*>(Vt + Lds<T, DT, NWT>::TILE);
@@ -520,7 +524,7 @@ struct RProb {
           bool jv = false;
           unsigned lrow = 0;
           if (active) {
-            const int strip = wig + si * WPP;
+            const int strip = strip_of(wig, si, half);
             const int j = 16 * strip + r;
             jv = j < B;
             V8 xb[G::KS];
@@ -614,13 +618,15 @@ struct TileIndex {
 
 // Z step for one column problem (e,h,j).  smem: aL tile, Y tile, cL bias.
 // Reference: z_ref (ma/ma_torch.py:55-62) and the final slice (:106-108).
-template <class T, int DT, int NWT>
+template <class T, int DT, int NWT, int HV = 1>   // HV: as in RProb
 struct ZProb {
     using G = Geom<DT>;
     using V8 = typename Ops<T>::v8;
     static constexpr int WPP = Split<NWT>::WPP;
     static constexpr int ROWS = Lds<T, DT, NWT>::ROWS;
-    static constexpr int SPW = NWT / WPP;   // strips per wave (strip = wig + i * WPP)
+    static_assert(NWT % (WPP * HV) == 0, "a half must be whole strips per wave");
+    static constexpr int SPW = NWT / WPP / HV;   // strips per wave
+    static __device__ __forceinline__ int strip_of(int wig, int i, int half) { return half * (NWT / HV) + wig + i * WPP; }
     struct Pre {
         V8 xq[SPW][G::KS];   // the Q rows of this wave's strips
     };
@@ -636,10 +642,11 @@ struct ZProb {
         load_x<T, DT, NT>(xb, S.q, ti.ok(P, l) ? tok_off(ti.token(P, l), P.N, S.qst) : kOob, P.D, lane >> 4);
     }
     template <bool NT = false>
-    static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int j, int wig, int lane) {
+    static __device__ __forceinline__ void issue(const Problem& P, const Slices& S, Pre& pre, bool active, int j, int wig, int lane,
+                                                 int half = 0) {
         if (!active) return;
 #pragma unroll
-        for (int i = 0; i < SPW; ++i) load_strip<NT>(P, S, pre.xq[i], j, wig + i * WPP, lane);
+        for (int i = 0; i < SPW; ++i) load_strip<NT>(P, S, pre.xq[i], j, strip_of(wig, i, half), lane);
     }
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int j, int wig, int lane) {
         if (!active) return;
@@ -653,7 +660,7 @@ struct ZProb {
         st.yc.template issue<true>(S.Y, D, [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; }, tix);
     }
     static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
-                                               int j, int wig, int lane) {
+                                               int j, int wig, int lane, int half = 0) {
         T* At = reinterpret_cast<T*>(smem);
         T* Yt = At + Lds<T, DT, NWT>::TILE;
         float* cb = reinterpret_cast<float*>(Yt + Lds<T, DT, NWT>::TILE);
@@ -671,7 +678,7 @@ struct ZProb {
         for (int si = 0; si < SPW; ++si) {
           V8 pb[(NWT + 1) / 2];
           if (active) {
-            const int strip = wig + si * WPP;
+            const int strip = strip_of(wig, si, half);
             V8 xb[G::KS];
 #pragma unroll
             for (int ks = 0; ks < G::KS; ++ks) xb[ks] = pre.xq[si][ks];
@@ -710,7 +717,7 @@ struct ZProb {
             pack_p<T, NWT>(pb, C);
           }
           if (active) {
-            const int l = 16 * (wig + si * WPP) + r;
+            const int l = 16 * strip_of(wig, si, half) + r;
             f32x4 O[DT];
             gemm2<T, DT, NWT>(O, Yt, pb, r, q);
             store_row<T, DT>(S.out, ti.ok(P, l) ? tok_off(ti.token(P, l), P.N, S.ost) : kOob, D, O, q, S.stream_out);   // padded query rows are dropped (:108)
@@ -892,28 +899,28 @@ struct LProb {
 };
 
 // the three parts back to back (one launch per half step has nothing to overlap them with)
-template <class T, int DT, int NWT>
+template <class T, int DT, int NWT, int HV = 1>
 __device__ __forceinline__ void r_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int m,
-                                          bool first, bool with_v, int wig, int lane) {
-    using RP = RProb<T, DT, NWT>;
+                                          bool first, bool with_v, int wig, int lane, int half = 0) {
+    using RP = RProb<T, DT, NWT, HV>;
     const Slices S = make_slices<T>(P, e, h, wh);
     typename RP::Pre pre;
     typename RP::St st;
-    RP::issue(P, S, pre, active, e, m, first, false, wig, lane);
-    RP::state(P, S, st, active, m, first, wig, lane);
+    RP::issue(P, S, pre, active, e, m, first, false, wig, lane, half);
+    RP::state(P, S, st, active, m, first, wig, lane, half);
     if (with_v) RP::issue_v(P, S, pre, active, m, wig, lane);
-    RP::run(P, S, smem, pre, st, active, m, first, with_v, wig, lane);
+    RP::run(P, S, smem, pre, st, active, m, first, with_v, wig, lane, half);
 }
-template <class T, int DT, int NWT>
+template <class T, int DT, int NWT, int HV = 1>
 __device__ __forceinline__ void z_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int j,
-                                          int wig, int lane) {
-    using ZP = ZProb<T, DT, NWT>;
+                                          int wig, int lane, int half = 0) {
+    using ZP = ZProb<T, DT, NWT, HV>;
     const Slices S = make_slices<T>(P, e, h, wh);
     typename ZP::Pre pre;
     typename ZP::St st;
-    ZP::issue(P, S, pre, active, j, wig, lane);
+    ZP::issue(P, S, pre, active, j, wig, lane, half);
     ZP::state(P, S, st, active, j, wig, lane);
-    ZP::run(P, S, smem, pre, st, active, j, wig, lane);
+    ZP::run(P, S, smem, pre, st, active, j, wig, lane, half);
 }
 template <class T, int DT, int NWT>
 __device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool active, int e, int h, long long wh, int j,
@@ -928,23 +935,33 @@ __device__ __forceinline__ void l_problem(const Problem& P, char* smem, bool act
 }
 
 // ---- staged kernels: one launch per half step ---------------------------------
-template <class T, int DT, int NWT>
+// Workgroup -> (problem, half) when a launch runs its problems as two halves (HV = 2, one problem per
+// workgroup): workgroups b and b + 8 are the halves of one problem - same XCD, dispatched close together,
+// so the second finds the operand tiles the first staged in that XCD's L2.
+__device__ __forceinline__ unsigned half_problem(unsigned b, int& half) {
+    half = static_cast<int>((b >> 3) & 1u);
+    return ((b >> 4) << 3) | (b & 7u);
+}
+
+template <class T, int DT, int NWT, int HV = 1>
 __global__ __launch_bounds__(64 * Split<NWT>::WG) void r_step_mfma(Problem P, int first, int with_v) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT, Split<NWT>::WG>::PPW;
+    static_assert(HV == 1 || PPW == 1, "halves: one problem per workgroup");
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
     // E * H * Np fits int32 (validated by the host), so all problem indices are 32-bit
     const unsigned total = static_cast<unsigned>(P.E) * P.H * P.M;
-    unsigned pid = blockIdx.x * PPW + slot;
+    int half = 0;
+    unsigned pid = HV == 1 ? blockIdx.x * PPW + slot : half_problem(blockIdx.x, half);
     const bool active = pid < total;
     if (!active) pid = 0;
     const int m = pid % static_cast<unsigned>(P.M);
     const unsigned eh = pid / static_cast<unsigned>(P.M);
     const int h = eh % static_cast<unsigned>(P.H);
     const int e = eh / static_cast<unsigned>(P.H);
-    r_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::R, active, e, h, static_cast<long long>(eh), m, first != 0,
-                          with_v != 0, wig, lane);
+    r_problem<T, DT, NWT, HV>(P, smem + slot * Lds<T, DT, NWT>::R, active, e, h, static_cast<long long>(eh), m, first != 0,
+                              with_v != 0, wig, lane, half);
 }
 
 template <class T, int DT, int NWT>
@@ -967,24 +984,26 @@ __global__ __launch_bounds__(64 * Split<NWT>::WG) void l_step_mfma(Problem P) {
     l_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::L, active, e, h, static_cast<long long>(eh), j, wig, lane);
 }
 
-template <class T, int DT, int NWT>
+template <class T, int DT, int NWT, int HV = 1>
 __global__ __launch_bounds__(64 * Split<NWT>::WG) void z_step_mfma(Problem P) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int WPP = Split<NWT>::WPP, PPW = Split<NWT, Split<NWT>::WG>::PPW;
+    static_assert(HV == 1 || PPW == 1, "halves: one problem per workgroup");
     const int wave = wave_id(), lane = threadIdx.x & 63;
     const int slot = wave / WPP, wig = wave % WPP;
     // problems per head: one per in-block position, or per group of positions that share a tile (TileIndex)
     const unsigned per = NWT == 1 ? static_cast<unsigned>(16 >> P.pack_shift) : 1u;
     const unsigned groups = (static_cast<unsigned>(P.B) + per - 1) / per;
     const unsigned total = static_cast<unsigned>(P.E) * P.H * groups;
-    unsigned pid = blockIdx.x * PPW + slot;
+    int half = 0;
+    unsigned pid = HV == 1 ? blockIdx.x * PPW + slot : half_problem(blockIdx.x, half);
     const bool active = pid < total;
     if (!active) pid = 0;
     const int j = static_cast<int>((pid % groups) * per);
     const unsigned eh = pid / groups;
     const int h = eh % static_cast<unsigned>(P.H);
     const int e = eh / static_cast<unsigned>(P.H);
-    z_problem<T, DT, NWT>(P, smem + slot * Lds<T, DT, NWT>::Z, active, e, h, static_cast<long long>(eh), j, wig, lane);
+    z_problem<T, DT, NWT, HV>(P, smem + slot * Lds<T, DT, NWT>::Z, active, e, h, static_cast<long long>(eh), j, wig, lane, half);
 }
 
 }  // namespace mfma

@@ -97,6 +97,20 @@ int for_classes(int dt, int nt, F&& f) {
 #undef MA_NT
 }
 
+// Problems of 6 or 8 strips (one per workgroup, two strips per wave) can run as two workgroups of one strip
+// per wave each.  That pays when the launch does not fill the device: with both halves of every problem
+// inside the workgroup slots the device offers at once, twice as many waves work on the same bytes (8 heads
+// of 64 128-row blocks: 21.9 -> 20.2 us per forward, 2 heads: 13.8 -> 11.6).  Launches of more than one
+// round of slots gain nothing from halves (the dispatcher refills slots as workgroups end; measured 55.1 ->
+// 56.8 us for 1536 problems on 1024 slots) and stay whole.  *err is set when the device cannot be queried.
+template <class K>
+bool halves_pay(K whole, int threads, size_t lds, long long problems, int* err) {
+    const DeviceCaps caps = device_caps(whole, threads, lds);
+    *err = caps.err;
+    const long long slots = static_cast<long long>(caps.cus) * caps.per_cu;
+    return !caps.err && 2 * problems <= slots;
+}
+
 template <class T>
 int launch_r(const Problem& P, bool first, bool with_v, hipStream_t s) {
     return for_classes(dt_class(P.D), nt_class(P.B), [&](auto dt, auto nt) {
@@ -106,6 +120,17 @@ int launch_r(const Problem& P, bool first, bool with_v, hipStream_t s) {
         const int attr = set_lds_limit(r_step_mfma<T, DT, NWT>, lds);
         if (attr) return attr;
         const long long problems = static_cast<long long>(P.E) * P.H * P.M;
+        if constexpr (NWT == 6 || NWT == 8) {
+            int err = 0;
+            if (halves_pay(r_step_mfma<T, DT, NWT>, 64 * WG, lds, problems, &err)) {
+                const int attr2 = set_lds_limit(r_step_mfma<T, DT, NWT, 2>, lds);
+                if (attr2) return attr2;
+                hipLaunchKernelGGL((r_step_mfma<T, DT, NWT, 2>), dim3(16 * ((problems + 7) / 8)), dim3(64 * WG), lds, s, P,
+                                   first ? 1 : 0, with_v ? 1 : 0);
+                return static_cast<int>(hipGetLastError());
+            }
+            if (err) return err;
+        }
         hipLaunchKernelGGL((r_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(64 * WG), lds, s, P,
                            first ? 1 : 0, with_v ? 1 : 0);
         return static_cast<int>(hipGetLastError());
@@ -137,6 +162,16 @@ int launch_z(const Problem& P, hipStream_t s) {
         if (attr) return attr;
         const long long per = NWT == 1 ? (16 >> P.pack_shift) : 1;
         const long long problems = static_cast<long long>(P.E) * P.H * ((P.B + per - 1) / per);
+        if constexpr (NWT == 6 || NWT == 8) {
+            int err = 0;
+            if (halves_pay(z_step_mfma<T, DT, NWT>, 64 * WG, lds, problems, &err)) {
+                const int attr2 = set_lds_limit(z_step_mfma<T, DT, NWT, 2>, lds);
+                if (attr2) return attr2;
+                hipLaunchKernelGGL((z_step_mfma<T, DT, NWT, 2>), dim3(16 * ((problems + 7) / 8)), dim3(64 * WG), lds, s, P);
+                return static_cast<int>(hipGetLastError());
+            }
+            if (err) return err;
+        }
         hipLaunchKernelGGL((z_step_mfma<T, DT, NWT>), dim3((problems + PPW - 1) / PPW), dim3(64 * WG), lds, s, P);
         return static_cast<int>(hipGetLastError());
     });
