@@ -258,7 +258,10 @@ bool fused_full_width(const ma_fwd_params* p) {
 //    pins heads to; head dims above 80 with more than 64 blocks of 64
 //    rows and more; fewer than 8 heads of thousands of tokens (a head's tasks all run on one
 //    XCD); a single step on an uneven head count from 4096 tokens on, or on 8 heads from ~7000
-//    on (two launches against an unbalanced one); blocks or block counts of 129 .. 256 rows
+//    on (two launches against an unbalanced one); few problems of 65 .. 128 rows (a single step:
+//    up to ~160 R problems, or 512 on at most 8 heads; more steps, 97 .. 128 rows only: up to 48,
+//    or at most 4 heads of up to 4096 tokens), which the stage kernels split in halves when a launch would leave the
+//    device mostly empty (10 - 30 % ahead there); blocks or block counts of 129 .. 256 rows
 //    (heads of up to 65536 tokens), which only the stage kernels have tile classes for;
 //  * else the chained kernel (one launch, tasks in dispatch order): 10 - 25 % ahead of the stage
 //    launches over most of the sweep, heads of 2 .. 8 blocks included (their L / Z problems share
@@ -288,7 +291,15 @@ int select_variant(const ma_fwd_params* p) {
                 const bool wide_dim = p->D > 80 && M > 64 && p->B >= 64;
                 const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
                 const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 7168));
-                if (!uneven_128 && !wide_dim && !few_heads && !one_step && chain_fits(p))
+                // launches that leave most of the device empty: the stage kernels run their 6- and 8-strip R and Z
+                // problems as two workgroups each then (halves_pay), which the one-launch kernels do not
+                const bool rows_halve = p->B > 64 && p->B <= 128, blocks_halve = M > 64 && M <= 128;
+                const long long r_problems = heads * M;
+                const bool underfilled =
+                    (rows_halve && (p->T == 1 ? (r_problems <= 160 || (heads <= 8 && r_problems <= 512))
+                                              : p->B > 96 && (r_problems <= 48 || (heads <= 4 && p->N <= 4096)))) ||
+                    (blocks_halve && p->T == 1 && heads * p->B <= 128);
+                if (!uneven_128 && !wide_dim && !few_heads && !one_step && !underfilled && chain_fits(p))
                     return MA_VARIANT_CHAINED;
             }
             return MA_VARIANT_STAGED;

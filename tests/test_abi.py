@@ -182,6 +182,10 @@ def test_auto_variant_policy():
     assert auto(1, 8, 6144, 64, 64) == "chained"        # 96 blocks: the team kernel would run them as 128
     assert auto(1, 8, 8192, 64, 64, T=1) == "staged"    # a single step: two launches
     assert auto(1, 8, 4096, 64, 64, T=1) == "chained"   # ... and teams only when they fill every workgroup slot (16 heads)
+    assert auto(1, 8, 2048, 64, 128, T=1) == "staged"   # few 128-row problems: the stage launches run them as halves
+    assert auto(1, 16, 2048, 64, 128, T=1) == "chained" # ... 256 of them on 16 heads: one launch again
+    assert auto(1, 4, 4096, 64, 128) == "staged"        # more steps: only very few problems, or at most 4 heads
+    assert auto(1, 8, 2048, 64, 128) == "chained"
     assert auto(1, 8, 1024, 64, 32) == "chained"        # teams of 16 workgroups: the chained kernel is ahead
     assert auto(1, 12, 4096, 64, 64) == "chained"       # 12 heads do not sit evenly on 8 XCDs: no teams
     assert auto(1, 12, 4096, 64, 64, T=1) == "staged"   # ... and with a single step two launches beat an unbalanced one
