@@ -32,13 +32,33 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def build(verbose: bool = False, jobs: int = 8) -> str:
+def depends_on(src: str) -> set:
+    """`src` and the headers of this tree it includes, directly or not."""
+    seen, todo = set(), [src]
+    while todo:
+        f = todo.pop()
+        if f in seen or not os.path.exists(f):
+            continue
+        seen.add(f)
+        with open(f) as fh:
+            for line in fh:
+                if line.startswith('#include "'):
+                    name = line.split('"')[1]
+                    todo += [os.path.join(CSRC, name), os.path.join(ROOT, "include", name)]
+    return seen
+
+
+def build(verbose: bool = False, jobs: int = 8, incremental: bool = False) -> str:
+    """Compile every source and link the library.  incremental: keep the objects that are newer than
+    their source and every header it includes (a developer's shortcut; the default compiles everything)."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(OBJ_DIR, exist_ok=True)
 
     def compile_one(src):
         obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
+        if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(f) for f in depends_on(src)):
+            return obj
         cmd = [hipcc, *FLAGS, "-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -63,4 +83,4 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, incremental="--incremental" in sys.argv))

@@ -106,24 +106,29 @@ __device__ __forceinline__ void swap_rows16(float& a, float& b) {
 __device__ __forceinline__ void swap_halves32(float& a, float& b) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
 }
+// (the maximum / sum sits inside the asm statement: on a value that comes out of one the compiler would first
+// quieten a possible signalling NaN with an extra instruction per operand; the s_nop behind the swap covers the
+// wait states a VALU read of its results needs.  The statements are volatile on purpose: they keep their place
+// in the instruction stream, and with it the compiler from moving the loads and matrix products of a whole block
+// problem in front of its softmax, which costs twice the registers.)
 __device__ __forceinline__ float quad_rows_max(float x) {
     float a = x, b = x;
-    swap_rows16(a, b);
-    x = fmaxf(a, b);
-    a = x, b = x;
-    swap_halves32(a, b);
-    return fmaxf(a, b);
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1\n\tv_max_f32 %0, %0, %1" : "+v"(a), "+v"(b));
+    b = a;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1\n\tv_max_f32 %0, %0, %1" : "+v"(a), "+v"(b));
+    return a;
 }
 __device__ __forceinline__ float quad_rows_sum(float x) {
     float a = x, b = x;
-    swap_rows16(a, b);
-    x = a + b;
-    a = x, b = x;
-    swap_halves32(a, b);
-    return a + b;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1\n\tv_add_f32 %0, %0, %1" : "+v"(a), "+v"(b));
+    b = a;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1\n\tv_add_f32 %0, %0, %1" : "+v"(a), "+v"(b));
+    return a;
 }
 // 1 / x to 1 ulp (v_rcp_f32) instead of the ten-instruction IEEE division
 __device__ __forceinline__ float rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+// log2(x) of a normal positive x to 1 ulp (v_log_f32), without the denormal handling of the library call
+__device__ __forceinline__ float log2_normal(float x) { return __builtin_amdgcn_logf(x); }
 
 // ---- global memory through buffer resources ---------------------------------
 // Every tensor slice a block problem touches is addressed as (uniform base in
@@ -573,7 +578,7 @@ struct RProb {
             // cL = sum_i r log r with r = p / den (ma_torch.py:20); rows of tiny r add ~1e-36
             lrow = static_cast<unsigned>(j * M + m);   // row of aL / cL / Y: (j, m)
             if (q == 0)
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, kLn2 * ent * inv - __logf(den) * (sum * inv)),
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, kLn2 * (ent * inv - log2_normal(den) * (sum * inv))),
                                                       S.cL, jv ? lrow * 4u : kOob, 0, 0);
 
             pack_p<T, NWT>(pb, C);

@@ -299,7 +299,7 @@ struct Resident {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) C[wt][v] *= inv;
             const int lrow = j * M + m;
-            if (jv && q == 0) c.cLs[lrow] = kLn2 * ent * inv - __logf(den) * (sum * inv);
+            if (jv && q == 0) c.cLs[lrow] = kLn2 * (ent * inv - log2_normal(den) * (sum * inv));
             V8 pb[(NTB + 1) / 2];
             pack_p<T, NTB>(pb, C);
             {

@@ -6,6 +6,7 @@
 
 #include "ma_mfma_launch.h"
 #include "ma_resident.h"
+#include "ma_resident_head.h"
 
 namespace ma {
 namespace mfma {
@@ -54,10 +55,41 @@ int launch_resident_w(const Problem& P, bool dry_run, hipStream_t s) {
                                 : launch_resident_mode<T, DT, NTB, NTM, W, false>(P, mode, lds, s);
 }
 
+// Heads whose inputs fit the LDS beside the state: the head-resident kernel (one workgroup per CU).
+template <class T, int DT, int NTB, int NTM, int W, int NI>
+int launch_resident_head_ni(const Problem& P, bool dry_run, hipStream_t s) {
+    using HR = HeadRes<T, DT, NTB, NTM, W, NI>;
+    const int Np = P.M * P.B;
+    if (!HR::fits(Np, P.B, P.M, kLdsPerCu)) return MA_ERR_UNSUPPORTED;
+    if (dry_run) return MA_OK;
+    auto kernel = resident_head_mfma<T, DT, NTB, NTM, W, NI>;
+    const int lds_err = set_lds_limit(kernel, kLdsPerCu);
+    if (lds_err) return lds_err;
+    const DeviceCaps caps = device_caps(kernel, 0, 0);
+    if (caps.err) return caps.err;
+    if (caps.cus < 1) return MA_ERR_DEVICE;
+    const long long heads = static_cast<long long>(P.E) * P.H;
+    const long long grid = heads < caps.cus ? heads : caps.cus;
+    hipLaunchKernelGGL((resident_head_mfma<T, DT, NTB, NTM, W, NI>), dim3(grid), dim3(64 * W), HR::layout(Np, P.B, P.M).total, s, P);
+    return static_cast<int>(hipGetLastError());
+}
+template <class T, int DT, int NTB, int NTM>
+int launch_resident_head(const Problem& P, bool dry_run, hipStream_t s) {
+    constexpr int W = (NTB <= 2 && NTM <= 2) ? 16 : 8;
+    // two 16-byte chunks per thread and input tile where that covers the head (fewer registers held through the rounds), else three
+    const int err = launch_resident_head_ni<T, DT, NTB, NTM, W, 2>(P, dry_run, s);
+    if (err != MA_ERR_UNSUPPORTED) return err;
+    return launch_resident_head_ni<T, DT, NTB, NTM, W, 3>(P, dry_run, s);
+}
+
 // The problems of a head are small and latency-bound: more waves per workgroup run more of
 // them at once, so the wide workgroup is preferred wherever its staging fits beside the state.
 template <class T, int DT, int NTB, int NTM>
 int launch_resident_one(const Problem& P, bool dry_run, hipStream_t s) {
+    {   // everything in LDS where the head is short enough for that
+        const int err = launch_resident_head<T, DT, NTB, NTM>(P, dry_run, s);
+        if (err != MA_ERR_UNSUPPORTED) return err;
+    }
     if constexpr (NTB <= 2 && NTM <= 2) {
         const int err = launch_resident_w<T, DT, NTB, NTM, kResidentWavesWide>(P, dry_run, s);
         if (err != MA_ERR_UNSUPPORTED) return err;
