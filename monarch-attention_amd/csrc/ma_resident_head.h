@@ -87,7 +87,10 @@ struct HeadRes {
     // input tile (row c / CH, 16-byte piece c % CH), and the mask element of one token.
     struct Pre {
         u32x4 q[NI], k[NI], v[NI];
-        u32x2 mk;
+        // mask element of the thread's token, as loaded; one register per element width: a single one written by
+        // loads of different widths is merged with copies, and a copy waits for the load
+        unsigned mk8, mk16, mk32;
+        u32x2 mk64;
     };
     struct Ctx {
         char* smem;
@@ -125,10 +128,8 @@ struct HeadRes {
         return hd;
     }
 
-    // The loads of the next head, in three parts (Q and the mask, K, V) that are started at the top of three
-    // different phases of the current head: all at once they would hold every wave at the memory pipeline's
-    // queue for half a microsecond, in front of a barrier.  Their offsets are recomputed every time: a few
-    // dozen instructions per head, against registers that would be held through every round.
+    // The loads of the next head: Q and the mask, K, V.  Their offsets are recomputed every time: a few dozen
+    // instructions per head, against registers that would be held through every round.
     static __device__ __forceinline__ void chunk_offsets(const Problem& P, const Ctx& c, unsigned st, unsigned (&off)[NI]) {
         const int Np = P.M * P.B;
 #pragma unroll
@@ -144,12 +145,10 @@ struct HeadRes {
             // the thread's entry of tokb: block tid / ROWSB, row tid % ROWSB
             const int m = c.tid / ROWSB, i = c.tid % ROWSB, t = m * P.B + i - P.pad_off;
             const unsigned moff = (m < P.M && i < P.B && static_cast<unsigned>(t) < static_cast<unsigned>(P.N)) ? static_cast<unsigned>(t) * c.mst : kOob;
-            switch (P.mask_shift) {   // uniform
-                case 0: pre.mk[0] = __builtin_amdgcn_raw_buffer_load_b8(hd.mask, moff, 0, 0); break;
-                case 1: pre.mk[0] = __builtin_amdgcn_raw_buffer_load_b16(hd.mask, moff, 0, 0); break;
-                case 2: pre.mk[0] = __builtin_amdgcn_raw_buffer_load_b32(hd.mask, moff, 0, 0); break;
-                default: pre.mk = __builtin_amdgcn_raw_buffer_load_b64(hd.mask, moff, 0, 0);
-            }
+            if (P.mask_shift == 0) pre.mk8 = __builtin_amdgcn_raw_buffer_load_b8(hd.mask, moff, 0, 0);   // uniform, all four
+            if (P.mask_shift == 1) pre.mk16 = __builtin_amdgcn_raw_buffer_load_b16(hd.mask, moff, 0, 0);
+            if (P.mask_shift == 2) pre.mk32 = __builtin_amdgcn_raw_buffer_load_b32(hd.mask, moff, 0, 0);
+            if (P.mask_shift == 3) pre.mk64 = __builtin_amdgcn_raw_buffer_load_b64(hd.mask, moff, 0, 0);
         }
         unsigned off[NI];
         chunk_offsets(P, c, c.qst, off);
@@ -183,7 +182,10 @@ struct HeadRes {
     static __device__ __forceinline__ void commit_tokb(const Problem& P, const Ctx& c, const Pre& pre) {
         const int m = c.tid / ROWSB, i = c.tid % ROWSB, t = m * P.B + i - P.pad_off;
         bool keep = m < P.M && i < P.B && static_cast<unsigned>(t) < static_cast<unsigned>(P.N);
-        if (P.mask != nullptr) keep = keep && mask_nonzero(P, pre.mk[0], P.mask_shift == 3 ? pre.mk[1] : 0u);   // uniform
+        if (P.mask != nullptr) {   // uniform
+            const unsigned lo = P.mask_shift == 0 ? pre.mk8 : P.mask_shift == 1 ? pre.mk16 : P.mask_shift == 2 ? pre.mk32 : pre.mk64[0];
+            keep = keep && mask_nonzero(P, lo, P.mask_shift == 3 ? pre.mk64[1] : 0u);
+        }
         if (m < P.M) c.fat(c.L.tokb)[c.tid] = keep ? 0.f : kNegBig;
     }
 
@@ -548,9 +550,11 @@ __global__ __launch_bounds__(64 * W) void resident_head_mfma(Problem P) {
         const int next = head + stride;
         const bool more = next < heads;
         typename HR::Head hn = hd;
-        // The next head's rows fly while this one computes.  (All of them are started here, at ONE place outside
-        // the loops over phases and rounds: loads that the compiler finds inside a loop it carries from iteration
-        // to iteration through register copies, and a copy of a register waits for the load that is still filling it.)
+        // The next head's rows fly while this one computes.  All of them are started here, at ONE place outside the
+        // loops over phases and rounds: loads started at several places of a loop are carried from iteration to
+        // iteration through register copies, and a copy of a register waits for the load that is still filling it.
+        // (While they arrive - 96 KB into the registers of a compute unit - the first phase runs at half its speed;
+        // starting them in front of a later phase, or a tile per phase, measured 1 - 2 us slower per forward.)
         if (more) {
             hn = HR::head_of(P, c, next);
             HR::issue_q(P, c, hn, pre);
