@@ -150,6 +150,9 @@ def main():
     ap.add_argument("--variant", default="auto", choices=["auto", "generic", "staged", "fused", "resident", "chained"])
     ap.add_argument("--rotate-workspaces", action="store_true",
                     help="a workspace per input set (default: all sets share one, like the calls of a model)")
+    ap.add_argument("--shared-device", action="store_true",
+                    help="do not state that the benchmark owns the GPU (MA_FLAG_DEVICE_EXCLUSIVE): 'auto' then never "
+                         "resolves to the fused kernel, as for a caller that shares the device")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sdpa", action="store_true", help="skip the dense SDPA comparison")
     ap.add_argument("--no-sweep", action="store_true", help="skip the T = 1, 2, 3 sweep over the variants")
@@ -183,7 +186,8 @@ def main():
     import torch
 
     from ma import _hip_lib as L
-    from ma.ma_hip import make_params, monarch_attention_hip
+    from ma import ma_hip
+    from ma.ma_hip import monarch_attention_hip
     from oracle.ma_oracle import forward_bytes, forward_flops, monarch_attention_oracle
 
     if not torch.cuda.is_available():
@@ -194,6 +198,18 @@ def main():
     stream = torch.cuda.current_stream(dev)
     sp = stream.cuda_stream
     F = torch.nn.functional
+
+    # The benchmark runs alone on its GPU and says so to the library (the fused kernel, whose
+    # workgroups wait for each other, is only chosen for such callers): in the parameter blocks it
+    # fills itself and, for the module-level leg, through the host wrapper's switch.
+    EXCL = 0 if args.shared_device else L.MA_FLAG_DEVICE_EXCLUSIVE
+    READY = L.MA_FLAG_SYNC_READY | EXCL
+    ma_hip.DEVICE_EXCLUSIVE = not args.shared_device
+
+    def make_params(*a, **kw):
+        p = ma_hip.make_params(*a, **kw)
+        p.flags = EXCL
+        return p
 
     def checked(status):
         if status:
@@ -249,7 +265,7 @@ def main():
             nbytes = lib.ma_fwd_workspace_bytes(ps[0])
             ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
             for p in ps:
-                p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), nbytes, L.MA_FLAG_SYNC_READY
+                p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), nbytes, READY
             variant = L.VARIANT_NAMES[lib.ma_fwd_select_variant(ps[0])]
             n = 100 if set_bytes < (1 << 30) else 20
             ma = batch_stats(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), n)
@@ -306,7 +322,7 @@ def main():
                 nbytes = lib.ma_fwd_workspace_bytes(ps[0])
                 ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
                 for p in ps:
-                    p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), nbytes, L.MA_FLAG_SYNC_READY
+                    p.workspace, p.workspace_bytes, p.flags = ws.data_ptr(), nbytes, READY
                 if any(lib.ma_fwd(ps[i % nbuf], sp) for i in range(4)):
                     continue   # e.g. a team grid that does not fit the device
                 row[variant] = round(batch_stats(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), 100)["median_ms"] * 1e3, 2)
@@ -352,7 +368,7 @@ def main():
         nws = max(1, min(nbuf, (2 << 30) // max(nbytes, 1))) if rotate else 1
         ws = [torch.zeros(nbytes, dtype=torch.uint8, device=dev) for _ in range(nws)]
         for i, p in enumerate(ps):
-            p.workspace, p.workspace_bytes, p.flags = ws[i % nws].data_ptr(), nbytes, L.MA_FLAG_SYNC_READY
+            p.workspace, p.workspace_bytes, p.flags = ws[i % nws].data_ptr(), nbytes, READY
         return ps, ws
 
     def run_steps(ps, n):
@@ -472,7 +488,8 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dt, "data": "synthetic",
         "config": {"workload": f"{args.config}: {dt} E{E} H{H} N{N} D{D} block{B} T{T} post-pad no-mask", "variant": resolved,
-                   "flop_per_fwd": flops, "compulsory_bytes_per_fwd": cbytes, "rotating_input_sets": nbuf, "rotating_workspaces": len(ws)},
+                   "flop_per_fwd": flops, "compulsory_bytes_per_fwd": cbytes, "rotating_input_sets": nbuf, "rotating_workspaces": len(ws),
+                   "device_exclusive": not args.shared_device},
         "stream_ms_per_step": round(ev_ms, 5),
         "ms_per_step_stats": timing,
         "fwd_hbm_frac": round(cbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

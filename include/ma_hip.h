@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define MA_ABI_VERSION 1
+#define MA_ABI_VERSION 2
 
 typedef enum ma_dtype { MA_F32 = 0, MA_F16 = 1, MA_BF16 = 2 } ma_dtype;
 
@@ -56,7 +56,10 @@ typedef enum ma_mask_dtype {
 } ma_mask_dtype;
 
 typedef enum ma_variant {
-    MA_VARIANT_AUTO = 0,    /* fastest variant that supports the problem            */
+    MA_VARIANT_AUTO = 0,    /* fastest variant that supports the problem and needs  */
+                            /* nothing of the rest of the device: FUSED is chosen    */
+                            /* only for callers that pass MA_FLAG_DEVICE_EXCLUSIVE,  */
+                            /* everybody else gets CHAINED or STAGED in its place    */
     MA_VARIANT_GENERIC = 1, /* FMA kernels, 2T(+T-1) launches: any dtype/shape/stride */
     MA_VARIANT_STAGED = 2,  /* MFMA kernels, one launch per half step (2T launches); */
                             /* 16-bit: blocks and block counts of up to 256 rows     */
@@ -66,9 +69,11 @@ typedef enum ma_variant {
                             /* per head, state exchanged through the workspace.  Its */
                             /* workgroups wait for each other, so the grid is sized  */
                             /* to what the device holds at once when idle: a kernel  */
-                            /* of another stream that occupies compute units for     */
-                            /* longer than the bounded waits (about a millisecond)   */
-                            /* makes the call fail loudly (NaN rows + error word)    */
+                            /* of another stream or process that occupies compute    */
+                            /* units for longer than the bounded waits (2^18 polls   */
+                            /* of the flag a workgroup waits for, 0.1 - 0.5 s) makes */
+                            /* the call fail loudly (NaN rows + error word).  Only   */
+                            /* for callers that own the device while the call runs   */
     MA_VARIANT_RESIDENT = 4,/* MFMA, ONE launch, one workgroup per head with the     */
                             /* per-head state resident in LDS (heads of up to ~256   */
                             /* tokens at d = 64; up to ~512 with Y passed through    */
@@ -90,7 +95,9 @@ typedef enum ma_status {
     MA_ERR_UNSUPPORTED = -6, /* the requested variant cannot run this problem     */
     MA_ERR_VARIANT = -7,     /* unknown ma_variant                                */
     MA_ERR_DEVICE = -8,      /* no usable gfx950 device / device query failed     */
-    MA_ERR_STATIC_LIMIT = -9 /* ma_fwd_static: state beyond the built-in scratch  */
+    MA_ERR_STATIC_LIMIT = -9,/* ma_fwd_static: state beyond the built-in scratch  */
+    MA_ERR_BUSY = -10        /* ma_fwd_static: the scratch is still in use by a   */
+                             /* call on another stream                            */
 } ma_status;
 
 /* ma_fwd_params.flags.  MA_FLAG_SYNC_READY: the caller guarantees that the sync
@@ -105,6 +112,14 @@ typedef enum ma_status {
  * out of time would, every kernel still runs to its end, and the next call on the
  * workspace is a normal one. */
 #define MA_FLAG_TEST_NO_SPIN 2
+/* MA_FLAG_DEVICE_EXCLUSIVE: the caller states that nothing else - no other stream, thread
+ * or process - competes for the device's compute units while this call runs.  Only then
+ * does MA_VARIANT_AUTO choose MA_VARIANT_FUSED, whose workgroups have to be on the device
+ * together (on the metric workload it is 10 - 15 % ahead of CHAINED).  Setting the
+ * environment variable MA_HIP_DEVICE_EXCLUSIVE=1 has the same effect for every call of the
+ * process.  Without either, AUTO stays with kernels that make progress beside any other
+ * work (CHAINED, RESIDENT, STAGED, GENERIC).  An explicit MA_VARIANT_FUSED is not affected. */
+#define MA_FLAG_DEVICE_EXCLUSIVE 4
 
 /* Arguments of one forward call; replaces the argument list of
  * monarch_attention_torch (ma/ma_torch.py:65-73). */
@@ -131,6 +146,13 @@ typedef struct ma_fwd_params {
     int64_t mask_stride[2];  /* element strides of (e, n)                        */
     float eps;               /* 1e-12 in the reference (ma/ma_torch.py:10,38)    */
     int32_t mask_dtype;      /* ma_mask_dtype of the mask's elements (0 = bytes)   */
+    uint32_t* error_word;    /* NULL, or a 32-bit word in pinned host memory the   */
+                             /* device can write (hipHostMalloc), zero before the  */
+                             /* call: a one-launch kernel whose wait runs out      */
+                             /* stores the code of the sticky error word (see      */
+                             /* ma_ws_layout) here as well, so that the host can    */
+                             /* look at it without a copy or a synchronisation of  */
+                             /* its own once the call's work is complete           */
 } ma_fwd_params;
 
 /* Byte offsets of the per-call state inside the workspace.  The arrays have
@@ -182,9 +204,15 @@ int ma_fwd(const ma_fwd_params* p, void* stream);
  * MA_STATIC_WORKSPACE_BYTES return MA_ERR_STATIC_LIMIT and launch nothing (the
  * metric workload, fp16 E=1 H=16 N=4096 D=64, needs 26.8 MiB).  No device memory
  * is allocated or freed.  All calls on one GPU share that GPU's array: calls that
- * overlap in time on one GPU (different streams or threads) race.  The first
- * call on a device looks up the array's address (not a stream operation: make it
- * once before capturing a graph). */
+ * overlap in time on one GPU (different streams or threads) race.  The library
+ * guards against the common case: a call on another stream than the previous
+ * call's, made while that call's work has not completed, returns MA_ERR_BUSY and
+ * launches nothing (calls on one stream are ordered and always accepted; streams
+ * that the caller orders with events must still not have a call in flight when the
+ * next is made - give such callers a workspace each through ma_fwd).  Under stream
+ * capture the guard is off: replays of a captured call cannot be seen by it.  The
+ * first call on a device looks up the array's address and creates the guard's event
+ * (not stream operations: make one call before capturing a graph). */
 #define MA_STATIC_WORKSPACE_BYTES (32u << 20)
 int ma_fwd_static(const ma_fwd_params* p, void* stream);
 

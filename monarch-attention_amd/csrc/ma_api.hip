@@ -5,6 +5,7 @@
 #include "ma_common.h"
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -30,7 +31,7 @@ int check_shape(const ma_fwd_params* p) {
     if (p->E < 1 || p->H < 1 || p->N < 1 || p->D < 1 || p->Dv < 1 || p->B < 1 || p->T < 1) return MA_ERR_SHAPE;
     if (!dtype_ok(p->dtype_qk) || !dtype_ok(p->dtype_v)) return MA_ERR_DTYPE;
     if (p->variant < MA_VARIANT_AUTO || p->variant > MA_VARIANT_CHAINED) return MA_ERR_VARIANT;
-    if (p->flags & ~(MA_FLAG_SYNC_READY | MA_FLAG_TEST_NO_SPIN)) return MA_ERR_SHAPE;
+    if (p->flags & ~(MA_FLAG_SYNC_READY | MA_FLAG_TEST_NO_SPIN | MA_FLAG_DEVICE_EXCLUSIVE)) return MA_ERR_SHAPE;
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
     const long long Np = M * p->B;
     // every launch grid and every in-kernel int index must stay inside int32
@@ -82,6 +83,7 @@ int check_buffers(const ma_fwd_params* p, const ma_ws_layout& L) {
     if (reinterpret_cast<uintptr_t>(p->q) % aq || reinterpret_cast<uintptr_t>(p->k) % aq ||
         reinterpret_cast<uintptr_t>(p->v) % av || reinterpret_cast<uintptr_t>(p->out) % av)
         return MA_ERR_STRIDE;
+    if (reinterpret_cast<uintptr_t>(p->error_word) % 4) return MA_ERR_STRIDE;
     return MA_OK;
 }
 
@@ -118,6 +120,7 @@ Problem make_problem(const ma_fwd_params* p, const ma_ws_layout& L) {
     P.sm_scale = static_cast<float>(1.0 / std::sqrt(static_cast<double>(p->D)));
     P.eps = p->eps;
     P.test_no_spin = (p->flags & MA_FLAG_TEST_NO_SPIN) ? 1 : 0;
+    P.host_error = p->error_word;
     P.pack_shift = 4;
     return P;
 }
@@ -252,7 +255,9 @@ bool fused_full_width(const ma_fwd_params* p) {
 //    1.05 - 1.3);
 //  * the fused kernel (one team of workgroups per head, counter barriers) for 8 or 16 heads whose
 //    phases fill the device (fused_full_width; the metric workload: 17.7 us against 20.0 chained
-//    and 22.4 as two launches);
+//    and 22.4 as two launches) - only for callers that own the device (device_exclusive): its
+//    workgroups wait for each other, and beside a kernel of somebody else they may not all be
+//    running; everybody else continues down this list;
 //  * one launch per half step where the one-launch kernels are at a disadvantage: 128-row
 //    problems both ways on a head count that does not divide by the 8 XCDs the chained kernel
 //    pins heads to; head dims above 80 with more than 64 blocks of 64
@@ -266,6 +271,17 @@ bool fused_full_width(const ma_fwd_params* p) {
 //  * else the chained kernel (one launch, tasks in dispatch order): 10 - 25 % ahead of the stage
 //    launches over most of the sweep, heads of 2 .. 8 blocks included (their L / Z problems share
 //    tiles, see pack_shift_of).
+// Does the caller own the device while its calls run (MA_FLAG_DEVICE_EXCLUSIVE, or the environment
+// variable MA_HIP_DEVICE_EXCLUSIVE set to something other than 0 / empty)?  Only then may AUTO choose
+// the fused kernel, whose workgroups wait for each other and so must all be on the device together.
+bool device_exclusive(const ma_fwd_params* p) {
+    static const bool env = [] {
+        const char* v = std::getenv("MA_HIP_DEVICE_EXCLUSIVE");
+        return v != nullptr && v[0] != '\0' && !(v[0] == '0' && v[1] == '\0');
+    }();
+    return env || (p->flags & MA_FLAG_DEVICE_EXCLUSIVE) != 0;
+}
+
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
     const bool fast32 = mfma32_supported(p);   // fp32 operands: per-stage launches only
@@ -286,7 +302,7 @@ int select_variant(const ma_fwd_params* p) {
                 if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D <= 64 &&
                     ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))
                     return MA_VARIANT_RESIDENT;
-                if (fused_full_width(p)) return MA_VARIANT_FUSED;
+                if (device_exclusive(p) && fused_full_width(p)) return MA_VARIANT_FUSED;
                 const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
                 const bool wide_dim = p->D > 80 && M > 64 && p->B >= 64;
                 const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
@@ -306,8 +322,9 @@ int select_variant(const ma_fwd_params* p) {
     }
 }
 
-__global__ void zero_sync_kernel(unsigned* sync, int words) {
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x) sync[i] = 0u;
+// 16 bytes per lane and store, one workgroup per compute unit or so: the 2 MiB area is gone in two passes
+__global__ void zero_sync_kernel(uint4* sync, int chunks) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < chunks; i += gridDim.x * blockDim.x) sync[i] = make_uint4(0u, 0u, 0u, 0u);
 }
 
 struct Prepared {
@@ -442,31 +459,45 @@ int bwd_prepare(const ma_bwd_params* b, ma_fwd_params* pp, BwdLayout* L) {
 
 // Device address of `scratch` on the current device, resolved once per device.
 constexpr int kMaxDevices = 64;
+// Per device: the scratch array's address, and what the in-use guard of ma_fwd_static needs - an
+// event recorded behind the last call's work and the stream that call was made on.
+struct StaticScratch {
+    void* ptr = nullptr;
+    hipEvent_t done = nullptr;
+    hipStream_t last_stream = nullptr;
+    bool in_flight = false;
+};
 std::mutex g_scratch_mutex;
-void* g_scratch_ptr[kMaxDevices];
+StaticScratch g_scratch[kMaxDevices];
 
-int static_scratch(void** out) {
+// Looks up (first call on a device: sets up) the current device's entry; the caller holds g_scratch_mutex.
+int static_scratch(StaticScratch** out) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return static_cast<int>(e);
     if (dev < 0 || dev >= kMaxDevices) return MA_ERR_DEVICE;
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (g_scratch_ptr[dev] == nullptr) {
+    StaticScratch& sc = g_scratch[dev];
+    if (sc.ptr == nullptr) {
         void* ptr = nullptr;
         e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return static_cast<int>(e);
         if (ptr == nullptr) return MA_ERR_DEVICE;
-        g_scratch_ptr[dev] = ptr;
+        hipEvent_t ev = nullptr;
+        e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+        if (e != hipSuccess) return static_cast<int>(e);
+        sc.done = ev;
+        sc.ptr = ptr;
     }
-    *out = g_scratch_ptr[dev];
+    *out = &sc;
     return MA_OK;
 }
 
 }  // namespace
 
 int launch_zero_sync(unsigned* sync, hipStream_t s) {
-    const int words = static_cast<int>(kSyncAreaBytes / 4);
-    hipLaunchKernelGGL(zero_sync_kernel, dim3(8), dim3(256), 0, s, sync, words);
+    static_assert(kSyncAreaBytes % 16 == 0, "the sync area is cleared in 16-byte chunks");
+    const int chunks = static_cast<int>(kSyncAreaBytes / 16);   // the area starts the workspace: 256-byte aligned
+    hipLaunchKernelGGL(zero_sync_kernel, dim3(256), dim3(256), 0, s, reinterpret_cast<uint4*>(sync), chunks);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -489,6 +520,7 @@ const char* ma_strerror(int status) {
         case MA_ERR_UNSUPPORTED: return "the requested variant does not support this problem";
         case MA_ERR_VARIANT: return "unknown variant";
         case MA_ERR_DEVICE: return "no usable gfx950 device";
+        case MA_ERR_BUSY: return "the built-in scratch of ma_fwd_static is still in use by a call on another stream: order the calls on one stream, wait for the earlier one, or call ma_fwd with a workspace per stream";
         case MA_ERR_STATIC_LIMIT: return "the problem's state exceeds MA_STATIC_WORKSPACE_BYTES, the built-in scratch of ma_fwd_static: call ma_fwd with a workspace";
         default: break;
     }
@@ -569,16 +601,45 @@ int ma_fwd_static(const ma_fwd_params* p, void* stream) {
     int st = layout_of(p, &L);
     if (st != MA_OK) return st;
     if (L.total > MA_STATIC_WORKSPACE_BYTES) return MA_ERR_STATIC_LIMIT;
-    void* ptr = nullptr;
-    st = static_scratch(&ptr);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        capture = hipStreamCaptureStatusNone;
+    }
+    const bool capturing = capture != hipStreamCaptureStatusNone;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);   // the guard's bookkeeping; launches are short
+    StaticScratch* sc = nullptr;
+    st = static_scratch(&sc);
     if (st != MA_OK) return st;
+    // In-use guard: the array belongs to the last call until that call's work is complete.  A call on
+    // the same stream is ordered behind it; one on another stream is turned away while the event
+    // recorded behind the last call has not completed.  (Captured calls are neither checked nor
+    // recorded: an event recorded during capture belongs to the graph.)
+    if (!capturing && sc->in_flight && sc->last_stream != s) {
+        const hipError_t q = hipEventQuery(sc->done);
+        if (q == hipErrorNotReady) {
+            (void)hipGetLastError();
+            return MA_ERR_BUSY;
+        }
+        if (q != hipSuccess) return static_cast<int>(q);
+        sc->in_flight = false;
+    }
     ma_fwd_params pp = *p;
-    pp.workspace = ptr;
+    pp.workspace = sc->ptr;
     pp.workspace_bytes = MA_STATIC_WORKSPACE_BYTES;
     // the array keeps what the last call left: nothing may be assumed about its sync area, so the
     // one-launch variants clear it with their fill kernel in front of the forward kernel
     pp.flags &= ~MA_FLAG_SYNC_READY;
-    return ma_fwd(&pp, stream);
+    st = ma_fwd(&pp, stream);
+    if (!capturing) {
+        // also after a failed launch sequence: some of its kernels may have been queued
+        const hipError_t r = hipEventRecord(sc->done, s);
+        if (r != hipSuccess) return st != MA_OK ? st : static_cast<int>(r);
+        sc->last_stream = s;
+        sc->in_flight = true;
+    }
+    return st;
 }
 
 int ma_matrix(const ma_fwd_params* p, float* A, void* stream) {

@@ -80,17 +80,17 @@ __device__ __forceinline__ unsigned release_of(unsigned long long total, unsigne
 }
 
 // one thread: poll the release word of the previous phase; returns it, or 0 if the wait ran out
-__device__ __forceinline__ unsigned chain_wait(const unsigned* go, unsigned spin_limit, unsigned* error) {
+__device__ __forceinline__ unsigned chain_wait(const unsigned* go, unsigned spin_limit, unsigned* error, unsigned* host_error) {
     unsigned spins = 0;
     if (spin_limit == 0u) {   // failure-path tests: give up without looking, whatever the word holds
-        __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        raise_error(error, host_error, 1u);
         return 0u;
     }
     for (;;) {
         const unsigned w = __hip_atomic_load(go, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (w != 0u) return w;
         if (++spins > spin_limit) {
-            __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            raise_error(error, host_error, 1u);
             return 0u;
         }
         __builtin_amdgcn_s_sleep(2);
@@ -133,11 +133,11 @@ __global__ __launch_bounds__(64 * W) void chain_fwd_mfma(Problem P, ChainPlan pl
     auto wait_prev = [&] {
         if (p == 0) return;
         if (threadIdx.x == 0) {
-            const unsigned w = chain_wait(go + (p - 1), plan.spin_limit, error);
+            const unsigned w = chain_wait(go + (p - 1), plan.spin_limit, error, P.host_error);
             bool bad = w == 0u || (w & kGoFailed) != 0u;
             if (w != 0u && ((w & kGoSplit) != 0u || ((w >> 1) & 0xfu) != my_xcc)) {
                 // not the id -> XCD dealing this kernel is built on: what this task would read is not reliable
-                __hip_atomic_store(error, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                raise_error(error, P.host_error, 2u);
                 bad = true;
             }
             wg_word = bad ? 1u : 0u;

@@ -40,7 +40,17 @@ struct Problem {
     // three tiles do not fit (heads of up to ~512 tokens at d = 64).
     int one_tile_ok;
     int test_no_spin;    // waits between workgroups give up at once (failure-path tests)
+    // Copy of the error word in host memory the device can write (or null): a workgroup that raises the
+    // word in the sync area stores the code here as well, where the host reads it without a copy.
+    unsigned* host_error;
 };
+
+// Raise the sticky error word of the one-launch kernels: in the sync area of the workspace, and in the
+// caller's host-visible word if there is one.
+__device__ __forceinline__ void raise_error(unsigned* error, unsigned* host_error, unsigned code) {
+    __hip_atomic_store(error, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (host_error != nullptr) __hip_atomic_store(host_error, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // Is a mask element non-zero (torch.logical_and's truthiness, ma/ma_torch.py:98)?  `lo` / `hi` are
 // its low and high 32 bits (zero-extended for narrow elements); for floating-point masks the

@@ -70,6 +70,7 @@ struct TeamSync {
     unsigned* go;          // epoch of the latest complete barrier
     unsigned* xcc;         // [member] XCC (XCD) id the member runs on
     unsigned* error;
+    unsigned* host_error;
     unsigned* word;        // LDS word through which wave 0 tells the workgroup how a wait ended
     unsigned epoch;        // epoch of this member's latest arrival
     unsigned target;       // value of the counter when that barrier is complete
@@ -122,14 +123,14 @@ __device__ __forceinline__ void team_arrive(TeamSync& ts) {
 __device__ __forceinline__ bool poll_release(const TeamSync& ts) {
     unsigned spins = 0;
     if (ts.spin_limit == 0u) {   // failure-path tests: give up without looking, whatever the word holds
-        __hip_atomic_store(ts.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        raise_error(ts.error, ts.host_error, 1u);
         return false;
     }
     for (;;) {
         const unsigned f = __hip_atomic_load(ts.go, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (static_cast<int>(f - ts.epoch) >= 0) return true;
         if (++spins > ts.spin_limit) {
-            __hip_atomic_store(ts.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            raise_error(ts.error, ts.host_error, 1u);
             return false;
         }
         __builtin_amdgcn_s_sleep(2);
@@ -288,6 +289,7 @@ __global__ __launch_bounds__(64 * W) void fused_fwd_mfma(Problem P, FusedPlan pl
     ts.go = ts.base + kSyncGo;
     ts.xcc = ts.base + kSyncXcc;
     ts.error = P.sync + 1;
+    ts.host_error = P.host_error;
     ts.word = &team_word;
     ts.spin_limit = plan.spin_limit;
     ts.G = G;

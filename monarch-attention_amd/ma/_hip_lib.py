@@ -11,7 +11,7 @@ import ctypes as C
 import os
 import threading
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 MA_F32, MA_F16, MA_BF16 = 0, 1, 2
 VARIANTS = {"auto": 0, "generic": 1, "staged": 2, "fused": 3, "resident": 4, "chained": 5}
@@ -21,6 +21,7 @@ MA_OK = 0
 MA_ERR_NULL, MA_ERR_SHAPE, MA_ERR_DTYPE, MA_ERR_STRIDE = -1, -2, -3, -4
 MA_ERR_WORKSPACE, MA_ERR_UNSUPPORTED, MA_ERR_VARIANT, MA_ERR_DEVICE = -5, -6, -7, -8
 MA_ERR_STATIC_LIMIT = -9
+MA_ERR_BUSY = -10
 MA_STATIC_WORKSPACE_BYTES = 32 << 20
 
 
@@ -34,7 +35,7 @@ class FwdParams(C.Structure):
         ("dtype_qk", C.c_int32), ("dtype_v", C.c_int32), ("variant", C.c_int32), ("flags", C.c_int32),
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("out_stride", C.c_int64 * 3), ("mask_stride", C.c_int64 * 2),
-        ("eps", C.c_float), ("mask_dtype", C.c_int32),
+        ("eps", C.c_float), ("mask_dtype", C.c_int32), ("error_word", C.c_void_p),
     ]
 
 
@@ -55,6 +56,7 @@ class WsLayout(C.Structure):
 MA_MASK_U8, MA_MASK_I16, MA_MASK_I32, MA_MASK_I64, MA_MASK_F16, MA_MASK_BF16, MA_MASK_F32, MA_MASK_F64 = range(8)
 MA_FLAG_SYNC_READY = 1
 MA_FLAG_TEST_NO_SPIN = 2
+MA_FLAG_DEVICE_EXCLUSIVE = 4
 
 EXPORTS = ("ma_abi_version", "ma_strerror", "ma_fwd_workspace_layout", "ma_fwd_workspace_bytes",
            "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_fwd_static", "ma_r_step", "ma_l_step", "ma_z_step",

@@ -17,6 +17,9 @@ and the stream; all arithmetic happens in libma_hip.so.
 """
 from __future__ import annotations
 
+import os
+import threading
+
 import torch
 
 from . import _hip_lib as L
@@ -32,6 +35,14 @@ _MASK_DTYPES = {torch.bool: L.MA_MASK_U8, torch.uint8: L.MA_MASK_U8, torch.int8:
 # per call through the `variant` keyword
 DEFAULT_VARIANT = "auto"
 
+# Does this process own the GPU while its forward calls run - no other stream,
+# thread or process competing for compute units?  Only then may 'auto' resolve
+# to the 'fused' kernel, whose workgroups wait for each other and so must all be
+# on the device together (MA_FLAG_DEVICE_EXCLUSIVE).  Off unless the environment
+# says MA_HIP_DEVICE_EXCLUSIVE=1 or the application sets this attribute; 'auto'
+# then stays with kernels that make progress beside any other work.
+DEVICE_EXCLUSIVE = os.environ.get("MA_HIP_DEVICE_EXCLUSIVE", "") not in ("", "0")
+
 # One workspace per (device, stream), grown on demand and reused call after
 # call: calls on one stream are ordered, so they can share it.  It is allocated
 # zero-filled, and every forward call leaves its sync area in the state the next
@@ -40,28 +51,31 @@ DEFAULT_VARIANT = "auto"
 #
 # The one-launch kernels (fused, chained) wait for each other's workgroups with
 # bounded waits; a wait that runs out raises a sticky error word in the
-# workspace and the workgroup writes NaN instead of results.  That word is
-# brought to the host WITHOUT synchronising: every few calls a 4-byte copy into
-# pinned memory is queued on a side stream behind the forward kernel, and the
-# next call on the workspace that finds the copy complete looks at it - a failed
-# call is reported by a RuntimeError from a later call, the sync area is cleared
-# again, and the call after that is a normal one.
-_CHECK_EVERY = 16          # calls between two looks at the error word (the first call always looks)
+# workspace and the workgroup writes NaN instead of results.  The kernel stores
+# the same code into a word of pinned host memory that belongs to the workspace
+# (ma_fwd_params.error_word), and EVERY call on the workspace looks at that word
+# first - a plain host read, nothing is copied or synchronised: a failed call is
+# reported by a RuntimeError from the first later call that finds the word set
+# (at the latest the first call after the failed call's work has completed), the
+# sync area is cleared again, and the call after that is a normal one.
 _TEST_FLAGS = 0            # extra ma_fwd_params.flags for the failure-path tests (MA_FLAG_TEST_NO_SPIN)
 _SYNCING = (L.VARIANTS["fused"], L.VARIANTS["chained"])
 
 
 class _Workspace:
     def __init__(self, device: torch.device, nbytes: int):
-        self.buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         self.err_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
-        self.pending = None     # (event on the side stream, buffer the copy reads from)
-        self.calls = 0
+        self.err = self.err_host.numpy()          # the same word, read without a torch call
+        self.err_ptr = self.err_host.data_ptr()
         self.dirty = False      # the sync area must be cleared before the next one-launch kernel
+        self.resize(device, nbytes)
+
+    def resize(self, device: torch.device, nbytes: int) -> None:
+        self.buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        self.ptr, self.nbytes = self.buf.data_ptr(), self.buf.numel()
 
 
 _WORKSPACES: dict[tuple[int, int], _Workspace] = {}
-_SIDE_STREAMS: dict[int, torch.cuda.Stream] = {}
 
 
 def _workspace(device: torch.device, stream_ptr: int, nbytes: int) -> _Workspace:
@@ -69,46 +83,25 @@ def _workspace(device: torch.device, stream_ptr: int, nbytes: int) -> _Workspace
     w = _WORKSPACES.get(key)
     if w is None:
         w = _WORKSPACES[key] = _Workspace(device, nbytes)
-    elif w.buf.numel() < nbytes:
-        if w.pending is not None:          # let the queued look at the old buffer finish first
-            w.pending[0].synchronize()
-            _collect(w)
-        w.buf = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    elif w.nbytes < nbytes:
+        # calls on this stream that still use the old buffer are ahead of everything queued from here on,
+        # and the caching allocator hands a freed block to other streams only after that work is done
+        w.resize(device, nbytes)
     return w
 
 
-def _collect(w: _Workspace) -> None:
-    """Look at a completed copy of the error word; raise if a call on this workspace failed."""
-    w.pending = None
-    code = int(w.err_host.item())
-    if code == 0:
-        return
-    w.err_host.zero_()
+def _raise_failed(w: _Workspace) -> None:
+    """The host-visible error word of this workspace is set: an earlier call on it failed."""
+    code = int(w.err[0])
+    w.err[0] = 0
     w.dirty = True
-    w.buf[4:8].zero_()      # the word is sticky: clear it for the calls to come
+    w.buf[4:8].zero_()      # the word in the workspace is sticky: clear it for the calls to come
     what = {1: "a bounded wait between workgroups ran out",
             2: "workgroups of one head ran on different XCDs (the one-launch kernels rely on ids x, x + 8, ... "
                "sharing an XCD)"}.get(code, f"error word {code}")
     raise RuntimeError(f"monarch_attention_hip: an earlier forward call on this stream failed: {what}; its output "
                        f"holds NaN rows.  The workspace has been reset; pass variant='staged' to avoid the "
                        f"one-launch kernels")
-
-
-def _queue_check(w: _Workspace, device: torch.device, main: "torch.cuda.Stream") -> None:
-    """Queue a copy of the error word to pinned memory behind the work queued on `main` so far,
-    on a side stream: the main stream never waits for it."""
-    idx = device.index if device.index is not None else torch.cuda.current_device()
-    side = _SIDE_STREAMS.get(idx)
-    if side is None:
-        side = _SIDE_STREAMS[idx] = torch.cuda.Stream(device=device)
-    after = torch.cuda.Event()
-    after.record(main)
-    side.wait_event(after)
-    with torch.cuda.stream(side):
-        w.err_host.copy_(w.buf[4:8].view(torch.int32), non_blocking=True)
-        done = torch.cuda.Event()
-        done.record(side)
-    w.pending = (done, w.buf)
 
 
 def sync_status() -> int:
@@ -125,11 +118,10 @@ def sync_status() -> int:
 
 
 def clear_workspace_cache() -> None:
-    """Drop the cached per-stream workspaces (frees their device memory)."""
-    for w in _WORKSPACES.values():
-        if w.pending is not None:
-            w.pending[0].synchronize()
+    """Drop the cached per-stream workspaces (frees their device memory once the
+    work queued on them is complete) and the per-signature call plans."""
     _WORKSPACES.clear()
+    _TLS.__dict__.pop("plans", None)
 
 
 def _check_inputs(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int) -> None:
@@ -210,31 +202,54 @@ def make_params(q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B
     return p
 
 
-# Filling a ma_fwd_params field by field costs more host time than a small forward takes on the
-# GPU, and a model calls the operator with the same few shapes over and over: the filled block
-# (and the workspace size the library reports for it) is kept per call signature, and a call only
-# copies it and patches the pointers.
-_PARAM_CACHE: dict[tuple, tuple] = {}
-_PARAM_CACHE_MAX = 256
+# Filling a ma_fwd_params field by field, validating the arguments and asking the library for the
+# workspace size cost more host time than a small forward takes on the GPU, and a model calls the
+# operator with the same few signatures over and over.  Everything that depends on the signature
+# alone - shapes, strides, dtypes, devices, pointer alignment, T, B, padding side, variant - is
+# worked out once and kept as a plan: a validated, filled parameter block that later calls only
+# patch pointers into.  Plans are per thread (a block is modified in place right before the call).
+_TLS = threading.local()
+_PLAN_MAX = 256
 
 
-def _params_for(lib, q: Tensor, k: Tensor, v: Tensor, mask_u8, out: Tensor, T: int, B: int, pre_pad: bool,
-                variant: str) -> tuple:
-    key = (q.shape, q.stride(), k.stride(), v.shape, v.stride(), out.stride(),
-           None if mask_u8 is None else (mask_u8.stride(), mask_u8.dtype), q.dtype, v.dtype, T, B, bool(pre_pad), variant)
-    hit = _PARAM_CACHE.get(key)
-    if hit is None:
-        tmpl = make_params(q, k, v, mask_u8, out, T, B, pre_pad, variant)
-        nbytes = lib.ma_fwd_workspace_bytes(tmpl)
-        if nbytes == 0:   # invalid problem: let the library say why
-            L.check(lib.ma_fwd_workspace_layout(tmpl, L.WsLayout()), "monarch_attention_hip")
-        if len(_PARAM_CACHE) >= _PARAM_CACHE_MAX:
-            _PARAM_CACHE.clear()
-        hit = _PARAM_CACHE[key] = (bytes(tmpl), nbytes, lib.ma_fwd_select_variant(tmpl))
-    p = L.FwdParams.from_buffer_copy(hit[0])
-    p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
-    p.mask = mask_u8.data_ptr() if mask_u8 is not None else None
-    return p, hit[1], hit[2]
+class _Plan:
+    __slots__ = ("p", "ref", "nbytes", "syncing", "flags", "permuted", "alloc_shape", "dtype", "device", "index")
+
+
+def _signature(q: Tensor, k: Tensor, v: Tensor, attn_mask, T, B, pre_pad, variant, align: int) -> tuple:
+    return (q.shape, k.shape, v.shape, q.stride(), k.stride(), v.stride(), q.dtype, k.dtype, v.dtype,
+            q.device, k.device, v.device, T, B, not pre_pad, variant, DEVICE_EXCLUSIVE, _TEST_FLAGS, align,
+            None if attn_mask is None else (attn_mask.shape, attn_mask.stride(), attn_mask.dtype, attn_mask.device))
+
+
+def _make_plan(lib, q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int, pre_pad, variant):
+    """Validate a call signature and prepare its parameter block; None for inputs that have to be
+    copied first (the general path does that)."""
+    _check_inputs(q, k, v, attn_mask, T, B)
+    if _inner_contiguous(q) is not q or _inner_contiguous(k) is not k or _inner_contiguous(v) is not v:
+        return None
+    mask_u8 = _mask_bytes(attn_mask)
+    E, H, N, _ = q.shape
+    plan = _Plan()
+    with torch.cuda.device(q.device):
+        out = _empty_like_layout(v, (E, H, N, v.shape[-1]))
+    plan.permuted = not out.is_contiguous()
+    plan.alloc_shape = (E, N, H, v.shape[-1]) if plan.permuted else (E, H, N, v.shape[-1])
+    plan.dtype, plan.device = v.dtype, v.device
+    plan.index = v.device.index if v.device.index is not None else torch.cuda.current_device()
+    plan.flags = _TEST_FLAGS | (L.MA_FLAG_DEVICE_EXCLUSIVE if DEVICE_EXCLUSIVE else 0)
+    p = make_params(q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
+    p.flags = plan.flags
+    plan.nbytes = lib.ma_fwd_workspace_bytes(p)
+    if plan.nbytes == 0:   # invalid problem: let the library say why
+        L.check(lib.ma_fwd_workspace_layout(p, L.WsLayout()), "monarch_attention_hip")
+    plan.syncing = lib.ma_fwd_select_variant(p) in _SYNCING
+    plan.p, plan.ref = p, L.C.byref(p)
+    return plan
+
+
+def _raw_stream(index: int) -> int:
+    return torch._C._cuda_getCurrentRawStream(index)
 
 
 def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, T: int, B: int,
@@ -245,32 +260,83 @@ def monarch_attention_hip(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | N
     Differentiable with respect to q, k and v: when one of them requires grad
     (and grad mode is on) the call is recorded as one autograd node whose
     backward is ``ma_bwd``."""
-    _check_inputs(q, k, v, attn_mask, T, B)
-    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+    try:
+        needs_grad = (q.requires_grad or k.requires_grad or v.requires_grad) and torch.is_grad_enabled()
+        qp, kp, vp = q.data_ptr(), k.data_ptr(), v.data_ptr()
+        key = _signature(q, k, v, attn_mask, T, B, pre_pad, variant, (qp | kp | vp) & 15)
+    except (AttributeError, TypeError):
+        _check_inputs(q, k, v, attn_mask, T, B)   # says what is wrong with the arguments
+        raise
+    if needs_grad:
+        _check_inputs(q, k, v, attn_mask, T, B)
         return _MonarchAttentionHip.apply(q, k, v, attn_mask, T, B, bool(pre_pad), variant)
-    return _forward(q, k, v, attn_mask, T, B, pre_pad, variant)
+    try:
+        plans = _TLS.plans
+    except AttributeError:
+        plans = _TLS.plans = {}
+    plan = plans.get(key, False)
+    if plan is False:
+        plan = _make_plan(L.load(), q, k, v, attn_mask, T, B, pre_pad, variant)
+        if len(plans) >= _PLAN_MAX:
+            plans.clear()
+        plans[key] = plan
+    if plan is None or torch.cuda.current_device() != plan.index:
+        return _forward(q, k, v, attn_mask, T, B, pre_pad, variant)
+    out = torch.empty(plan.alloc_shape, dtype=plan.dtype, device=plan.device)
+    if plan.permuted:
+        out = out.permute(0, 2, 1, 3)
+    stream = _raw_stream(plan.index)
+    w = _WORKSPACES.get((plan.index, stream))
+    if w is None or w.nbytes < plan.nbytes:
+        w = _workspace(plan.device, stream, plan.nbytes)
+    if w.err[0]:
+        _raise_failed(w)   # an earlier call on this workspace failed
+    p = plan.p
+    p.q, p.k, p.v, p.out = qp, kp, vp, out.data_ptr()
+    if attn_mask is not None:
+        p.mask = attn_mask.data_ptr()
+    p.workspace, p.workspace_bytes, p.error_word = w.ptr, w.nbytes, w.err_ptr
+    p.flags = plan.flags if w.dirty else plan.flags | L.MA_FLAG_SYNC_READY
+    st = _FWD(plan.ref, stream)
+    if st:
+        L.check(st, "ma_fwd")
+    if plan.syncing:
+        w.dirty = False   # the library cleared the sync area in front of this launch if it had to
+    return out
+
+
+def _FWD(ref, stream) -> int:
+    """ma_fwd of the loaded library (replaces itself by the bound function on first use)."""
+    global _FWD
+    _FWD = L.load().ma_fwd
+    return _FWD(ref, stream)
 
 
 def _forward(q: Tensor, k: Tensor, v: Tensor, attn_mask, T: int, B: int, pre_pad: bool, variant) -> Tensor:
+    """The general path: any device, inputs that need a copy first; nothing is cached."""
     lib = L.load()
+    _check_inputs(q, k, v, attn_mask, T, B)
     q, k, v = _inner_contiguous(q), _inner_contiguous(k), _inner_contiguous(v)
     mask_u8 = _mask_bytes(attn_mask)
     E, H, N, _ = q.shape
     with torch.cuda.device(q.device):
         out = _empty_like_layout(v, (E, H, N, v.shape[-1]))
-        p, nbytes, resolved = _params_for(lib, q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
-        main = torch.cuda.current_stream(q.device)
-        w = _workspace(q.device, main.cuda_stream, nbytes)
-        if w.pending is not None and w.pending[0].query():
-            _collect(w)   # raises if an earlier call on this workspace failed
-        p.workspace, p.workspace_bytes = w.buf.data_ptr(), w.buf.numel()
-        p.flags = (0 if w.dirty else L.MA_FLAG_SYNC_READY) | _TEST_FLAGS
-        L.check(lib.ma_fwd(p, main.cuda_stream), "ma_fwd")
-        if resolved in _SYNCING:
+        p = make_params(q, k, v, mask_u8, out, T, B, pre_pad, variant or DEFAULT_VARIANT)
+        p.flags = _TEST_FLAGS | (L.MA_FLAG_DEVICE_EXCLUSIVE if DEVICE_EXCLUSIVE else 0)
+        nbytes = lib.ma_fwd_workspace_bytes(p)
+        if nbytes == 0:   # invalid problem: let the library say why
+            L.check(lib.ma_fwd_workspace_layout(p, L.WsLayout()), "monarch_attention_hip")
+        syncing = lib.ma_fwd_select_variant(p) in _SYNCING
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        w = _workspace(q.device, stream, nbytes)
+        if w.err[0]:
+            _raise_failed(w)   # an earlier call on this workspace failed
+        p.workspace, p.workspace_bytes, p.error_word = w.ptr, w.nbytes, w.err_ptr
+        if not w.dirty:
+            p.flags |= L.MA_FLAG_SYNC_READY
+        L.check(lib.ma_fwd(p, stream), "ma_fwd")
+        if syncing:
             w.dirty = False   # the library cleared the sync area in front of this launch if it had to
-            if w.pending is None and (w.calls % _CHECK_EVERY == 0 or _TEST_FLAGS):
-                _queue_check(w, q.device, main)
-            w.calls += 1
     return out
 
 

@@ -38,16 +38,16 @@ def test_struct_layout_matches_header(tmp_path):
     prog = tmp_path / "sz.c"
     prog.write_text(
         '#include <stdio.h>\n#include <stddef.h>\n#include "ma_hip.h"\n'
-        "int main(void){printf(\"%zu %zu %zu %zu %zu %zu\\n\", sizeof(ma_fwd_params), offsetof(ma_fwd_params,E),"
+        "int main(void){printf(\"%zu %zu %zu %zu %zu %zu %zu %zu\\n\", sizeof(ma_fwd_params), offsetof(ma_fwd_params,E),"
         " offsetof(ma_fwd_params,q_stride), offsetof(ma_fwd_params,mask_stride), offsetof(ma_fwd_params,eps),"
-        " sizeof(ma_ws_layout)); return 0;}\n")
+        " offsetof(ma_fwd_params,error_word), sizeof(ma_bwd_params), sizeof(ma_ws_layout)); return 0;}\n")
     exe = tmp_path / "sz"
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(prog), "-o", str(exe)],
                    check=True)
     got = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
     F = L.FwdParams
     assert got == [C.sizeof(F), F.E.offset, F.q_stride.offset, F.mask_stride.offset, F.eps.offset,
-                   C.sizeof(L.WsLayout)]
+                   F.error_word.offset, C.sizeof(L.BwdParams), C.sizeof(L.WsLayout)]
 
 
 def good_params(**kw):
@@ -158,13 +158,15 @@ def test_check_maps_status_to_python_exceptions():
 
 def test_auto_variant_policy():
     """AUTO: generic when the MFMA kernels do not apply; resident for many heads of small problems
-    whose state fits in LDS; the fused kernel for 8 or 16 heads of ~4096 tokens in 64-row problems;
+    whose state fits in LDS; the fused kernel for 8 or 16 heads of ~4096 tokens in 64-row problems, but
+    only for callers that state that they own the device (MA_FLAG_DEVICE_EXCLUSIVE);
     per-stage launches where the one-launch kernels are at a disadvantage (uneven head counts of 128-row problems, wide heads with many blocks,
     very few long heads); the chained kernel otherwise."""
     lib = L.load()
 
-    def auto(E, H, N, D, B, dt=L.MA_F16, Dv=None, T=2):
+    def auto(E, H, N, D, B, dt=L.MA_F16, Dv=None, T=2, exclusive=False):
         p = L.FwdParams()
+        p.flags = L.MA_FLAG_DEVICE_EXCLUSIVE if exclusive else 0
         p.E, p.H, p.N, p.D, p.Dv, p.B, p.T = E, H, N, D, Dv or D, B, T
         p.dtype_qk = p.dtype_v = dt
         for name, w in (("q_stride", D), ("k_stride", D), ("v_stride", p.Dv), ("out_stride", p.Dv)):
@@ -172,12 +174,20 @@ def test_auto_variant_policy():
         p.eps = 1e-12
         return L.VARIANT_NAMES[lib.ma_fwd_select_variant(p)]
 
-    assert auto(1, 16, 4096, 64, 64) == "fused"         # 16 heads x 64 workgroups: every head has a full team at once
-    assert auto(1, 16, 4096, 64, 64, T=1) == "fused"
-    assert auto(2, 16, 4096, 64, 64) == "chained"
-    assert auto(1, 8, 8192, 64, 64) == "fused"          # with more than one step also 128 tasks per phase: 8 heads of 8192 tokens,
-    assert auto(1, 16, 4096, 64, 128) == "fused"        # 16 heads of 4096 in 128-row blocks (two positions per workgroup)
-    assert auto(1, 8, 8192, 72, 128) == "fused"         # 8 heads also with head dims up to 80
+    ex = dict(exclusive=True)
+    assert auto(1, 16, 4096, 64, 64, **ex) == "fused"         # 16 heads x 64 workgroups: every head has a full team at once
+    assert auto(1, 16, 4096, 64, 64, T=1, **ex) == "fused"
+    assert auto(2, 16, 4096, 64, 64, **ex) == "chained"
+    assert auto(1, 8, 8192, 64, 64, **ex) == "fused"          # with more than one step also 128 tasks per phase: 8 heads of 8192 tokens,
+    assert auto(1, 16, 4096, 64, 128, **ex) == "fused"        # 16 heads of 4096 in 128-row blocks (two positions per workgroup)
+    assert auto(1, 8, 8192, 72, 128, **ex) == "fused"         # 8 heads also with head dims up to 80
+    # the fused kernel's workgroups wait for each other: without the caller's word that the device is its
+    # own, AUTO stays with kernels that make progress beside any other work
+    for T_ in (1, 2, 3):
+        for shape in ((1, 16, 4096, 64, 64), (1, 8, 8192, 64, 64), (1, 16, 4096, 64, 128), (1, 8, 8192, 72, 128)):
+            assert auto(*shape, T=T_) in ("chained", "staged"), (shape, T_)
+    assert auto(1, 16, 4096, 64, 64) == "chained"
+    assert auto(1, 16, 4096, 64, 64, T=1) == "chained"
     assert auto(1, 16, 4096, 72, 64) == "chained"       # ... 16 heads not
     assert auto(1, 8, 6144, 64, 64) == "chained"        # 96 blocks: the team kernel would run them as 128
     assert auto(1, 8, 8192, 64, 64, T=1) == "staged"    # a single step: two launches

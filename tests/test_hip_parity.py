@@ -213,18 +213,29 @@ TEAM_SHAPES = [  # E, H, N, D, B, T, pre, dt, masked: 8 or 16 heads whose phases
 
 
 @pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", TEAM_SHAPES)
-def test_few_long_heads_run_in_the_team_kernel(E, H, N, D, B, T, pre, dt, masked):
-    """AUTO sends 8 or 16 heads of 64 .. 128 tasks per phase to the team kernel when T > 1 (teams larger than
-    the workgroups the device holds per head loop over their tasks): parity, and the bounded waits all met."""
+def test_few_long_heads_run_in_the_team_kernel(E, H, N, D, B, T, pre, dt, masked, monkeypatch):
+    """For a caller that owns the device (MA_FLAG_DEVICE_EXCLUSIVE; the module's DEVICE_EXCLUSIVE switch) AUTO
+    sends 8 or 16 heads of 64 .. 128 tasks per phase to the team kernel when T > 1 (teams larger than the
+    workgroups the device holds per head loop over their tasks): parity, and the bounded waits all met.
+    Without that statement the same call stays away from the team kernel and gives the same result to tolerance."""
+    from ma import ma_hip
     q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
     mask = block_safe_mask(E, N, B, seed=B) if masked else None
     ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
     dev = to_dev(q, k, v, mask)
     out = torch.empty_like(dev[2])
-    assert L.VARIANT_NAMES[L.load().ma_fwd_select_variant(make_params(*dev[:3], None, out, T, B, pre, "auto"))] == "fused"
+    p = make_params(*dev[:3], None, out, T, B, pre, "auto")
+    assert L.VARIANT_NAMES[L.load().ma_fwd_select_variant(p)] in ("chained", "staged")
+    p.flags = L.MA_FLAG_DEVICE_EXCLUSIVE
+    assert L.VARIANT_NAMES[L.load().ma_fwd_select_variant(p)] == "fused"
+    shared = monarch_attention_hip(*dev, T, B, pre, variant="auto")
+    monkeypatch.setattr(ma_hip, "DEVICE_EXCLUSIVE", True)
     got = monarch_attention_hip(*dev, T, B, pre, variant="auto")
+    fused = monarch_attention_hip(*dev, T, B, pre, variant="fused")
     torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.uint8), fused.view(torch.uint8)), "with DEVICE_EXCLUSIVE 'auto' must run the team kernel"
     assert_parity(got.cpu(), ref, dt, f"team shapes {(E, H, N, D, B, T, pre, dt, masked)}")
+    assert_parity(shared.cpu(), ref, dt, f"team shapes, shared device {(E, H, N, D, B, T, pre, dt, masked)}")
     assert sync_status() == 0
 
 
@@ -720,12 +731,14 @@ def test_wait_that_runs_out_is_loud_and_leaves_the_workspace_usable(variant, sha
     ws = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
     word = ws[4:8].view(torch.int32)
     p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
+    host_word = torch.zeros(1, dtype=torch.int32, pin_memory=True)   # ma_fwd_params.error_word: the same code, in host memory
+    p.error_word = host_word.data_ptr()
     stream = torch.cuda.current_stream().cuda_stream
 
     p.flags = L.MA_FLAG_SYNC_READY
     L.check(lib.ma_fwd(p, stream), "ma_fwd")
     torch.cuda.synchronize()
-    assert int(word.item()) == 0
+    assert int(word.item()) == 0 and int(host_word[0]) == 0
     assert_parity(out.cpu(), want, "f16", f"{variant} before")
 
     for rep in range(4):
@@ -735,21 +748,24 @@ def test_wait_that_runs_out_is_loud_and_leaves_the_workspace_usable(variant, sha
             L.check(lib.ma_fwd(p, stream), "ma_fwd")
         torch.cuda.synchronize()
         assert int(word.item()) == 1, "the wait that ran out was not reported"
+        assert int(host_word[0]) == 1, "the wait that ran out was not reported in the caller's host word"
         assert torch.isnan(out.float()).any(dim=-1).all(), "every output row depends on a wait that gave up: all must be NaN"
 
         word.zero_()
+        host_word.zero_()
         out.zero_()
         p.flags = L.MA_FLAG_SYNC_READY   # no clearing of the sync area: the failed call must have left it consistent
         for _ in range(2):
             L.check(lib.ma_fwd(p, stream), "ma_fwd")
         torch.cuda.synchronize()
-        assert int(word.item()) == 0
+        assert int(word.item()) == 0 and int(host_word[0]) == 0
         assert_parity(out.cpu(), want, "f16", f"{variant} after failed call {rep}")
 
 
 def test_module_reports_a_failed_call_at_a_later_call(monkeypatch):
-    """The Python operator never synchronises to look at the error word: a failed call is reported
-    by a RuntimeError from a later call on the same stream, after which calls are normal again."""
+    """The Python operator never synchronises to look at the error word: the kernel stores it into
+    pinned host memory as well, every call looks there first, and so a failed call is reported by a
+    RuntimeError from the next call made after its work is complete; calls are normal again after that."""
     from ma import ma_hip
     E, H, N, D, B, T = 1, 2, 1024, 64, 32, 2
     q, k, v = to_dev(*seeded_qkv(E, H, N, D, torch.float16, seed=4))
@@ -763,9 +779,7 @@ def test_module_reports_a_failed_call_at_a_later_call(monkeypatch):
     torch.cuda.synchronize()
     assert torch.isnan(bad.float()).any()
     with pytest.raises(RuntimeError, match="earlier forward call"):
-        for _ in range(3):    # the look at the error word is queued behind a call and read by a later one
-            monarch_attention_hip(q, k, v, None, T, B, False, variant="fused")
-            torch.cuda.synchronize()
+        monarch_attention_hip(q, k, v, None, T, B, False, variant="fused")   # the very next call
     again = monarch_attention_hip(q, k, v, None, T, B, False, variant="fused")
     torch.cuda.synchronize()
     assert_parity(good.cpu(), want, "f16", "before the failure")

@@ -5,7 +5,10 @@ caller-provided workspace, through the C ABI.
 Both run the same kernels on the same inputs, so the gate is the strictest one:
 bit-identical outputs (and, as a cross-check of the test itself, parity with the
 CPU oracle at the usual tolerance).  Two calls in a row share the array, the
-second on a smaller problem; problems beyond the array's size are refused.
+second on a smaller problem; problems beyond the array's size are refused; the
+calls change neither the device's free memory nor PyTorch's allocator
+statistics; and a call that would overlap with one on another stream is turned
+away (MA_ERR_BUSY).
 """
 import pytest
 import torch
@@ -76,3 +79,59 @@ def test_static_refuses_what_does_not_fit():
     torch.cuda.synchronize()
     assert torch.isnan(out).all()   # nothing was launched
     assert "MA_STATIC_WORKSPACE_BYTES" in L.strerror(L.MA_ERR_STATIC_LIMIT)
+
+
+def test_static_allocates_and_frees_nothing():
+    """After a warm-up call (code objects, the array's address, the guard's event) a ma_fwd_static
+    call leaves the device's free memory (hipMemGetInfo) and PyTorch's allocator statistics as they
+    were - for a one-launch variant, whose sync area is cleared by a fill kernel, and for the
+    per-stage launches."""
+    lib = L.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    for (E, H, N, D, B, T, dt, variant) in [(1, 16, 4096, 64, 64, 2, "f16", "chained"), (1, 16, 4096, 64, 64, 1, "f16", "fused"),
+                                            (2, 3, 512, 64, 32, 3, "bf16", "staged"), (1, 2, 300, 48, 16, 2, "f32", "auto")]:
+        q, k, v = (t.to(DEV) for t in seeded_qkv(E, H, N, D, DT[dt], seed=1))
+        out = torch.empty_like(v)
+        p = make_params(q, k, v, None, out, T, B, False, variant)
+        L.check(lib.ma_fwd_static(p, stream), "warm-up")
+        torch.cuda.synchronize()
+        free0, total0 = torch.cuda.mem_get_info()
+        stats0 = {k_: v_ for k_, v_ in torch.cuda.memory_stats().items() if k_.endswith(".current") or k_.endswith(".allocated") or k_.endswith(".freed")}
+        for _ in range(3):
+            L.check(lib.ma_fwd_static(p, stream), "ma_fwd_static")
+        torch.cuda.synchronize()
+        free1, total1 = torch.cuda.mem_get_info()
+        stats1 = {k_: v_ for k_, v_ in torch.cuda.memory_stats().items() if k_ in stats0}
+        assert (free1, total1) == (free0, total0), f"{variant}: free device memory changed by {free0 - free1} bytes"
+        assert stats1 == stats0, f"{variant}: PyTorch allocator statistics changed"
+
+
+def test_static_turns_away_a_call_that_would_overlap():
+    """All calls on a GPU share one array.  A call on another stream than the previous call's, made
+    while that call's work is still queued or running, returns MA_ERR_BUSY and launches nothing;
+    calls on one stream are ordered and always accepted; once the earlier work is complete the
+    other stream's call is accepted too."""
+    lib = L.load()
+    E, H, N, D, B, T = 1, 4, 1000, 64, 32, 2
+    q, k, v = (t.to(DEV) for t in seeded_qkv(E, H, N, D, torch.float16, seed=11))
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    out1, out1b, out2 = (torch.full(v.shape, float("nan"), dtype=v.dtype, device=DEV) for _ in range(3))
+    p1, p1b, p2 = (make_params(q, k, v, None, o, T, B, False, "auto") for o in (out1, out1b, out2))
+    L.check(lib.ma_fwd_static(p1, s1.cuda_stream), "warm-up")
+    torch.cuda.synchronize()
+    out1.fill_(float("nan"))
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        torch.cuda._sleep(400_000_000)    # keeps s1 busy for a good tenth of a second: what follows on s1 stays queued
+    assert lib.ma_fwd_static(p1, s1.cuda_stream) == L.MA_OK
+    assert lib.ma_fwd_static(p2, s2.cuda_stream) == L.MA_ERR_BUSY      # would run while s1's call is pending
+    assert lib.ma_fwd_static(p1b, s1.cuda_stream) == L.MA_OK           # ordered behind it: fine
+    assert "another stream" in L.strerror(L.MA_ERR_BUSY)
+    torch.cuda.synchronize()
+    assert torch.isnan(out2).all()                                      # the refused call launched nothing
+    assert lib.ma_fwd_static(p2, s2.cuda_stream) == L.MA_OK            # s1's work is complete now
+    torch.cuda.synchronize()
+    want = monarch_attention_oracle(q.cpu(), k.cpu(), v.cpu(), None, T, B, False)
+    assert_parity(out1.cpu(), want, "f16", "static call on the first stream")
+    for o in (out1b, out2):
+        assert torch.equal(o.view(torch.uint8), out1.view(torch.uint8))
