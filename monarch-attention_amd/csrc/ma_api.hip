@@ -172,6 +172,7 @@ bool mfma32_supported(const ma_fwd_params* p) {
 }
 
 int run_resident(const Problem& P, int dtype_qk, bool dry_run, hipStream_t s) {
+    if (dtype_qk == MA_F32) return launch_head32(P, dry_run, s);
     const bool h = dtype_qk == MA_F16;
     const int D = P.D;
     if (D <= 32) return h ? launch_resident_f16_d2(P, dry_run, s) : launch_resident_bf16_d2(P, dry_run, s);
@@ -291,9 +292,19 @@ int select_variant(const ma_fwd_params* p) {
         case MA_VARIANT_STAGED: return fast || fast32 ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_FUSED: return fast && one_launch_tiles(p) ? MA_VARIANT_FUSED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_CHAINED: return fast && chain_fits(p) ? MA_VARIANT_CHAINED : MA_ERR_UNSUPPORTED;
-        case MA_VARIANT_RESIDENT: return fast && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
+        case MA_VARIANT_RESIDENT: return (fast || fast32) && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
         default:
-            if (fast32) return MA_VARIANT_STAGED;
+            // fp32: heads of up to 16 blocks of up to 16 rows can run whole in one workgroup each (one launch, no
+            // state in memory).  A head then has one compute unit to itself, which pays from 64 heads on
+            // (256 tokens x 64: 0.93 of the stage launches' time at 96 heads, 0.5 - 0.7 from 192 on, also
+            // beyond one pass over the compute units) and for any head count when the head is small
+            // (128 tokens x 32: 0.45 - 0.8); few large heads are faster spread over many compute units
+            // by the stage launches (one head of 256 x 64: 8 us against 13).
+            if (fast32) {
+                const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+                const bool pays = heads >= 64 || M * p->B * p->D <= 4096;
+                return pays && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_VARIANT_STAGED;
+            }
             if (!fast) return MA_VARIANT_GENERIC;
             {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;

@@ -182,6 +182,9 @@ int launch_resident_bf16_d4(const Problem& P, bool dry_run, hipStream_t s);
 int launch_resident_bf16_d5(const Problem& P, bool dry_run, hipStream_t s);
 int launch_resident_bf16_d8(const Problem& P, bool dry_run, hipStream_t s);
 
+// fp32 heads of at most 16 blocks of at most 16 rows, head dim up to 64: one launch, state in LDS.
+int launch_head32(const Problem& P, bool dry_run, hipStream_t s);
+
 // Chained forward (one launch, one workgroup per block problem, flags between phases).
 int launch_chain_f16_d2(const Problem& P, bool sync_ready, hipStream_t s);
 int launch_chain_f16_d4(const Problem& P, bool sync_ready, hipStream_t s);

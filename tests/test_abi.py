@@ -143,7 +143,7 @@ def test_select_variant_reports_a_known_variant():
     v = lib.ma_fwd_select_variant(good_params())
     assert v in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["chained"], L.VARIANTS["resident"], L.VARIANTS["fused"])
     p32 = good_params(dtype_qk=L.MA_F32, dtype_v=L.MA_F32)
-    assert lib.ma_fwd_select_variant(p32) in (L.VARIANTS["generic"], L.VARIANTS["staged"])
+    assert lib.ma_fwd_select_variant(p32) in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["resident"])
 
 
 def test_check_maps_status_to_python_exceptions():
@@ -222,6 +222,12 @@ def test_auto_variant_policy():
     assert auto(1, 1, 16, 64, 4) == "chained"
     assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "staged"       # fp32 MFMA stage kernels
     assert auto(1, 2, 7600, 48, 128, dt=L.MA_F32) == "staged"
+    assert auto(1, 1, 256, 64, 16, dt=L.MA_F32, T=1) == "staged"    # one small fp32 head: spread over compute units by the stage launches
+    assert auto(8, 8, 197, 64, 16, dt=L.MA_F32) == "resident"       # from 64 heads on: one workgroup per head, one launch
+    assert auto(64, 12, 197, 64, 16, dt=L.MA_F32) == "resident"
+    assert auto(1, 2, 128, 32, 16, dt=L.MA_F32) == "resident"       # ... and for very small heads always
+    assert auto(8, 8, 272, 64, 16, dt=L.MA_F32) == "staged"         # 17 blocks
+    assert auto(8, 8, 256, 80, 16, dt=L.MA_F32) == "staged"         # head dim above 64
     assert auto(1, 16, 16384, 128, 128, dt=L.MA_F32) == "generic"   # 128 x 128 fp32 tiles do not fit the LDS
     assert auto(1, 16, 4096, 62, 64, dt=L.MA_F32) == "generic"      # D % 4 != 0
     assert auto(1, 16, 4096, 64, 64, Dv=128) == "generic"

@@ -262,6 +262,40 @@ def test_resident_kernel_with_one_state_tile(E, H, N, D, B, T, pre, dt, masked):
     assert torch.equal(out, again)
 
 
+SMALL_F32 = [  # E, H, N, D, B, T, pre, masked: fp32 heads of at most 16 blocks of at most 16 rows
+    (1, 1, 256, 64, 16, 1, False, False),      # the reference's CPU-sized case
+    (1, 1, 256, 64, 16, 3, True, True), (2, 3, 197, 64, 16, 2, True, True), (1, 4, 100, 32, 8, 3, False, True),
+    (3, 2, 250, 48, 16, 2, True, False), (2, 2, 37, 20, 5, 2, False, True), (1, 2, 16, 64, 16, 2, False, False),
+    (1, 3, 49, 64, 7, 1, True, True), (1, 2, 33, 4, 3, 2, False, False), (40, 8, 197, 64, 16, 2, False, True),   # 320 heads: workgroups walk several
+]
+
+
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,masked", SMALL_F32)
+def test_small_fp32_heads_in_one_launch(E, H, N, D, B, T, pre, masked):
+    """fp32 heads of up to 256 tokens run whole in one workgroup each (variant 'resident', what 'auto' picks from
+    64 heads on and for very small heads): parity with the oracle at the fp32 gate, and - the arithmetic being
+    that of the fp32 stage kernels, operation for operation - bit-identical to the per-stage launches."""
+    q, k, v = seeded_qkv(E, H, N, D, torch.float32, seed=N + B)
+    mask = block_safe_mask(E, N, B, seed=B) if masked else None
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre)
+    dev = to_dev(q, k, v, mask)
+    out = monarch_attention_hip(*dev, T, B, pre, variant="resident")   # the variant must take these shapes
+    staged = monarch_attention_hip(*dev, T, B, pre, variant="staged")
+    auto = monarch_attention_hip(*dev, T, B, pre, variant="auto")
+    torch.cuda.synchronize()
+    assert_parity(out.cpu(), ref, "f32", f"fp32 head kernel {(E, H, N, D, B, T, pre, masked)}")
+    assert torch.equal(out.view(torch.int32), staged.view(torch.int32)), "differs from the per-stage fp32 kernels"
+    assert torch.equal(out.view(torch.int32), auto.view(torch.int32))
+    p = make_params(*dev[:3], None, torch.empty_like(dev[2]), T, B, pre, "auto")
+    M = -(-N // B)
+    assert L.VARIANT_NAMES[L.load().ma_fwd_select_variant(p)] == ("resident" if E * H >= 64 or M * B * D <= 4096 else "staged")
+    for shape, why in (((1, 2, 272, 64, 16), "17 blocks"), ((1, 2, 64, 64, 32), "32-row blocks"), ((1, 2, 64, 80, 16), "head dim 80")):
+        e, h, n, d, b = shape
+        x = torch.zeros(e, h, n, d, device=DEV)
+        with pytest.raises(NotImplementedError):
+            monarch_attention_hip(x, x, x, None, 1, b, False, variant="resident")
+
+
 def test_broadcast_over_tokens_is_accepted():
     """expand()-ed inputs (stride 0 along N) are legal for the reference (it pads, i.e. copies); the
     operator takes them too, by making the one copy the library's row-overlap check asks for."""
