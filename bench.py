@@ -166,9 +166,12 @@ def main():
                          "N = 256 .. 8192, blocks of 16 .. 128 rows (T from --T, default 2; head dim from --head-dim); prints the rows "
                          "and how far AUTO's choice is from the fastest variant")
     ap.add_argument("--head-dim", type=int, default=64, help="head dim of --sweep-variants")
-    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96", "fewheads"],
+    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96", "fewheads", "ragged"],
                     help="shapes of --sweep-variants: power-of-two lengths and blocks, blocks / block counts in the 96-row tile class, "
-                         "or few heads of thousands of tokens")
+                         "few heads of thousands of tokens, or lengths that are no multiple of the block (197, 500, 1000, 3000, 5000, 7600)")
+    ap.add_argument("--sweep-dtype", default="f16", choices=["f16", "bf16", "f32"], help="operand dtype of --sweep-variants")
+    ap.add_argument("--sweep-mask", action="store_true", help="--sweep-variants with a key / query mask (int64, ~10 %% of the tokens masked out in whole runs)")
+    ap.add_argument("--sweep-pre-pad", action="store_true", help="--sweep-variants with the padding at the front")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="fold two rocprofv3 --pmc counter_collection.csv files into profiles/traffic.json (no GPU needed)")
     ap.add_argument("--matrix", action="store_true",
@@ -286,11 +289,18 @@ def main():
     # ------------------------------------------------------------------ every variant over a grid of shapes
     if args.sweep_variants:
         T_, D = args.T or 2, args.head_dim
-        names = ("staged", "chained", "fused", "resident")
+        # without the statement that the benchmark owns the device AUTO may not choose the team kernel: it is
+        # then judged against the variants it may choose
+        names = ("staged", "chained", "resident") if args.shared_device else ("staged", "chained", "fused", "resident")
+        sdt = DT[args.sweep_dtype]
+        selt = torch.empty((), dtype=sdt).element_size()
         rows, logsum, worst = [], 0.0, None
         if args.sweep_grid == "pow2":
             grid = [(h, N, B) for h in (1, 2, 4, 6, 8, 12, 16, 32, 64, 128, 192, 384) for N in (256, 512, 1024, 2048, 4096, 8192)
                     for B in (16, 32, 64, 128)]
+        elif args.sweep_grid == "ragged":     # lengths of the reference's models: ViT 197, BART / RoBERTa prefixes, GPS graphs
+            grid = [(h, N, B) for h in (2, 8, 12, 16, 48, 96, 192, 768) for (N, B) in ((197, 14), (197, 16), (500, 24), (1000, 32), (1000, 48),
+                                                                                  (3000, 55), (3000, 64), (5000, 71), (5000, 128), (7600, 88), (7600, 128))]
         elif args.sweep_grid == "fewheads":   # 8, 16, 24 heads of thousands of tokens: where the team kernel competes
             grid = [(h, N, B) for h in (8, 16, 24) for N in (2048, 4096, 5000, 6144, 8000, 8192) for B in (32, 64, 128)]
         else:   # blocks and / or block counts of 65 .. 96 rows (and two 128-row shapes with ragged block counts)
@@ -299,20 +309,24 @@ def main():
                                    (7000, 128), (12000, 128), (768, 96))]
         for (heads, N, B) in grid:
             M = -(-N // B)
-            set_bytes = 4 * heads * N * D * 2
+            set_bytes = 4 * heads * N * D * selt
             if M > 128 or M < 2 or set_bytes > (1.2e9 if args.sweep_grid == "pow2" else 0.6e9):
                 continue
             E, H = (heads // 4, 4) if heads % 4 == 0 else (1, heads)
             gen = torch.Generator().manual_seed(0)
             nbuf = max(2, min(8, -(-400 * 2 ** 20 // set_bytes)))
-            base = [torch.randn(E, H, N, D, generator=gen).to(torch.float16) for _ in range(3)]
+            base = [torch.randn(E, H, N, D, generator=gen).to(sdt) for _ in range(3)]
             sets = []
             for i in range(nbuf):
                 q, k, v = (t.to(dev).roll(i, dims=2).contiguous() for t in base)
                 sets.append((q, k, v, torch.empty_like(q)))
+            mask = None
+            if args.sweep_mask:   # a tokenizer-style int64 mask: the tail of every sequence masked out, at most 10 % of it
+                keep = N - (torch.arange(E) * 7 % max(N // 10, 1))
+                mask = (torch.arange(N)[None, :] < keep[:, None]).to(torch.int64).to(dev)
             row = {"heads": heads, "N": N, "block": B}
             for variant in ("auto",) + names:
-                ps = [make_params(q, k, v, None, o, T_, B, False, variant) for (q, k, v, o) in sets]
+                ps = [make_params(q, k, v, mask, o, T_, B, args.sweep_pre_pad, variant) for (q, k, v, o) in sets]
                 sel = lib.ma_fwd_select_variant(ps[0])
                 if variant == "auto":
                     row["auto"] = L.VARIANT_NAMES[sel]
@@ -327,6 +341,8 @@ def main():
                     continue   # e.g. a team grid that does not fit the device
                 row[variant] = round(batch_stats(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), 100)["median_ms"] * 1e3, 2)
                 del ws
+            if row["auto"] not in row:   # AUTO went to a variant outside the list (the FMA kernels): nothing to judge it against
+                continue
             best = min(names, key=lambda v: row.get(v, float("inf")))
             row["best"] = best
             row["auto_over_best"] = round(row[row["auto"]] / row[best], 3)
@@ -336,8 +352,9 @@ def main():
             rows.append(row)
             del sets
             torch.cuda.empty_cache()
-        print(json.dumps({"metric": "AUTO's choice against the fastest variant", "unit": "us (median)", "n_gpus": 1, "dtype": "f16",
+        print(json.dumps({"metric": "AUTO's choice against the fastest variant", "unit": "us (median)", "n_gpus": 1, "dtype": args.sweep_dtype,
                           "data": "synthetic", "T": T_, "D": D, "grid": args.sweep_grid, "points": len(rows),
+                          "mask": bool(args.sweep_mask), "pre_pad": bool(args.sweep_pre_pad), "device_exclusive": not args.shared_device,
                           "geomean_auto_over_best": round(math.exp(logsum / max(len(rows), 1)), 4), "worst": worst, "rows": rows}))
         return
 

@@ -192,6 +192,16 @@ bool resident_fits(const ma_fwd_params* p, bool one_tile) {
     return run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
 }
 
+// Does the head - Q, K, V and the state - fit in LDS whole (the fastest form of the resident kernel)?
+bool resident_head_fits(const ma_fwd_params* p) {
+    Problem P;
+    std::memset(&P, 0, sizeof(P));
+    P.E = p->E; P.H = p->H; P.N = p->N; P.D = p->D; P.Dv = p->Dv; P.B = p->B; P.T = p->T;
+    P.M = (p->N + p->B - 1) / p->B;
+    P.resident_head_only = 1;
+    return p->dtype_qk != MA_F32 && run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
+}
+
 // The fused, chained and resident kernels are built for block problems of at most 128 rows.
 bool one_launch_tiles(const ma_fwd_params* p) {
     const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
@@ -248,8 +258,10 @@ bool fused_full_width(const ma_fwd_params* p) {
 // rows, T = 1, 2, 3, head dims 32, 64, 128; every variant that takes a shape timed: the choice
 // below is within 0.0 - 0.7 % of the fastest variant in the geometric mean of each sweep and 18 %
 // at worst):
-//  * the resident kernel for many heads of small problems: with two or three state tiles (heads
-//    of up to ~256 tokens) for blocks of at most 16 rows from 128 heads on; in its one-tile form
+//  * the resident kernel for heads that fit in LDS with their inputs (up to ~256 tokens at d = 64) in
+//    blocks of at most 32 rows: from 128 heads on, and with more than one step for any number of
+//    heads in 16-row blocks; with two or three state tiles for blocks of at most 16 rows from 128
+//    heads on; in its one-tile form
 //    (up to ~512 tokens) for problems of one or two strips when the head count fills the
 //    device's 256 one-per-CU workgroups to three quarters or more in its last pass (192 heads:
 //    0.95 of the chained kernel's time with 0.6 of its traffic, 768: 0.84; 128 or 384 heads:
@@ -308,14 +320,35 @@ int select_variant(const ma_fwd_params* p) {
             if (!fast) return MA_VARIANT_GENERIC;
             {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
+                // heads that fit in LDS whole, in blocks and block counts of at most two strips (16 waves): every
+                // input is read once and no state leaves the compute unit.  From 128 heads on (0.63 - 0.93 of
+                // the next best variant's time at T = 1, 2), and with more than one step also for any number of
+                // heads in 16-row blocks (0.85 - 0.95 at 256 tokens, 0.55 - 0.8 for shorter heads and three steps; a
+                // single step of few heads: 1.03 - 1.23, they stay away).  Head dims up to 64: in the 128-column class
+                // the kernel holds heads of ~128 tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
+                if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= 128 || (p->T >= 2 && p->B <= 16)) && resident_head_fits(p))
+                    return MA_VARIANT_RESIDENT;
                 if (p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= 128 && resident_fits(p, false))
                     return MA_VARIANT_RESIDENT;
                 if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D <= 64 &&
                     ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))
                     return MA_VARIANT_RESIDENT;
                 if (device_exclusive(p) && fused_full_width(p)) return MA_VARIANT_FUSED;
+                // Head dims of 65 .. 80 (the 80-column tile class; measured at 72) with 128-row problems - blocks or
+                // block counts of 97 .. 128 - and more than one step: the team kernel is 8 - 21 % ahead of the chained
+                // kernel for 6 .. 128 heads of thousands of tokens (from 2048 tokens on with 32 heads and more, 4096
+                // below that), the stage launches 4 - 15 % for 192 heads and more in 128-row blocks.
+                {
+                    const bool wide5 = p->D > 64 && p->D <= 80, class128 = (M > 96 || p->B > 96) && one_launch_tiles(p);
+                    if (wide5 && class128 && p->T >= 2) {
+                        if (device_exclusive(p) && heads >= 6 && heads <= 128 && p->N >= (heads >= 32 ? 2048 : 4096)) return MA_VARIANT_FUSED;
+                        if (heads >= 192 && p->B > 96 && M >= 4) return MA_VARIANT_STAGED;
+                    }
+                }
                 const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
-                const bool wide_dim = p->D > 80 && M > 64 && p->B >= 64;
+                // head dims above 80 (the 128-column class; measured at 96 and 128): many blocks of 64 rows and
+                // more, or 128-row problems on many tokens in total (4 - 16 % behind the stage launches there)
+                const bool wide_dim = p->D > 80 && ((M > 64 && p->B >= 64) || ((p->B > 96 || M > 96) && heads * p->N >= 393216));
                 const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
                 const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 7168));
                 // launches that leave most of the device empty: the stage kernels run their 6- and 8-strip R and Z

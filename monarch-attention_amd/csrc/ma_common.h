@@ -39,6 +39,8 @@ struct Problem {
     // The resident kernel may keep aL and aR in ONE LDS tile and pass Y through the workspace where two or
     // three tiles do not fit (heads of up to ~512 tokens at d = 64).
     int one_tile_ok;
+    // Query only: does the form of the resident kernel that keeps Q, K and V in LDS as well take this head?
+    int resident_head_only;
     int test_no_spin;    // waits between workgroups give up at once (failure-path tests)
     // Copy of the error word in host memory the device can write (or null): a workgroup that raises the
     // word in the sync area stores the code here as well, where the host reads it without a copy.

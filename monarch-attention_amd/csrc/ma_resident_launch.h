@@ -88,7 +88,7 @@ template <class T, int DT, int NTB, int NTM>
 int launch_resident_one(const Problem& P, bool dry_run, hipStream_t s) {
     {   // everything in LDS where the head is short enough for that
         const int err = launch_resident_head<T, DT, NTB, NTM>(P, dry_run, s);
-        if (err != MA_ERR_UNSUPPORTED) return err;
+        if (err != MA_ERR_UNSUPPORTED || P.resident_head_only) return err;
     }
     if constexpr (NTB <= 2 && NTM <= 2) {
         const int err = launch_resident_w<T, DT, NTB, NTM, kResidentWavesWide>(P, dry_run, s);

@@ -210,7 +210,11 @@ def test_auto_variant_policy():
     assert auto(32, 12, 512, 64, 32) == "chained"      # (384 heads: 1.5 passes over 256 CUs)
     assert auto(16, 12, 512, 64, 64) == "chained"      # ... and for problems of one or two strips
     assert auto(32, 12, 256, 64, 64) == "chained"      # 64-row blocks never run resident
-    assert auto(16, 12, 256, 64, 32) == "chained"      # nor do 32-row blocks in 8 blocks (the chained kernel packs them)
+    assert auto(16, 12, 256, 64, 32) == "resident"     # 256-token heads fit in LDS with their inputs: from 128 heads on
+    assert auto(2, 16, 256, 64, 32) == "chained"       # ... fewer heads of 32-row blocks stay with the chained kernel
+    assert auto(1, 2, 256, 64, 16) == "resident"       # ... those of 16-row blocks do not when there is more than one step
+    assert auto(1, 2, 256, 64, 16, T=1) == "chained"
+    assert auto(16, 12, 197, 64, 16, T=1) == "resident"
     assert auto(8, 16, 1024, 72, 32) == "chained"
     assert auto(4, 16, 16384, 64, 128) == "chained"
     assert auto(512, 16, 1024, 64, 32) == "staged"      # more heads than the chained kernel has flag words for
@@ -218,8 +222,10 @@ def test_auto_variant_policy():
     assert auto(2, 16, 8192, 128, 64) == "staged"       # ... but not for wide heads
     assert auto(2, 16, 5000, 64, 64) == "chained"       # 79 blocks: the 96-row class
     assert auto(1, 2, 8192, 64, 64) == "staged"         # two long heads would run on two of the eight XCDs
-    assert auto(2, 2, 197, 64, 16) == "chained"         # few short heads: one launch
-    assert auto(1, 1, 16, 64, 4) == "chained"
+    assert auto(2, 2, 197, 64, 16) == "resident"        # few short heads in 16-row blocks, two steps: whole in LDS
+    assert auto(2, 2, 197, 64, 16, T=1) == "chained"    # ... a single step: one launch of the chained kernel
+    assert auto(1, 1, 16, 64, 4) == "resident"
+    assert auto(1, 1, 16, 64, 4, T=1) == "chained"
     assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "staged"       # fp32 MFMA stage kernels
     assert auto(1, 2, 7600, 48, 128, dt=L.MA_F32) == "staged"
     assert auto(1, 1, 256, 64, 16, dt=L.MA_F32, T=1) == "staged"    # one small fp32 head: spread over compute units by the stage launches

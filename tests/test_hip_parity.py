@@ -116,8 +116,8 @@ CONFIGS = [  # name, E, H, N, D, B, T, pre, dt, scale
     ("b48_m40", 2, 4, 1900, 64, 48, 2, False, "f16", 1.0),         # 3-strip problems in both kinds of phases
     ("b96_m90", 1, 2, 8600, 64, 96, 2, True, "bf16", 1.0),         # 6-strip problems (per-stage launches; 8-strip class in one launch)
     ("b40_m6_d72", 2, 3, 230, 72, 40, 3, False, "f16", 1.0),       # 3 strips of keys, one of blocks, head dim 72
-    ("big_block", 1, 2, 600, 64, 200, 2, False, "f16", 1.0),       # B > 128: beyond the MFMA tiles, AUTO -> generic
-    ("many_blocks", 1, 2, 4096, 32, 16, 2, False, "bf16", 1.0),    # M = 256 > 128: AUTO -> generic
+    ("big_block", 1, 2, 600, 64, 200, 2, False, "f16", 1.0),       # B > 128: the 16-strip class of the stage kernels (AUTO -> staged)
+    ("many_blocks", 1, 2, 4096, 32, 16, 2, False, "bf16", 1.0),    # M = 256 > 128: likewise, 16 strips of blocks
     ("one_block", 2, 2, 100, 64, 128, 3, True, "f16", 1.0),        # M = 1: dense softmax attention
     ("unit_blocks", 1, 2, 96, 32, 1, 1, False, "f16", 1.0),        # B = 1, M = N
     ("many_heads", 40, 64, 64, 32, 16, 2, False, "f16", 1.0),      # more heads than co-resident workgroups
