@@ -67,7 +67,7 @@ MFMA_PEAK_TFLOPS_F32 = 157.3   # dense fp32
 FETCH_SIZE_FACTOR = 2.00       # FETCH_SIZE under-reports a plain copy of known size by this factor (profiles/traffic_forward_kernels.md)
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
 KERNEL_DIR = os.path.join(ROOT, "monarch-attention_amd", "csrc")
-ONE_LAUNCH = {"fused": "fused_fwd_mfma", "resident": "resident_fwd_mfma", "chained": "chain_fwd_mfma"}
+ONE_LAUNCH = ("fused", "resident", "chained")   # variants that are one kernel launch per forward (its name: ma_fwd_kernel_name)
 
 
 def kernel_source_hash() -> str:
@@ -100,7 +100,8 @@ def record_traffic(args) -> None:
     every forward kernel times the kernels one forward launches."""
     fetch_csv, write_csv = args.record_traffic
 
-    names = ("r_step_mfma", "l_step_mfma", "z_step_mfma", "fused_fwd_mfma", "chain_fwd_mfma", "resident_fwd_mfma")
+    names = ("r_step_mfma", "l_step_mfma", "z_step_mfma", "fused_fwd_mfma", "chain_fwd_mfma", "resident_fwd_mfma", "resident_head_mfma",
+             "r_step_f32", "l_step_f32", "z_step_f32", "head_fwd_f32")
 
     def per_kernel(path, counter):
         acc = {}
@@ -118,7 +119,8 @@ def record_traffic(args) -> None:
     T = args.T or T
     # launches of each kernel in one forward (the bench also launches single stages for the per-stage timings:
     # the per-dispatch means make that irrelevant)
-    per_fwd = {"r_step_mfma": T, "l_step_mfma": T - 1, "z_step_mfma": 1, "fused_fwd_mfma": 1, "chain_fwd_mfma": 1, "resident_fwd_mfma": 1}
+    per_fwd = {"r_step_mfma": T, "l_step_mfma": T - 1, "z_step_mfma": 1, "fused_fwd_mfma": 1, "chain_fwd_mfma": 1, "resident_fwd_mfma": 1,
+               "resident_head_mfma": 1, "r_step_f32": T, "l_step_f32": T - 1, "z_step_f32": 1, "head_fwd_f32": 1}
     kernels, total = {}, 0.0
     for name in sorted(set(fetch) & set(write)):
         rd, wr = fetch[name][0] * 1024 * FETCH_SIZE_FACTOR, write[name][0] * 1024
@@ -461,7 +463,7 @@ def main():
         res = resolve(T_, variant)
         stages = {}
         if res in ONE_LAUNCH:
-            kernels = {ONE_LAUNCH[res]: (event_avg(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), n), 1)}
+            kernels = {lib.ma_fwd_kernel_name(ps[0]).decode(): (event_avg(lambda i: checked(lib.ma_fwd(ps[i % nbuf], sp)), n), 1)}
         else:
             # per-stage kernels on the state a full forward left in the workspace; (average ms, launches per forward)
             kernels = {"r_step(with V)": (event_avg(lambda i: checked(lib.ma_r_step(ps[i % nbuf], int(T_ == 1), 1, sp)), n), 1),

@@ -189,6 +189,11 @@ int ma_workspace_init(const ma_fwd_params* p, void* stream);
  * a negative ma_status. */
 int ma_fwd_select_variant(const ma_fwd_params* p);
 
+/* Name of the kernel that does the bulk of the work for this problem under the variant it resolves to
+ * (for the per-stage variants: the R-step kernel), as it appears in a profiler's kernel list; NULL for an
+ * invalid problem.  Introspection for benchmarks and profiles; no counterpart in the reference. */
+const char* ma_fwd_kernel_name(const ma_fwd_params* p);
+
 /* Whole forward pass: replaces monarch_attention_torch (ma/ma_torch.py:65-108).
  * `stream` is a hipStream_t (NULL = the default stream). */
 int ma_fwd(const ma_fwd_params* p, void* stream);

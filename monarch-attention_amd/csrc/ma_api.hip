@@ -250,6 +250,7 @@ bool fused_full_width(const ma_fwd_params* p) {
     const long long tR = phase_tasks(M, p->B), tL = phase_tasks(p->B, M);
     const long long widest = tR > tL ? tR : tL;
     if (!steps && heads * widest != 1024) return false;   // a single step: only with every workgroup slot of the device taken
+    if (!steps && (tR < 60 || tL < 60)) return false;     // ... in both phases (16 heads of 3000 tokens: 47 R tasks, 12 % behind the chained kernel)
     return heads < 32 && heads % 8 == 0 && widest >= 64 && heads * widest <= 1024;
 }
 
@@ -326,11 +327,11 @@ int select_variant(const ma_fwd_params* p) {
                 // heads in 16-row blocks (0.85 - 0.95 at 256 tokens, 0.55 - 0.8 for shorter heads and three steps; a
                 // single step of few heads: 1.03 - 1.23, they stay away).  Head dims up to 64: in the 128-column class
                 // the kernel holds heads of ~128 tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
-                if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= 128 || (p->T >= 2 && p->B <= 16)) && resident_head_fits(p))
+                if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= (p->T >= 2 ? 128 : 96) || (p->T >= 2 && p->B <= 16)) && resident_head_fits(p))
                     return MA_VARIANT_RESIDENT;
                 if (p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= 128 && resident_fits(p, false))
                     return MA_VARIANT_RESIDENT;
-                if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D <= 64 &&
+                if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D > 48 && p->D <= 64 &&   // (D = 48: 1.12 - 1.19 of the chained kernel's time)
                     ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))
                     return MA_VARIANT_RESIDENT;
                 if (device_exclusive(p) && fused_full_width(p)) return MA_VARIANT_FUSED;
@@ -346,6 +347,10 @@ int select_variant(const ma_fwd_params* p) {
                     }
                 }
                 const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
+                // 128-row blocks in 33 .. 48 blocks (three-strip L / Z problems beside eight-strip R problems) on a head
+                // count that does not divide by 8, or on very many heads: 12 / 192 heads of 5000 tokens are 7 - 21 %
+                // behind the stage launches in the chained kernel (16 .. 96 heads: 9 - 23 % ahead)
+                const bool odd_mix = p->B > 96 && M > 32 && M <= 48 && (heads % 8 != 0 || heads >= 192);
                 // head dims above 80 (the 128-column class; measured at 96 and 128): many blocks of 64 rows and
                 // more, or 128-row problems on many tokens in total (4 - 16 % behind the stage launches there)
                 const bool wide_dim = p->D > 80 && ((M > 64 && p->B >= 64) || ((p->B > 96 || M > 96) && heads * p->N >= 393216));
@@ -359,7 +364,7 @@ int select_variant(const ma_fwd_params* p) {
                     (rows_halve && (p->T == 1 ? (r_problems <= 160 || (heads <= 8 && r_problems <= 512))
                                               : p->B > 96 && (r_problems <= 48 || (heads <= 4 && p->N <= 4096)))) ||
                     (blocks_halve && p->T == 1 && heads * p->B <= 128);
-                if (!uneven_128 && !wide_dim && !few_heads && !one_step && !underfilled && chain_fits(p))
+                if (!uneven_128 && !odd_mix && !wide_dim && !few_heads && !one_step && !underfilled && chain_fits(p))
                     return MA_VARIANT_CHAINED;
             }
             return MA_VARIANT_STAGED;
@@ -594,6 +599,19 @@ int ma_fwd_select_variant(const ma_fwd_params* p) {
     const int st = check_shape(p);
     if (st != MA_OK) return st;
     return select_variant(p);
+}
+
+const char* ma_fwd_kernel_name(const ma_fwd_params* p) {
+    if (check_shape(p) != MA_OK) return nullptr;
+    const bool f32 = p->dtype_qk == MA_F32;
+    switch (select_variant(p)) {
+        case MA_VARIANT_GENERIC: return "r_step_kernel";
+        case MA_VARIANT_STAGED: return f32 ? "r_step_f32" : "r_step_mfma";
+        case MA_VARIANT_FUSED: return "fused_fwd_mfma";
+        case MA_VARIANT_CHAINED: return "chain_fwd_mfma";
+        case MA_VARIANT_RESIDENT: return f32 ? "head_fwd_f32" : resident_head_fits(p) ? "resident_head_mfma" : "resident_fwd_mfma";
+        default: return nullptr;
+    }
 }
 
 int ma_r_step(const ma_fwd_params* p, int first, int with_v, void* stream) {

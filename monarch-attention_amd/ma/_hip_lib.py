@@ -59,7 +59,7 @@ MA_FLAG_TEST_NO_SPIN = 2
 MA_FLAG_DEVICE_EXCLUSIVE = 4
 
 EXPORTS = ("ma_abi_version", "ma_strerror", "ma_fwd_workspace_layout", "ma_fwd_workspace_bytes",
-           "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd", "ma_fwd_static", "ma_r_step", "ma_l_step", "ma_z_step",
+           "ma_workspace_init", "ma_fwd_select_variant", "ma_fwd_kernel_name", "ma_fwd", "ma_fwd_static", "ma_r_step", "ma_l_step", "ma_z_step",
            "ma_matrix", "ma_bwd_workspace_bytes", "ma_bwd")
 
 _lock = threading.Lock()
@@ -99,6 +99,8 @@ def load() -> C.CDLL:
         lib.ma_workspace_init.argtypes = [P, C.c_void_p]
         lib.ma_fwd_select_variant.restype = C.c_int
         lib.ma_fwd_select_variant.argtypes = [P]
+        lib.ma_fwd_kernel_name.restype = C.c_char_p
+        lib.ma_fwd_kernel_name.argtypes = [P]
         lib.ma_fwd.restype = C.c_int
         lib.ma_fwd.argtypes = [P, C.c_void_p]
         lib.ma_fwd_static.restype = C.c_int

@@ -146,6 +146,30 @@ def test_select_variant_reports_a_known_variant():
     assert lib.ma_fwd_select_variant(p32) in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["resident"])
 
 
+def test_kernel_name_follows_the_resolved_variant():
+    lib = L.load()
+
+    def name(E, H, N, D, B, dt=L.MA_F16, T=2, variant="auto", flags=0):
+        p = good_params()
+        p.E, p.H, p.N, p.D, p.Dv, p.B, p.T, p.flags = E, H, N, D, D, B, T, flags
+        p.dtype_qk = p.dtype_v = dt
+        p.variant = L.VARIANTS[variant]
+        for field in ("q_stride", "k_stride", "v_stride", "out_stride"):
+            setattr(p, field, (C.c_int64 * 3)(H * N * D, N * D, D))
+        got = lib.ma_fwd_kernel_name(p)
+        return got.decode() if got is not None else None
+
+    assert name(1, 16, 4096, 64, 64) == "chain_fwd_mfma"
+    assert name(1, 16, 4096, 64, 64, flags=L.MA_FLAG_DEVICE_EXCLUSIVE) == "fused_fwd_mfma"
+    assert name(64, 12, 197, 64, 16) == "resident_head_mfma"      # the head fits in LDS with its inputs
+    assert name(16, 12, 512, 64, 32) == "resident_fwd_mfma"       # state only
+    assert name(1, 16, 4096, 64, 256) == "r_step_mfma"
+    assert name(1, 1, 256, 64, 16, dt=L.MA_F32, T=1) == "r_step_f32"
+    assert name(8, 8, 197, 64, 16, dt=L.MA_F32) == "head_fwd_f32"
+    assert name(1, 16, 4096, 60, 64) == "r_step_kernel"           # D % 8 != 0: the FMA kernels
+    assert name(1, 16, 0, 64, 64) is None                         # invalid problem
+
+
 def test_check_maps_status_to_python_exceptions():
     with pytest.raises(ValueError):
         L.check(L.MA_ERR_SHAPE, "x")
