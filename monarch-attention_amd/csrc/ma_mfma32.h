@@ -150,10 +150,10 @@ struct Which {
     long long eh;
     bool active;
 };
-__device__ __forceinline__ Which which_problem(const Problem& P, int count) {
+__device__ __forceinline__ Which which_problem(const Problem& P, int count, int parts = 1) {
     Which w;
     const unsigned total = static_cast<unsigned>(P.E) * P.H * count;
-    unsigned pid = blockIdx.x;
+    unsigned pid = blockIdx.x / static_cast<unsigned>(parts);
     w.active = pid < total;
     if (!w.active) pid = 0;
     w.idx = pid % static_cast<unsigned>(count);
@@ -165,16 +165,22 @@ __device__ __forceinline__ Which which_problem(const Problem& P, int count) {
 }
 
 // ---------------------------------------------------------------- R step: al_cl_ref / al_y_cl_ref (ma/ma_torch.py:10-23, :38-52)
-template <int DTF, int NWT>
+// HV = 2: a problem whose waves walk two strips each is run as two workgroups of one strip per wave (workgroups
+// 2 p and 2 p + 1; both stage the whole key / value tiles).  The fp32 matrix instructions of a strip are one
+// dependent chain per accumulator, so a wave's time is its strips' MFMA count: a launch that leaves compute
+// units idle asks for the halves (the graph-transformer shape: 120 problems of 128 rows on 256 compute units).
+template <int DTF, int NWT, int HV = 1>
 __global__ __launch_bounds__(64 * Split<NWT>::WPP) void r_step_f32(Problem P, int first_i, int with_v_i) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    constexpr int WPP = Split<NWT>::WPP, SPW = NWT / WPP, ROWS = 16 * NWT, LD = Geom32<DTF>::LD;
+    constexpr int WPP = Split<NWT>::WPP, SPW = NWT / WPP / HV, ROWS = 16 * NWT, LD = Geom32<DTF>::LD;
+    static_assert(NWT % (WPP * HV) == 0, "a half must be whole strips per wave");
+    const int half = HV == 1 ? 0 : static_cast<int>(blockIdx.x % HV);
     float* Kt = reinterpret_cast<float*>(smem);
     float* Vt = Kt + Lds32<DTF, NWT>::TILE;
     float* kbias = Vt + Lds32<DTF, NWT>::TILE;
     const bool first = first_i != 0, with_v = with_v_i != 0;
     const int wig = wave_id(), lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4, tix = threadIdx.x;
-    const Which w = which_problem(P, P.M);
+    const Which w = which_problem(P, P.M, HV);
     if (!w.active) return;
     const int B = P.B, M = P.M, D = P.D, m = w.idx;
     const Slices S = make_slices<float>(P, w.e, w.h, w.eh);
@@ -194,7 +200,7 @@ __global__ __launch_bounds__(64 * Split<NWT>::WPP) void r_step_f32(Problem P, in
 
 #pragma unroll
     for (int si = 0; si < SPW; ++si) {
-        const int j = 16 * (wig + si * WPP) + r;
+        const int j = 16 * (half * (NWT / HV) + wig + si * WPP) + r;
         const bool jv = j < B;
         f32x4 xb[DTF];
         float cr = 1.0f;

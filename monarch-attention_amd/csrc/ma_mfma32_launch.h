@@ -40,6 +40,16 @@ inline int launch_r(const Problem& P, bool first, bool with_v, hipStream_t s) {
         const int attr = mfma::set_lds_limit(r_step_f32<DTF, NWT>, lds);
         if (attr) return attr;
         const long long problems = static_cast<long long>(P.E) * P.H * P.M;
+        if constexpr (NWT == 8) {   // two strips per wave: as two workgroups each while that still leaves compute units idle
+            const mfma::DeviceCaps caps = mfma::device_caps(r_step_f32<DTF, NWT>, 0, 0);
+            if (caps.err) return caps.err;
+            if (2 * problems <= caps.cus) {
+                const int attr2 = mfma::set_lds_limit(r_step_f32<DTF, NWT, 2>, lds);
+                if (attr2) return attr2;
+                hipLaunchKernelGGL((r_step_f32<DTF, NWT, 2>), dim3(2 * problems), dim3(64 * Split<NWT>::WPP), lds, s, P, first ? 1 : 0, with_v ? 1 : 0);
+                return static_cast<int>(hipGetLastError());
+            }
+        }
         hipLaunchKernelGGL((r_step_f32<DTF, NWT>), dim3(problems), dim3(64 * Split<NWT>::WPP), lds, s, P, first ? 1 : 0, with_v ? 1 : 0);
         return static_cast<int>(hipGetLastError());
     });
