@@ -400,14 +400,18 @@ def main():
     def time_forward(T_, variant, steps, warmup, rotate=None):
         ps, ws = prepared(T_, variant, rotate)
         run_steps(ps, max(warmup, nbuf))
+        # the timed region: exactly `steps` forward calls between two synchronisations, nothing else queued
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        run_steps(ps, steps)
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        # the same steps once more between two events on the launch stream (device-side time per step)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
         run_steps(ps, steps)
         e1.record(stream)
         torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
         return wall_ms, e0.elapsed_time(e1) / steps, ps, ws
 
     if args.matrix:
