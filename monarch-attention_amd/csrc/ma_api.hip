@@ -312,10 +312,13 @@ int select_variant(const ma_fwd_params* p) {
             // (256 tokens x 64: 0.93 of the stage launches' time at 96 heads, 0.5 - 0.7 from 192 on, also
             // beyond one pass over the compute units) and for any head count when the head is small
             // (128 tokens x 32: 0.45 - 0.8); few large heads are faster spread over many compute units
-            // by the stage launches (one head of 256 x 64: 8 us against 13).
+            // by the stage launches (one head of 256 x 64, two steps: 16.6 us against 20.4) - unless there is a
+            // single step: then a workgroup per (head, position) needs nothing from any other (one head of
+            // 256 x 64: 5.3 us against 7.9 as two launches; 16 heads: 6.7 against 10.3).
             if (fast32) {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-                const bool pays = heads >= 64 || M * p->B * p->D <= 4096;
+                const bool single_step = p->T == 1 && heads * p->B <= kHead32T1MaxGroups;
+                const bool pays = heads >= 64 || M * p->B * p->D <= 4096 || single_step;
                 return pays && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_VARIANT_STAGED;
             }
             if (!fast) return MA_VARIANT_GENERIC;
@@ -609,7 +612,14 @@ const char* ma_fwd_kernel_name(const ma_fwd_params* p) {
         case MA_VARIANT_STAGED: return f32 ? "r_step_f32" : "r_step_mfma";
         case MA_VARIANT_FUSED: return "fused_fwd_mfma";
         case MA_VARIANT_CHAINED: return "chain_fwd_mfma";
-        case MA_VARIANT_RESIDENT: return f32 ? "head_fwd_f32" : resident_head_fits(p) ? "resident_head_mfma" : "resident_fwd_mfma";
+        case MA_VARIANT_RESIDENT: {
+            if (!f32) return resident_head_fits(p) ? "resident_head_mfma" : "resident_fwd_mfma";
+            Problem P;
+            std::memset(&P, 0, sizeof(P));
+            P.E = p->E; P.H = p->H; P.N = p->N; P.D = p->D; P.Dv = p->Dv; P.B = p->B; P.T = p->T;
+            P.M = (p->N + p->B - 1) / p->B;
+            return head32_single_step(P) ? "head_t1_f32" : "head_fwd_f32";
+        }
         default: return nullptr;
     }
 }

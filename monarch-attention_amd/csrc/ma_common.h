@@ -186,6 +186,14 @@ int launch_resident_bf16_d8(const Problem& P, bool dry_run, hipStream_t s);
 
 // fp32 heads of at most 16 blocks of at most 16 rows, head dim up to 64: one launch, state in LDS.
 int launch_head32(const Problem& P, bool dry_run, hipStream_t s);
+// ... of which few heads with a single step run as one workgroup per (head, in-block position) that
+// recomputes the rows of the R step it needs (no exchange between workgroups): every workgroup reads
+// the head's whole K and V, so only while the launch stays within kHead32T1MaxGroups workgroups.
+constexpr long long kHead32T1MaxGroups = 256;
+inline bool head32_single_step(const Problem& P) {
+    return P.T == 1 && P.B <= 16 && P.M <= 16 && P.D <= 64 && P.D % 4 == 0 && P.Dv == P.D &&
+           static_cast<long long>(P.E) * P.H * P.B <= kHead32T1MaxGroups;
+}
 
 // Chained forward (one launch, one workgroup per block problem, flags between phases).
 int launch_chain_f16_d2(const Problem& P, bool sync_ready, hipStream_t s);

@@ -164,7 +164,8 @@ def test_kernel_name_follows_the_resolved_variant():
     assert name(64, 12, 197, 64, 16) == "resident_head_mfma"      # the head fits in LDS with its inputs
     assert name(16, 12, 512, 64, 32) == "resident_fwd_mfma"       # state only
     assert name(1, 16, 4096, 64, 256) == "r_step_mfma"
-    assert name(1, 1, 256, 64, 16, dt=L.MA_F32, T=1) == "r_step_f32"
+    assert name(1, 1, 256, 64, 16, dt=L.MA_F32, T=1) == "head_t1_f32"
+    assert name(1, 1, 256, 64, 16, dt=L.MA_F32, T=2) == "r_step_f32"
     assert name(8, 8, 197, 64, 16, dt=L.MA_F32) == "head_fwd_f32"
     assert name(1, 16, 4096, 60, 64) == "r_step_kernel"           # D % 8 != 0: the FMA kernels
     assert name(1, 16, 0, 64, 64) is None                         # invalid problem
@@ -252,7 +253,9 @@ def test_auto_variant_policy():
     assert auto(1, 1, 16, 64, 4, T=1) == "chained"
     assert auto(1, 16, 4096, 64, 64, dt=L.MA_F32) == "staged"       # fp32 MFMA stage kernels
     assert auto(1, 2, 7600, 48, 128, dt=L.MA_F32) == "staged"
-    assert auto(1, 1, 256, 64, 16, dt=L.MA_F32, T=1) == "staged"    # one small fp32 head: spread over compute units by the stage launches
+    assert auto(1, 1, 256, 64, 16, dt=L.MA_F32, T=1) == "resident"  # few small fp32 heads, one step: a workgroup per (head, position)
+    assert auto(1, 1, 256, 64, 16, dt=L.MA_F32, T=2) == "staged"    # ... more steps: spread over compute units by the stage launches
+    assert auto(1, 17, 256, 64, 16, dt=L.MA_F32, T=1) == "staged"   # ... more than 256 workgroups likewise
     assert auto(8, 8, 197, 64, 16, dt=L.MA_F32) == "resident"       # from 64 heads on: one workgroup per head, one launch
     assert auto(64, 12, 197, 64, 16, dt=L.MA_F32) == "resident"
     assert auto(1, 2, 128, 32, 16, dt=L.MA_F32) == "resident"       # ... and for very small heads always

@@ -10,6 +10,8 @@ calls change neither the device's free memory nor PyTorch's allocator
 statistics; and a call that would overlap with one on another stream is turned
 away (MA_ERR_BUSY).
 """
+import gc
+
 import pytest
 import torch
 
@@ -95,13 +97,20 @@ def test_static_allocates_and_frees_nothing():
         p = make_params(q, k, v, None, out, T, B, False, variant)
         L.check(lib.ma_fwd_static(p, stream), "warm-up")
         torch.cuda.synchronize()
-        free0, total0 = torch.cuda.mem_get_info()
-        stats0 = {k_: v_ for k_, v_ in torch.cuda.memory_stats().items() if k_.endswith(".current") or k_.endswith(".allocated") or k_.endswith(".freed")}
-        for _ in range(3):
-            L.check(lib.ma_fwd_static(p, stream), "ma_fwd_static")
-        torch.cuda.synchronize()
-        free1, total1 = torch.cuda.mem_get_info()
-        stats1 = {k_: v_ for k_, v_ in torch.cuda.memory_stats().items() if k_ in stats0}
+        # nothing of this process may allocate or free in the measured region but the calls themselves: tensors
+        # that earlier tests left to the garbage collector are collected now, and the collector is held off
+        gc.collect()
+        gc.disable()
+        try:
+            free0, total0 = torch.cuda.mem_get_info()
+            stats0 = {k_: v_ for k_, v_ in torch.cuda.memory_stats().items() if k_.startswith(("allocation.all.", "segment.all."))}
+            for _ in range(3):
+                L.check(lib.ma_fwd_static(p, stream), "ma_fwd_static")
+            torch.cuda.synchronize()
+            free1, total1 = torch.cuda.mem_get_info()
+            stats1 = {k_: v_ for k_, v_ in torch.cuda.memory_stats().items() if k_ in stats0}
+        finally:
+            gc.enable()
         assert (free1, total1) == (free0, total0), f"{variant}: free device memory changed by {free0 - free1} bytes"
         assert stats1 == stats0, f"{variant}: PyTorch allocator statistics changed"
 
