@@ -168,7 +168,7 @@ def main():
                          "N = 256 .. 8192, blocks of 16 .. 128 rows (T from --T, default 2; head dim from --head-dim); prints the rows "
                          "and how far AUTO's choice is from the fastest variant")
     ap.add_argument("--head-dim", type=int, default=64, help="head dim of --sweep-variants")
-    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96", "fewheads", "ragged"],
+    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96", "fewheads", "ragged", "mid"],
                     help="shapes of --sweep-variants: power-of-two lengths and blocks, blocks / block counts in the 96-row tile class, "
                          "few heads of thousands of tokens, or lengths that are no multiple of the block (197, 500, 1000, 3000, 5000, 7600)")
     ap.add_argument("--sweep-dtype", default="f16", choices=["f16", "bf16", "f32"], help="operand dtype of --sweep-variants")
@@ -303,6 +303,10 @@ def main():
         elif args.sweep_grid == "ragged":     # lengths of the reference's models: ViT 197, BART / RoBERTa prefixes, GPS graphs
             grid = [(h, N, B) for h in (2, 8, 12, 16, 48, 96, 192, 768) for (N, B) in ((197, 14), (197, 16), (500, 24), (1000, 32), (1000, 48),
                                                                                   (3000, 55), (3000, 64), (5000, 71), (5000, 128), (7600, 88), (7600, 128))]
+        elif args.sweep_grid == "mid":        # heads of 256 .. 1000 tokens: the forms of the resident kernel against the rest
+            grid = [(h, N, B) for h in (4, 16, 32, 64, 96, 128, 192, 256, 384, 512, 768)
+                    for (N, B) in ((256, 16), (256, 32), (288, 16), (320, 32), (384, 16), (384, 24), (384, 32), (400, 25), (448, 32), (448, 64),
+                                   (500, 24), (512, 16), (512, 32), (512, 64), (540, 36), (768, 32), (1000, 32))]
         elif args.sweep_grid == "fewheads":   # 8, 16, 24 heads of thousands of tokens: where the team kernel competes
             grid = [(h, N, B) for h in (8, 16, 24) for N in (2048, 4096, 5000, 6144, 8000, 8192) for B in (32, 64, 128)]
         else:   # blocks and / or block counts of 65 .. 96 rows (and two 128-row shapes with ragged block counts)

@@ -192,13 +192,14 @@ bool resident_fits(const ma_fwd_params* p, bool one_tile) {
     return run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
 }
 
-// Does the head - Q, K, V and the state - fit in LDS whole (the fastest form of the resident kernel)?
-bool resident_head_fits(const ma_fwd_params* p) {
+// Does the head fit in LDS whole (the head-resident forms of the resident kernel)?  forms = 1: Q, K, V and the
+// state in four tiles; 2: that, or the state and one input tile at a time.
+bool resident_head_fits(const ma_fwd_params* p, int forms = 1) {
     Problem P;
     std::memset(&P, 0, sizeof(P));
     P.E = p->E; P.H = p->H; P.N = p->N; P.D = p->D; P.Dv = p->Dv; P.B = p->B; P.T = p->T;
     P.M = (p->N + p->B - 1) / p->B;
-    P.resident_head_only = 1;
+    P.resident_head_only = forms;
     return p->dtype_qk != MA_F32 && run_resident(P, p->dtype_qk, true, nullptr) == MA_OK;
 }
 
@@ -331,6 +332,15 @@ int select_variant(const ma_fwd_params* p) {
                 // single step of few heads: 1.03 - 1.23, they stay away).  Head dims up to 64: in the 128-column class
                 // the kernel holds heads of ~128 tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
                 if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= (p->T >= 2 ? 128 : 96) || (p->T >= 2 && p->B <= 16)) && resident_head_fits(p))
+                    return MA_VARIANT_RESIDENT;
+                // Heads of about twice that length (257 .. ~540 tokens at D = 64) keep the state and ONE input tile at a
+                // time in LDS.  A head has a compute unit to itself for its 2T phases, so the device has to be full of
+                // heads: from 192 heads on with more than one step (0.64 - 0.94 of the next best variant's time at
+                // 192 .. 768 heads, T = 2, 3; 0.95 - 1.10 at 128 heads), with a single step only where the heads fill
+                // the compute units once (256 heads: 0.84 - 0.96; 192 or 384 heads: 0.90 - 1.13).  Blocks and block
+                // counts of at most 32 (16 waves per workgroup; 64-row blocks at eight waves: 0.84 - 1.17).
+                if (p->D <= 80 && p->B <= 32 && M <= 32 && (p->T >= 2 ? heads >= 192 : (heads >= 224 && heads <= 256)) &&
+                    !resident_head_fits(p, 1) && resident_head_fits(p, 2))
                     return MA_VARIANT_RESIDENT;
                 if (p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= 128 && resident_fits(p, false))
                     return MA_VARIANT_RESIDENT;
@@ -613,7 +623,7 @@ const char* ma_fwd_kernel_name(const ma_fwd_params* p) {
         case MA_VARIANT_FUSED: return "fused_fwd_mfma";
         case MA_VARIANT_CHAINED: return "chain_fwd_mfma";
         case MA_VARIANT_RESIDENT: {
-            if (!f32) return resident_head_fits(p) ? "resident_head_mfma" : "resident_fwd_mfma";
+            if (!f32) return resident_head_fits(p, 1) ? "resident_head_mfma" : resident_head_fits(p, 2) ? "resident_head2_mfma" : "resident_fwd_mfma";
             Problem P;
             std::memset(&P, 0, sizeof(P));
             P.E = p->E; P.H = p->H; P.N = p->N; P.D = p->D; P.Dv = p->Dv; P.B = p->B; P.T = p->T;

@@ -39,7 +39,8 @@ struct Problem {
     // The resident kernel may keep aL and aR in ONE LDS tile and pass Y through the workspace where two or
     // three tiles do not fit (heads of up to ~512 tokens at d = 64).
     int one_tile_ok;
-    // Query only: does the form of the resident kernel that keeps Q, K and V in LDS as well take this head?
+    // Query only: does a head-resident form of the resident kernel take this head?  1: the one that keeps Q, K and V
+    // in LDS beside the state; 2: that one or the two-tile form (the state and one input tile at a time).
     int resident_head_only;
     int test_no_spin;    // waits between workgroups give up at once (failure-path tests)
     // Copy of the error word in host memory the device can write (or null): a workgroup that raises the

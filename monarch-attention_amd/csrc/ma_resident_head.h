@@ -130,8 +130,9 @@ struct HeadRes {
 
     // The loads of the next head: Q and the mask, K, V.  Their offsets are recomputed every time: a few dozen
     // instructions per head, against registers that would be held through every round.
-    static __device__ __forceinline__ void chunk_offsets(const Problem& P, const Ctx& c, unsigned st, unsigned (&off)[NI]) {
-        const int Np = P.M * P.B;
+    // (live = false: nothing is fetched - every chunk reads as zeros - but the registers are written all the same)
+    static __device__ __forceinline__ void chunk_offsets(const Problem& P, const Ctx& c, unsigned st, unsigned (&off)[NI], bool live = true) {
+        const int Np = live ? P.M * P.B : 0;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int cc = c.tid + i * NT, p = cc / CH, ch = cc % CH;
@@ -140,7 +141,7 @@ struct HeadRes {
             off[i] = ok ? static_cast<unsigned>(t) * st + ch * 16 : kOob;
         }
     }
-    static __device__ __forceinline__ void issue_q(const Problem& P, const Ctx& c, const Head& hd, Pre& pre) {
+    static __device__ __forceinline__ void issue_q(const Problem& P, const Ctx& c, const Head& hd, Pre& pre, bool live = true) {
         if (P.mask != nullptr) {   // uniform; first: whoever looks at it waits for nothing issued behind it
             // the thread's entry of tokb: block tid / ROWSB, row tid % ROWSB
             const int m = c.tid / ROWSB, i = c.tid % ROWSB, t = m * P.B + i - P.pad_off;
@@ -151,7 +152,7 @@ struct HeadRes {
             if (P.mask_shift == 3) pre.mk64 = __builtin_amdgcn_raw_buffer_load_b64(hd.mask, moff, 0, 0);
         }
         unsigned off[NI];
-        chunk_offsets(P, c, c.qst, off);
+        chunk_offsets(P, c, c.qst, off, live);
 #pragma unroll
         for (int i = 0; i < NI; ++i) pre.q[i] = bload16<false>(hd.q, off[i]);
     }
@@ -279,7 +280,13 @@ struct HeadRes {
     // ---------------------------------------------------------------- the three kinds of rounds
     // R round: al_cl_ref / al_y_cl_ref (ma/ma_torch.py:10-23, :38-52).  Problem m: keys and values are the rows of
     // block m, queries the rows aR(m, .) - Q's rows of the block in the first step.
-    static __device__ __forceinline__ void round_r(const Problem& P, const Ctx& c, int rnd, bool first, bool with_v, bool scale_is_f16) {
+    // TWO: the two-tile form (ma_resident_head2.h).  The first step's query rows are in S as well (S starts out as
+    // Q), and V is not in LDS: the waves of the problem load block m's V rows at the top of the round and write them
+    // over the block's K rows once every wave of the problem has had its last look at those.
+    static constexpr int NV = (ROWSB * CH + 64 * WPB - 1) / (64 * WPB);   // 16-byte chunks of a block's V rows per lane of the problem
+    template <bool TWO = false>
+    static __device__ __forceinline__ void round_r(const Problem& P, const Ctx& c, int rnd, bool first, bool with_v, bool scale_is_f16,
+                                                   const Head* hd = nullptr) {
         const int B = P.B, M = P.M;
         const int grp = c.wave / WPB, wig = c.wave % WPB;
         const int m = rnd * PPB + grp;
@@ -288,9 +295,21 @@ struct HeadRes {
         const int j = 16 * wig + r;
         const bool ok = j < B;
         V8 pb[(NTB + 1) / 2];
+        u32x4 vv[TWO ? NV : 1];
+        if constexpr (TWO) {
+            if (with_v && active) {   // uniform per wave
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    const int cc = wig * 64 + c.lane + i * 64 * WPB, row = cc / CH, ch = cc % CH;
+                    const int t = m * B + row - P.pad_off;
+                    const bool in = row < B && static_cast<unsigned>(t) < static_cast<unsigned>(P.N) && ch * 8 < P.D;
+                    vv[i] = bload16<false>(hd->v, in ? static_cast<unsigned>(t) * c.vst + ch * 16 : kOob);
+                }
+            }
+        }
         if (active) {
             const T* Kt = c.row(c.L.K, m, 0);
-            const T* xrow = ok ? c.row(first ? c.L.Q : c.L.S, m, j) : c.at(c.L.ZR);
+            const T* xrow = ok ? c.row((first && !TWO) ? c.L.Q : c.L.S, m, j) : c.at(c.L.ZR);
             V8 xb[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) xb[ks] = lds_row8<T>(xrow + 32 * ks + 8 * q);
@@ -340,6 +359,21 @@ struct HeadRes {
             f32x4 O[DT];
             gemm2_rows<NTB, true>(O, c, Kt, RB, ROWSB, pb);
             lds_store_row_scaled(ok ? c.row(c.L.S, m, j) : c.at(c.L.TR), O, q, P.sm_scale, scale_is_f16);
+        }
+        if constexpr (TWO) {
+            if (with_v) {   // uniform
+                problem_sync<WPB>();   // every wave of the problem has read the block's K rows for the last time
+                if (active) {
+#pragma unroll
+                    for (int i = 0; i < NV; ++i) {
+                        const int cc = wig * 64 + c.lane + i * 64 * WPB, row = cc / CH, ch = cc % CH;
+                        // (rows behind a block that is no multiple of 16 rows long belong to the next block: they stay as
+                        // they are - their probabilities are zero)
+                        *reinterpret_cast<u32x4*>(row < B ? reinterpret_cast<char*>(c.row(c.L.K, m, row)) + ch * 16 : c.smem + c.L.TR + ch * 16) = vv[i];
+                    }
+                }
+                problem_sync<WPB>();
+            }
         }
         if (with_v) {   // uniform
             f32x4 O[DT];
@@ -444,7 +478,20 @@ struct HeadRes {
     }
 
     // Z round: z_ref (ma/ma_torch.py:55-62) and the final slice (:106-108)
-    static __device__ __forceinline__ void round_z(const Problem& P, const Ctx& c, const Head& hd, int rnd) {
+    // the query row (l, j) of this lane in Z round rnd, straight from memory (two-tile form: Q is not in LDS then)
+    static __device__ __forceinline__ void load_zq(const Problem& P, const Ctx& c, const Head& hd, int rnd, V8 (&xq)[KS]) {
+        const int grp = c.wave / WPM, wig = c.wave % WPM;
+        const int j = rnd * PPM + grp, l = 16 * wig + c.r;
+        const int t = l * P.B + j - P.pad_off;
+        const bool in = j < P.B && l < P.M && static_cast<unsigned>(t) < static_cast<unsigned>(P.N);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int col = 32 * ks + 8 * c.q;
+            xq[ks] = __builtin_bit_cast(V8, bload16<false>(hd.q, (in && col < P.D) ? static_cast<unsigned>(t) * c.qst + col * 2 : kOob));
+        }
+    }
+    template <bool TWO = false>
+    static __device__ __forceinline__ void round_z(const Problem& P, const Ctx& c, const Head& hd, int rnd, const V8* zq = nullptr) {
         const int B = P.B, M = P.M;
         const int grp = c.wave / WPM, wig = c.wave % WPM;
         const int j = rnd * PPM + grp;
@@ -459,7 +506,10 @@ struct HeadRes {
         const T* xrow = l < M ? blk(Qj, l) : zr;
         V8 xq[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) xq[ks] = lds_row8<T>(xrow + 32 * ks + 8 * q);
+        for (int ks = 0; ks < KS; ++ks) {
+            if constexpr (TWO) xq[ks] = zq[ks];
+            else xq[ks] = lds_row8<T>(xrow + 32 * ks + 8 * q);
+        }
         f32x4 C[NTM];
 #pragma unroll
         for (int wt = 0; wt < NTM; ++wt) {

@@ -7,6 +7,7 @@
 #include "ma_mfma_launch.h"
 #include "ma_resident.h"
 #include "ma_resident_head.h"
+#include "ma_resident_head2.h"
 
 namespace ma {
 namespace mfma {
@@ -82,12 +83,43 @@ int launch_resident_head(const Problem& P, bool dry_run, hipStream_t s) {
     return launch_resident_head_ni<T, DT, NTB, NTM, W, 3>(P, dry_run, s);
 }
 
+// Heads of about twice that length: the state and one input tile at a time in LDS (ma_resident_head2.h).
+template <class T, int DT, int NTB, int NTM, int W, int NI>
+int launch_resident_head2_ni(const Problem& P, bool dry_run, hipStream_t s) {
+    using H2 = HeadRes2<T, DT, NTB, NTM, W, NI>;
+    const int Np = P.M * P.B;
+    if (!H2::fits(Np, P.B, P.M, kLdsPerCu)) return MA_ERR_UNSUPPORTED;
+    if (dry_run) return MA_OK;
+    auto kernel = resident_head2_mfma<T, DT, NTB, NTM, W, NI>;
+    const int lds_err = set_lds_limit(kernel, kLdsPerCu);
+    if (lds_err) return lds_err;
+    const DeviceCaps caps = device_caps(kernel, 0, 0);
+    if (caps.err) return caps.err;
+    if (caps.cus < 1) return MA_ERR_DEVICE;
+    const long long heads = static_cast<long long>(P.E) * P.H;
+    const long long grid = heads < caps.cus ? heads : caps.cus;
+    hipLaunchKernelGGL((resident_head2_mfma<T, DT, NTB, NTM, W, NI>), dim3(grid), dim3(64 * W), H2::layout(Np, P.B, P.M).total, s, P);
+    return static_cast<int>(hipGetLastError());
+}
+template <class T, int DT, int NTB, int NTM>
+int launch_resident_head2(const Problem& P, bool dry_run, hipStream_t s) {
+    constexpr int W = (NTB <= 2 && NTM <= 2) ? 16 : 8;
+    // 4096 or 5120 16-byte chunks per tile (the larger covers every tile that fits the LDS twice)
+    const int err = launch_resident_head2_ni<T, DT, NTB, NTM, W, 4096 / (64 * W)>(P, dry_run, s);
+    if (err != MA_ERR_UNSUPPORTED) return err;
+    return launch_resident_head2_ni<T, DT, NTB, NTM, W, 5120 / (64 * W)>(P, dry_run, s);
+}
+
 // The problems of a head are small and latency-bound: more waves per workgroup run more of
 // them at once, so the wide workgroup is preferred wherever its staging fits beside the state.
 template <class T, int DT, int NTB, int NTM>
 int launch_resident_one(const Problem& P, bool dry_run, hipStream_t s) {
     {   // everything in LDS where the head is short enough for that
         const int err = launch_resident_head<T, DT, NTB, NTM>(P, dry_run, s);
+        if (err != MA_ERR_UNSUPPORTED || P.resident_head_only == 1) return err;
+    }
+    {
+        const int err = launch_resident_head2<T, DT, NTB, NTM>(P, dry_run, s);
         if (err != MA_ERR_UNSUPPORTED || P.resident_head_only) return err;
     }
     if constexpr (NTB <= 2 && NTM <= 2) {

@@ -162,7 +162,11 @@ def test_kernel_name_follows_the_resolved_variant():
     assert name(1, 16, 4096, 64, 64) == "chain_fwd_mfma"
     assert name(1, 16, 4096, 64, 64, flags=L.MA_FLAG_DEVICE_EXCLUSIVE) == "fused_fwd_mfma"
     assert name(64, 12, 197, 64, 16) == "resident_head_mfma"      # the head fits in LDS with its inputs
-    assert name(16, 12, 512, 64, 32) == "resident_fwd_mfma"       # state only
+    assert name(16, 12, 512, 64, 32) == "resident_head2_mfma"     # twice that length: the state and one input tile at a time
+    assert name(16, 16, 512, 64, 32, T=1) == "resident_head2_mfma"   # a single step: only where the heads fill the compute units once
+    assert name(16, 12, 512, 64, 32, T=1) == "chain_fwd_mfma"
+    assert name(8, 12, 512, 64, 32) == "chain_fwd_mfma"           # ... 96 heads do not fill the device
+    assert name(16, 12, 1000, 32, 32, variant="resident") == "resident_fwd_mfma"   # state only
     assert name(1, 16, 4096, 64, 256) == "r_step_mfma"
     assert name(1, 1, 256, 64, 16, dt=L.MA_F32, T=1) == "head_t1_f32"
     assert name(1, 1, 256, 64, 16, dt=L.MA_F32, T=2) == "r_step_f32"
@@ -230,9 +234,13 @@ def test_auto_variant_policy():
     assert auto(16, 12, 384, 64, 96) == "chained"       # ... also for 96-row blocks
     assert auto(1, 16, 8192, 64, 90) == "chained"       # 92 blocks of 90 rows: the chained kernel has the 96-row class too
     assert auto(64, 12, 197, 64, 16) == "resident"
-    assert auto(16, 12, 512, 64, 32) == "resident"     # 512-token heads: aL / aR in one LDS tile, Y through the workspace
-    assert auto(8, 12, 512, 64, 32) == "chained"       # ... when the head count fills the device's workgroups
-    assert auto(32, 12, 512, 64, 32) == "chained"      # (384 heads: 1.5 passes over 256 CUs)
+    assert auto(16, 12, 512, 64, 32) == "resident"     # 512-token heads: the state and one input tile at a time in LDS
+    assert auto(8, 12, 512, 64, 32) == "chained"       # ... when there are enough heads for the compute units (a head has one to itself)
+    assert auto(32, 12, 512, 64, 32) == "resident"     # (384 heads, 1.5 passes over 256 CUs: still 0.85 of the chained kernel's time)
+    assert auto(16, 12, 512, 64, 32, T=1) == "chained" # a single step: only where the heads fill the compute units once
+    assert auto(16, 16, 512, 64, 32, T=1) == "resident"
+    assert auto(16, 12, 512, 64, 64) == "chained"      # 64-row blocks (eight waves per workgroup)
+    assert auto(16, 12, 768, 64, 32) == "chained"      # beyond two tiles: the one-tile form is no match for the chained kernel here
     assert auto(16, 12, 512, 64, 64) == "chained"      # ... and for problems of one or two strips
     assert auto(32, 12, 256, 64, 64) == "chained"      # 64-row blocks never run resident
     assert auto(16, 12, 256, 64, 32) == "resident"     # 256-token heads fit in LDS with their inputs: from 128 heads on

@@ -239,23 +239,57 @@ def test_few_long_heads_run_in_the_team_kernel(E, H, N, D, B, T, pre, dt, masked
     assert sync_status() == 0
 
 
-ONE_TILE = [  # E, H, N, D, B, T, pre, dt, masked: heads whose aL / aR / Y do not fit in LDS as three (or two) tiles
+TWO_TILE = [  # E, H, N, D, B, T, pre, dt, masked: heads too long for Q, K, V and the state in LDS, short enough for the state and one input tile
     (2, 3, 512, 64, 32, 2, False, "bf16", False), (1, 4, 500, 64, 32, 3, True, "f16", True),
     (1, 2, 384, 64, 24, 1, False, "f16", True), (2, 2, 448, 64, 16, 2, True, "bf16", False),
-    (1, 3, 300, 72, 20, 2, False, "f16", True), (1, 2, 1000, 32, 32, 2, False, "f16", False),
-    (1, 2, 512, 64, 64, 2, False, "f16", True), (1, 2, 470, 64, 48, 2, True, "bf16", False),
+    (1, 3, 300, 72, 20, 2, False, "f16", True), (1, 2, 900, 32, 32, 2, False, "f16", False),
+    (1, 2, 512, 64, 64, 2, False, "f16", True), (1, 2, 384, 64, 48, 2, True, "bf16", False),
+    (1, 2, 272, 128, 16, 3, False, "f16", True), (1, 2, 480, 40, 27, 1, True, "bf16", True), (1, 1, 300, 64, 10, 2, False, "f16", False),
     (30, 12, 400, 64, 25, 2, False, "f16", True),   # more heads than workgroups: a workgroup walks several heads
+    (16, 12, 512, 64, 32, 2, False, "bf16", False), (16, 16, 512, 64, 32, 1, True, "f16", True),   # what 'auto' sends there
+]
+
+ONE_TILE = [  # heads beyond that whose aL / aR / Y do not fit in LDS as three (or two) tiles either
+    (1, 2, 1000, 32, 32, 2, False, "f16", False), (2, 3, 768, 64, 32, 2, False, "bf16", True), (1, 2, 640, 64, 40, 3, True, "f16", True),
+    (1, 2, 600, 64, 64, 1, False, "f16", False), (1, 3, 420, 72, 30, 2, True, "bf16", True),
+    (30, 12, 700, 64, 28, 2, False, "f16", True),   # more heads than workgroups
 ]
 
 
-@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", ONE_TILE)
-def test_resident_kernel_with_one_state_tile(E, H, N, D, B, T, pre, dt, masked):
-    """Heads of ~300 .. 1000 tokens in the resident kernel: aL and aR share one LDS tile in place and Y goes
-    through the workspace."""
+def resident_kernel_name(dev, T, B, pre):
+    p = make_params(*dev[:3], dev[3], torch.empty_like(dev[2]), T, B, pre, "resident")
+    return L.load().ma_fwd_kernel_name(p).decode()
+
+
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", TWO_TILE)
+def test_resident_kernel_with_the_state_and_one_input_tile(E, H, N, D, B, T, pre, dt, masked):
+    """Heads of ~260 .. 540 tokens (D = 64) in the resident kernel: the state tile and one input tile in LDS, the
+    tile swapped at every phase boundary, V and Y in place of the K rows in the last R phase."""
     q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
     mask = block_safe_mask(E, N, B, seed=B) if masked else None
     ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
     dev = to_dev(q, k, v, mask)
+    assert resident_kernel_name(dev, T, B, pre) == "resident_head2_mfma"
+    out = monarch_attention_hip(*dev, T, B, pre, variant="resident")   # the variant must take these shapes
+    assert_parity(out.cpu(), ref, dt, f"two-tile resident {(E, H, N, D, B, T, pre, dt, masked)}")
+    again = monarch_attention_hip(*dev, T, B, pre, variant="resident")
+    assert torch.equal(out, again)
+    if E * H >= 192:
+        auto = monarch_attention_hip(*dev, T, B, pre, variant="auto")
+        p = make_params(*dev[:3], dev[3], torch.empty_like(dev[2]), T, B, pre, "auto")
+        assert L.VARIANT_NAMES[L.load().ma_fwd_select_variant(p)] == "resident"
+        assert torch.equal(out, auto)
+
+
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", ONE_TILE)
+def test_resident_kernel_with_one_state_tile(E, H, N, D, B, T, pre, dt, masked):
+    """Heads of ~550 .. 1000 tokens in the resident kernel: aL and aR share one LDS tile in place, the inputs are
+    streamed and Y goes through the workspace."""
+    q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
+    mask = block_safe_mask(E, N, B, seed=B) if masked else None
+    ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
+    dev = to_dev(q, k, v, mask)
+    assert resident_kernel_name(dev, T, B, pre) == "resident_fwd_mfma"
     out = monarch_attention_hip(*dev, T, B, pre, variant="resident")   # the variant must take these shapes
     assert_parity(out.cpu(), ref, dt, f"one-tile resident {(E, H, N, D, B, T, pre, dt, masked)}")
     again = monarch_attention_hip(*dev, T, B, pre, variant="resident")
