@@ -326,23 +326,33 @@ int select_variant(const ma_fwd_params* p) {
             {
                 const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
                 // heads that fit in LDS whole, in blocks and block counts of at most two strips (16 waves): every
-                // input is read once and no state leaves the compute unit.  From 128 heads on (0.63 - 0.93 of
-                // the next best variant's time at T = 1, 2), and with more than one step also for any number of
-                // heads in 16-row blocks (0.85 - 0.95 at 256 tokens, 0.55 - 0.8 for shorter heads and three steps; a
-                // single step of few heads: 1.03 - 1.23, they stay away).  Head dims up to 64: in the 128-column class
-                // the kernel holds heads of ~128 tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
-                if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= (p->T >= 2 ? 128 : 96) || (p->T >= 2 && p->B <= 16)) && resident_head_fits(p))
+                // input is read once and no state leaves the compute unit.  From 96 heads on (0.63 - 0.93 of
+                // the next best variant's time at T = 1, 2, 3), and with more than one step also for any number of
+                // heads of at most 256 tokens in 16-row blocks (0.85 - 0.95 at 256 tokens, 0.55 - 0.8 for shorter heads
+                // and three steps; longer heads at D = 32: 1.2 - 1.4 below 64 heads; a single step of few heads: 1.03 -
+                // 1.23, they stay away).  Head dims up to 64: in the 128-column class the kernel holds heads of ~128
+                // tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
+                if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= 96 || (p->T >= 2 && p->B <= 16 && M * p->B <= 256)) && resident_head_fits(p))
                     return MA_VARIANT_RESIDENT;
                 // Heads of about twice that length (257 .. ~540 tokens at D = 64) keep the state and ONE input tile at a
                 // time in LDS.  A head has a compute unit to itself for its 2T phases, so the device has to be full of
-                // heads: from 192 heads on with more than one step (0.64 - 0.94 of the next best variant's time at
-                // 192 .. 768 heads, T = 2, 3; 0.95 - 1.10 at 128 heads), with a single step only where the heads fill
-                // the compute units once (256 heads: 0.84 - 0.96; 192 or 384 heads: 0.90 - 1.13).  Blocks and block
-                // counts of at most 32 (16 waves per workgroup; 64-row blocks at eight waves: 0.84 - 1.17).
-                if (p->D <= 80 && p->B <= 32 && M <= 32 && (p->T >= 2 ? heads >= 192 : (heads >= 224 && heads <= 256)) &&
-                    !resident_head_fits(p, 1) && resident_head_fits(p, 2))
-                    return MA_VARIANT_RESIDENT;
-                if (p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= 128 && resident_fits(p, false))
+                // heads: from 192 heads on (0.63 - 0.92 of the next best variant's time at 192 .. 768 heads with T = 2, 3;
+                // 0.71 - 1.02 with a single step), and with more than one step from 128 heads on for heads of 448 tokens
+                // and more that are a single strip one way (0.86 - 0.95; others 0.97 - 1.17).  Blocks and block counts
+                // of at most 32 (16 waves per workgroup; 64-row blocks at eight waves: 0.89 - 1.22).  Head dims above
+                // 80 (256 .. 320 tokens at D = 128): 16-row blocks of 256 tokens like the others (0.79 - 0.93), else only
+                // where the heads come in whole passes over the compute units (0.82 - 0.97; 192 or 384 heads: 1.03 - 1.24).
+                {
+                    const long long Np = M * p->B;
+                    bool enough = heads >= 192 || (p->T >= 2 && heads >= 128 && Np >= 448 && (M <= 16 || p->B <= 16));
+                    if (p->D > 80) enough = (heads >= 192 && Np <= 256 && p->B <= 16) || (heads >= 224 && heads <= 256) || heads >= 448;
+                    if (p->B <= 32 && M <= 32 && enough && !resident_head_fits(p, 1) && resident_head_fits(p, 2)) return MA_VARIANT_RESIDENT;
+                    // (blocks of 33 .. 64 rows, eight waves per workgroup: one pass of 256 heads, 0.88 - 0.91 at T = 2, 3)
+                    if (p->D <= 80 && p->B <= 64 && M <= 64 && p->T >= 2 && heads >= 224 && heads <= 256 && !resident_head_fits(p, 1) &&
+                        resident_head_fits(p, 2))
+                        return MA_VARIANT_RESIDENT;
+                }
+                if (p->D <= 80 && p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= 128 && resident_fits(p, false))   // (D = 128: 1.07 - 1.37)
                     return MA_VARIANT_RESIDENT;
                 if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D > 48 && p->D <= 64 &&   // (D = 48: 1.12 - 1.19 of the chained kernel's time)
                     ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))

@@ -213,8 +213,10 @@ struct HeadRes {
     // fp32.  For f16 with a scale that is an f16 value itself (1 / sqrt(D) is for D = 4^n) both roundings
     // and the multiplication run two values per instruction: the product of two f16 values rounded to f16
     // is what the fp32 multiplication followed by the rounding gives.
+    // (PACK = false leaves the two-value form out: its second code path costs the two-tile kernel registers it does not have)
+    template <bool PACK = true>
     static __device__ __forceinline__ void lds_store_row_scaled(T* row, const f32x4 (&O)[DT], int q, float sm_scale, bool scale_is_f16) {
-        if constexpr (std::is_same<T, f16>::value && DT % 2 == 0) {
+        if constexpr (PACK && std::is_same<T, f16>::value && DT % 2 == 0) {
             typedef _Float16 h2 __attribute__((ext_vector_type(2)));
             if (scale_is_f16) {   // uniform
                 const _Float16 s = static_cast<_Float16>(sm_scale);
@@ -358,7 +360,7 @@ struct HeadRes {
             pack_p<T, NTB>(pb, C);
             f32x4 O[DT];
             gemm2_rows<NTB, true>(O, c, Kt, RB, ROWSB, pb);
-            lds_store_row_scaled(ok ? c.row(c.L.S, m, j) : c.at(c.L.TR), O, q, P.sm_scale, scale_is_f16);
+            lds_store_row_scaled<!TWO>(ok ? c.row(c.L.S, m, j) : c.at(c.L.TR), O, q, P.sm_scale, scale_is_f16);
         }
         if constexpr (TWO) {
             if (with_v) {   // uniform

@@ -103,6 +103,7 @@ int launch_resident_head2_ni(const Problem& P, bool dry_run, hipStream_t s) {
 }
 template <class T, int DT, int NTB, int NTM>
 int launch_resident_head2(const Problem& P, bool dry_run, hipStream_t s) {
+    // (16 waves on 64-row blocks spill ~20 registers: 0.91 of the eight-wave time for few heads, 1.02 - 1.08 from 128 heads on)
     constexpr int W = (NTB <= 2 && NTM <= 2) ? 16 : 8;
     // 4096 or 5120 16-byte chunks per tile (the larger covers every tile that fits the LDS twice)
     const int err = launch_resident_head2_ni<T, DT, NTB, NTM, W, 4096 / (64 * W)>(P, dry_run, s);

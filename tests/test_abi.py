@@ -163,8 +163,7 @@ def test_kernel_name_follows_the_resolved_variant():
     assert name(1, 16, 4096, 64, 64, flags=L.MA_FLAG_DEVICE_EXCLUSIVE) == "fused_fwd_mfma"
     assert name(64, 12, 197, 64, 16) == "resident_head_mfma"      # the head fits in LDS with its inputs
     assert name(16, 12, 512, 64, 32) == "resident_head2_mfma"     # twice that length: the state and one input tile at a time
-    assert name(16, 16, 512, 64, 32, T=1) == "resident_head2_mfma"   # a single step: only where the heads fill the compute units once
-    assert name(16, 12, 512, 64, 32, T=1) == "chain_fwd_mfma"
+    assert name(16, 12, 512, 64, 32, T=1) == "resident_head2_mfma"
     assert name(8, 12, 512, 64, 32) == "chain_fwd_mfma"           # ... 96 heads do not fill the device
     assert name(16, 12, 1000, 32, 32, variant="resident") == "resident_fwd_mfma"   # state only
     assert name(1, 16, 4096, 64, 256) == "r_step_mfma"
@@ -237,8 +236,13 @@ def test_auto_variant_policy():
     assert auto(16, 12, 512, 64, 32) == "resident"     # 512-token heads: the state and one input tile at a time in LDS
     assert auto(8, 12, 512, 64, 32) == "chained"       # ... when there are enough heads for the compute units (a head has one to itself)
     assert auto(32, 12, 512, 64, 32) == "resident"     # (384 heads, 1.5 passes over 256 CUs: still 0.85 of the chained kernel's time)
-    assert auto(16, 12, 512, 64, 32, T=1) == "chained" # a single step: only where the heads fill the compute units once
-    assert auto(16, 16, 512, 64, 32, T=1) == "resident"
+    assert auto(16, 12, 512, 64, 32, T=1) == "resident"
+    assert auto(8, 16, 512, 64, 32) == "resident"      # 128 heads: for long heads that are a single strip one way
+    assert auto(8, 16, 500, 64, 24) == "chained"
+    assert auto(8, 16, 512, 64, 32, T=1) == "chained"
+    assert auto(8, 24, 256, 128, 16) == "resident"     # head dim 128: 256 tokens are a two-tile head
+    assert auto(8, 24, 272, 128, 16) == "chained"      # ... longer ones only in whole passes over the compute units
+    assert auto(8, 32, 272, 128, 16) == "resident"
     assert auto(16, 12, 512, 64, 64) == "chained"      # 64-row blocks (eight waves per workgroup)
     assert auto(16, 12, 768, 64, 32) == "chained"      # beyond two tiles: the one-tile form is no match for the chained kernel here
     assert auto(16, 12, 512, 64, 64) == "chained"      # ... and for problems of one or two strips
