@@ -48,6 +48,20 @@ struct Problem {
     unsigned* host_error;
 };
 
+// First statement of a kernel: one scalar load from every 64-byte line of a by-value kernel argument, all in flight
+// together.  The scalar cache starts every launch cold, and a kernel that reads its arguments where it needs them
+// (so that they are not held in registers) pays a miss per line, one after the other, before its first global load
+// is issued.  Measured: the team kernel gains 0.8 us per launch (17.9 -> 17.2 us on 16 heads of 4096 tokens); the
+// chained, resident and per-stage kernels measure the same or 0.2 - 0.3 us slower with it and do not call it.
+template <class A>
+__device__ __forceinline__ void warm_args(const A& a) {
+    const unsigned* w = reinterpret_cast<const unsigned*>(&a);
+    unsigned acc = 0;
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(A) / 4; i += 16) acc |= w[i];
+    asm volatile("" ::"s"(acc));
+}
+
 // Raise the sticky error word of the one-launch kernels: in the sync area of the workspace, and in the
 // caller's host-visible word if there is one.
 __device__ __forceinline__ void raise_error(unsigned* error, unsigned* host_error, unsigned code) {

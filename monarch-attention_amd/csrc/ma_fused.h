@@ -268,6 +268,8 @@ __device__ __forceinline__ void run_phase(const Problem& P, char* smem, int p, i
 
 template <class T, int DT, int NTB, int NTM, int W>
 __global__ __launch_bounds__(64 * W) void fused_fwd_mfma(Problem P, FusedPlan plan) {
+    warm_args(P);
+    warm_args(plan);
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ unsigned team_word;   // how wave 0's wait ended, for the whole workgroup
     const int wave = wave_id(), lane = threadIdx.x & 63;
