@@ -33,6 +33,7 @@ struct Problem {
     int mask_shift;      // log2 of the mask element size in bytes (ms strides are in elements)
     int mask_float;      // the mask holds floating-point values: -0.0 counts as zero
     int stream_stores;   // state / output rows that are whole 128-byte lines go out as streaming stores
+    int state_agent;     // state written by other workgroups is read with agent-scope loads instead of streaming ones
     // Per-stage launches of heads with few blocks (M <= 8): a 16-row tile of an L / Z problem holds 16 >> pack_shift
     // in-block positions of pack_m = 1 << pack_shift rows each (4: one position per tile, as everywhere else).
     int pack_shift;

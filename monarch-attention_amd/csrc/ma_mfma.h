@@ -141,16 +141,19 @@ constexpr unsigned kOob = 0xFFFF0000u;  // beyond any slice (extents are validat
 __device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
 }
-// SHARED = true is for state another workgroup wrote during this launch: a
-// streaming ("nt") load, which is served by L2 and never by a line this CU's L1
-// kept from an earlier step.
-template <bool SHARED>
+// The template argument is a cache policy: 0 / false = ordinary, 1 / true = streaming ("nt"), 2 = agent scope
+// ("sc1").  State that another workgroup wrote during this launch is read with one of the latter two: both are
+// served by the L2 and never by a line this CU's L1 kept from an earlier step.  Which of them is the caller's choice
+// per launch (Slices::agent_state): agent-scope loads keep their lines in the L2 like any other, which pays while
+// the state arrays fit the caches (2 - 6 % on heads x tokens up to ~256 K) and costs 4 - 6 % where they do not.
+constexpr int kPolStream = 1, kPolAgent = 2;
+template <int POL>
 __device__ __forceinline__ u32x4 bload16(rsrc_t r, unsigned off) {
-    return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, SHARED ? 2 : 0);
+    return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, POL == 0 ? 0 : POL == 1 ? 2 : 16);
 }
-template <bool SHARED>
+template <int POL>
 __device__ __forceinline__ float bloadf(rsrc_t r, unsigned off) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, SHARED ? 2 : 0));
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, POL == 0 ? 0 : POL == 1 ? 2 : 16));
 }
 
 // ---- operand tiles ----------------------------------------------------------
@@ -176,7 +179,7 @@ struct TileCopy {
     static constexpr bool EVEN = ROWS * CH % NTH == 0;   // else the last round of chunks is not for every thread
     u32x4 val[CNT];
 
-    template <bool SHARED, class RowOff>
+    template <int SHARED, class RowOff>
     __device__ __forceinline__ void issue(rsrc_t src, int D, RowOff rowoff, int tix) {
 #pragma unroll
         for (int i = 0; i < CNT; ++i) {
@@ -196,7 +199,7 @@ struct TileCopy {
 };
 
 // B operand of GEMM1 straight from memory: the row at byte offset ro (or kOob)
-template <class T, int DT, bool SHARED>
+template <class T, int DT, int SHARED>
 __device__ __forceinline__ void load_x(typename Ops<T>::v8 (&x)[Geom<DT>::KS], rsrc_t src, unsigned ro, int D, int q) {
 #pragma unroll
     for (int ks = 0; ks < Geom<DT>::KS; ++ks) {
@@ -346,6 +349,7 @@ struct Slices {
     rsrc_t q, k, v, out, aR, cR, aL, cL, Y, mask;
     unsigned qst, kst, vst, ost, mst;   // mst: byte pitch of the mask's token dimension, 0 = no mask
     bool stream_state, stream_out;      // rows of the state arrays / of out are whole, aligned 128-byte lines
+    bool agent_state;                   // state loads with agent scope instead of the streaming policy (Problem::state_agent)
 };
 
 template <class T>
@@ -371,6 +375,7 @@ __device__ __forceinline__ Slices make_slices(const Problem& P, int e, int h, lo
     S.cL = make_rsrc(P.cL + wh * np, stat4);
     // the state arrays are 256-byte aligned (workspace layout) with rows of db bytes
     S.stream_state = P.stream_stores != 0 && db % 128u == 0;
+    S.agent_state = P.state_agent != 0;
     S.stream_out = P.stream_stores != 0 && db % 128u == 0 && S.ost % 128u == 0 &&
                    (reinterpret_cast<unsigned long long>(P.out) + static_cast<unsigned long long>(e * P.os[0] + h * P.os[1]) * sizeof(T)) % 128u == 0;
     return S;
@@ -489,13 +494,14 @@ struct RProb {
         pre.vc.template issue<NT>(S.v, P.D, [&](int i) { return i < B ? tok_off(t0 + i, P.N, S.vst) : kOob; }, wig * 64 + lane);
     }
 
+    template <int POL>
     static __device__ __forceinline__ void load_state_strip(const Problem& P, const Slices& S, V8 (&xa)[G::KS], float& cr, int m,
                                                             int strip, int lane) {
         const int j = 16 * strip + (lane & 15);
         const unsigned rowid = static_cast<unsigned>(m * P.B + j);   // row inside the head's state
         const unsigned db = static_cast<unsigned>(P.D) * sizeof(T);
-        load_x<T, DT, true>(xa, S.aR, j < P.B ? rowid * db : kOob, P.D, lane >> 4);
-        cr = bloadf<true>(S.cR, j < P.B ? rowid * 4u : kOob);   // an out-of-range row reads 0: harmless, never stored
+        load_x<T, DT, POL>(xa, S.aR, j < P.B ? rowid * db : kOob, P.D, lane >> 4);
+        cr = bloadf<POL>(S.cR, j < P.B ? rowid * 4u : kOob);   // an out-of-range row reads 0: harmless, never stored
     }
 
     static __device__ __forceinline__ void state(const Problem& P, const Slices& S, St& st, bool active, int m, bool first, int wig,
@@ -503,7 +509,10 @@ struct RProb {
 #pragma unroll
         for (int i = 0; i < SPW; ++i) {
             st.cr[i] = 1.0f;
-            if (active && !first) load_state_strip(P, S, st.xa[i], st.cr[i], m, strip_of(wig, i, half), lane);
+            if (active && !first) {
+                if (S.agent_state) load_state_strip<kPolAgent>(P, S, st.xa[i], st.cr[i], m, strip_of(wig, i, half), lane);   // uniform
+                else load_state_strip<kPolStream>(P, S, st.xa[i], st.cr[i], m, strip_of(wig, i, half), lane);
+            }
         }
     }
 
@@ -660,9 +669,19 @@ struct ZProb {
         const unsigned db = static_cast<unsigned>(D) * sizeof(T);
         const TileIndex<NWT> ti(P, j);
         // the Y tile (needed last) last
-        st.ac.template issue<true>(S.aL, D, [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; }, tix);
-        st.cbv = (tix < ROWS && ti.ok(P, tix)) ? -kLog2e * bloadf<true>(S.cL, ti.state_row(P, tix) * 4u) : kNegBig;
-        st.yc.template issue<true>(S.Y, D, [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; }, tix);
+        const auto rowoff = [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; };
+        const unsigned cloff = (tix < ROWS && ti.ok(P, tix)) ? ti.state_row(P, tix) * 4u : kOob;
+        float clv;
+        if (S.agent_state) {   // uniform
+            st.ac.template issue<kPolAgent>(S.aL, D, rowoff, tix);
+            clv = bloadf<kPolAgent>(S.cL, cloff);
+            st.yc.template issue<kPolAgent>(S.Y, D, rowoff, tix);
+        } else {
+            st.ac.template issue<kPolStream>(S.aL, D, rowoff, tix);
+            clv = bloadf<kPolStream>(S.cL, cloff);
+            st.yc.template issue<kPolStream>(S.Y, D, rowoff, tix);
+        }
+        st.cbv = (tix < ROWS && ti.ok(P, tix)) ? -kLog2e * clv : kNegBig;
     }
     static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
                                                int j, int wig, int lane, int half = 0) {
@@ -802,8 +821,17 @@ struct LProb {
         const int tix = wig * 64 + lane;
         const unsigned db = static_cast<unsigned>(D) * sizeof(T);
         const TileIndex<NWT> ti(P, j);
-        st.ac.template issue<true>(S.aL, D, [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; }, tix);
-        st.cbv = (tix < ROWS && ti.ok(P, tix)) ? -kLog2e * bloadf<true>(S.cL, ti.state_row(P, tix) * 4u) : kNegBig;
+        const auto rowoff = [&](int k) { return ti.ok(P, k) ? ti.state_row(P, k) * db : kOob; };
+        const unsigned cloff = (tix < ROWS && ti.ok(P, tix)) ? ti.state_row(P, tix) * 4u : kOob;
+        float clv;
+        if (S.agent_state) {   // uniform
+            st.ac.template issue<kPolAgent>(S.aL, D, rowoff, tix);
+            clv = bloadf<kPolAgent>(S.cL, cloff);
+        } else {
+            st.ac.template issue<kPolStream>(S.aL, D, rowoff, tix);
+            clv = bloadf<kPolStream>(S.cL, cloff);
+        }
+        st.cbv = (tix < ROWS && ti.ok(P, tix)) ? -kLog2e * clv : kNegBig;
     }
     static __device__ __forceinline__ void run(const Problem& P, const Slices& S, char* smem, const Pre& pre, const St& st, bool active,
                                                int j, int wig, int lane) {
