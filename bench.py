@@ -100,7 +100,7 @@ def record_traffic(args) -> None:
     every forward kernel times the kernels one forward launches."""
     fetch_csv, write_csv = args.record_traffic
 
-    names = ("r_step_mfma", "l_step_mfma", "z_step_mfma", "fused_fwd_mfma", "chain_fwd_mfma", "resident_fwd_mfma", "resident_head_mfma",
+    names = ("r_step_mfma", "l_step_mfma", "z_step_mfma", "fused_fwd_mfma", "chain_fwd_mfma", "resident_fwd_mfma", "resident_head_mfma", "resident_head2_mfma",
              "r_step_f32", "l_step_f32", "z_step_f32", "head_fwd_f32", "head_t1_f32")
 
     def per_kernel(path, counter):
@@ -120,7 +120,7 @@ def record_traffic(args) -> None:
     # launches of each kernel in one forward (the bench also launches single stages for the per-stage timings:
     # the per-dispatch means make that irrelevant)
     per_fwd = {"r_step_mfma": T, "l_step_mfma": T - 1, "z_step_mfma": 1, "fused_fwd_mfma": 1, "chain_fwd_mfma": 1, "resident_fwd_mfma": 1,
-               "resident_head_mfma": 1, "r_step_f32": T, "l_step_f32": T - 1, "z_step_f32": 1, "head_fwd_f32": 1, "head_t1_f32": 1}
+               "resident_head_mfma": 1, "resident_head2_mfma": 1, "r_step_f32": T, "l_step_f32": T - 1, "z_step_f32": 1, "head_fwd_f32": 1, "head_t1_f32": 1}
     kernels, total = {}, 0.0
     for name in sorted(set(fetch) & set(write)):
         rd, wr = fetch[name][0] * 1024 * FETCH_SIZE_FACTOR, write[name][0] * 1024

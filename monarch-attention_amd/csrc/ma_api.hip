@@ -465,11 +465,16 @@ int prepare(const ma_fwd_params* p, Prepared* out) {
     out->P.stream_stores = v == MA_VARIANT_STAGED && p->dtype_qk != MA_F32 && p->B > 32 && out->P.M > 32 &&
                            static_cast<long long>(p->E) * p->H * out->P.M * p->B <= 128 * 1024;
     out->P.pack_shift = pack_shift_of(v, p, out->P.M);
-    // Agent-scope state loads keep the state's lines in the L2 (streaming loads give them up first): the per-stage and
-    // chained kernels gain 1 - 4 % while one state array is at most 48 MB (heads x tokens x D at 16 bits), and lose
-    // 4 - 6 % beyond; the team kernel is faster with streaming loads (17.2 against 18.0 us on the metric workload).
-    out->P.state_agent = (v == MA_VARIANT_STAGED || v == MA_VARIANT_CHAINED) && p->dtype_qk != MA_F32 &&
-                         static_cast<long long>(p->E) * p->H * out->P.M * p->B * p->D * 2 <= (48ll << 20);
+    // Agent-scope state loads keep the state's lines in the L2 (streaming loads give them up first).  Measured over
+    // heads x tokens grids at T = 1, 2, 3, by the size of one state array (heads x tokens x D at 16 bits): the chained
+    // kernel gains 2 - 3 % at 6 .. 24 MB, nothing below, 1 % up to 64 MB and loses 3 - 4 % from 128 MB on; the per-stage
+    // launches gain 2 - 5 % up to 1.5 MB and lose up to 8 % at 3 .. 12 MB (a single step most); the team kernel is
+    // faster with streaming loads (17.2 against 18.0 us on the metric workload).
+    {
+        const long long state_bytes = static_cast<long long>(p->E) * p->H * out->P.M * p->B * p->D * 2;
+        out->P.state_agent = p->dtype_qk != MA_F32 && ((v == MA_VARIANT_CHAINED && state_bytes >= (6ll << 20) && state_bytes <= (64ll << 20)) ||
+                                                       (v == MA_VARIANT_STAGED && state_bytes <= (3ll << 19)));
+    }
     out->P.one_tile_ok = 1;   // a problem that resolves to the resident kernel may use any of its forms
     return MA_OK;
 }
