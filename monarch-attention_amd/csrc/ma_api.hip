@@ -344,15 +344,20 @@ int select_variant(const ma_fwd_params* p) {
                 // where the heads come in whole passes over the compute units (0.82 - 0.97; 192 or 384 heads: 1.03 - 1.24).
                 {
                     const long long Np = M * p->B;
-                    bool enough = heads >= 192 || (p->T >= 2 && heads >= 128 && Np >= 448 && (M <= 16 || p->B <= 16));
-                    if (p->D > 80) enough = (heads >= 192 && Np <= 256 && p->B <= 16) || (heads >= 224 && heads <= 256) || heads >= 448;
+                    bool enough = heads >= 192 || (p->T >= 2 && heads >= 128 && Np >= 448 && (M <= 16 || p->B <= 16) && p->D > 48);
+                    // (head dims of 65 .. 80, measured at 72: a single step 1.24 - 1.35, one and a half passes over the compute
+                    // units 1.06 - 1.12)
+                    if (p->D > 64 && p->D <= 80 && (p->T == 1 || (heads > 256 && heads < 448))) enough = false;
+                    if (p->D > 80) enough = (heads >= 192 && heads <= 256 && Np <= 256 && p->B <= 16) || (heads >= 224 && heads <= 256) || heads >= 448;
                     if (p->B <= 32 && M <= 32 && enough && !resident_head_fits(p, 1) && resident_head_fits(p, 2)) return MA_VARIANT_RESIDENT;
                     // (blocks of 33 .. 64 rows, eight waves per workgroup: one pass of 256 heads, 0.88 - 0.91 at T = 2, 3)
                     if (p->D <= 80 && p->B <= 64 && M <= 64 && p->T >= 2 && heads >= 224 && heads <= 256 && !resident_head_fits(p, 1) &&
                         resident_head_fits(p, 2))
                         return MA_VARIANT_RESIDENT;
                 }
-                if (p->D <= 80 && p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= 128 && resident_fits(p, false))   // (D = 128: 1.07 - 1.37)
+                // (D = 128: 1.07 - 1.37; D = 72: a single step 1.2 - 1.35, 128 heads 1.03 - 1.16)
+                if (p->D <= 80 && p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= (p->D > 64 ? 192 : 128) && !(p->D > 64 && p->T == 1) &&
+                    resident_fits(p, false))
                     return MA_VARIANT_RESIDENT;
                 if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D > 48 && p->D <= 64 &&   // (D = 48: 1.12 - 1.19 of the chained kernel's time)
                     ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))
@@ -378,7 +383,8 @@ int select_variant(const ma_fwd_params* p) {
                 // more, or 128-row problems on many tokens in total (4 - 16 % behind the stage launches there)
                 const bool wide_dim = p->D > 80 && ((M > 64 && p->B >= 64) || ((p->B > 96 || M > 96) && heads * p->N >= 393216));
                 const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
-                const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 7168));
+                // (a single step of at most 4 heads from 1024 tokens on: two launches, 3 - 19 % ahead)
+                const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 7168) || (heads <= 4 && p->N >= 1024));
                 // launches that leave most of the device empty: the stage kernels run their 6- and 8-strip R and Z
                 // problems as two workgroups each then (halves_pay), which the one-launch kernels do not
                 const bool rows_halve = p->B > 64 && p->B <= 128, blocks_halve = M > 64 && M <= 128;
