@@ -582,6 +582,7 @@ __global__ __launch_bounds__(64 * W) void resident_head_mfma(Problem P) {
     for (int i = c.tid; i < P.B * HR::ROWSM; i += HR::NT) c.fat(c.L.cb)[i] = kNegBig;
     // (the state rows are written 16*DT columns wide but read as GEMM operands over all 32*KS columns: for head
     // dims of 65..80 the columns in between are never written and keep those zeros)
+    __syncthreads();   // no wave writes a tile row before every wave's zeros are in
 
     const int heads = P.E * P.H, stride = static_cast<int>(gridDim.x);
     int head = static_cast<int>(blockIdx.x);
