@@ -297,10 +297,104 @@ bool device_exclusive(const ma_fwd_params* p) {
     return env || (p->flags & MA_FLAG_DEVICE_EXCLUSIVE) != 0;
 }
 
+// ---- AUTO: which variant is the fastest for a problem.  Every threshold below is read off the sweeps of
+// bench.py --sweep-variants (each variant that takes a shape timed through this ABI); the figures in the comments are
+// time ratios against the next best variant.
+
+// fp32: heads of up to 16 blocks of up to 16 rows can run whole in one workgroup each (one launch, no state in
+// memory).  A head then has one compute unit to itself, which pays from 64 heads on (256 tokens x 64: 0.93 of the
+// stage launches' time at 96 heads, 0.5 - 0.7 from 192 on, also beyond one pass over the compute units) and for any
+// head count when the head is small (128 tokens x 32: 0.45 - 0.8); few large heads are faster spread over many
+// compute units by the stage launches (one head of 256 x 64, two steps: 16.6 us against 20.4) - unless there is a
+// single step: then a workgroup per (head, position) needs nothing from any other (one head of 256 x 64: 5.3 us
+// against 7.9 as two launches; 16 heads: 6.7 against 10.3).
+int auto_fp32(const ma_fwd_params* p, long long heads, long long M) {
+    const bool single_step = p->T == 1 && heads * p->B <= kHead32T1MaxGroups;
+    const bool pays = heads >= 64 || M * p->B * p->D <= 4096 || single_step;
+    return pays && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_VARIANT_STAGED;
+}
+
+// 16-bit: does one of the forms of the resident kernel (a whole head per workgroup) win?
+bool auto_resident(const ma_fwd_params* p, long long heads, long long M) {
+    const long long Np = M * p->B;
+    // Heads that fit in LDS whole - Q, K, V and the state in four tiles -, in blocks and block counts of at most two
+    // strips (16 waves): every input is read once and no state leaves the compute unit.  From 96 heads on (0.63 - 0.93
+    // at T = 1, 2, 3), and with more than one step also for any number of heads of at most 256 tokens in 16-row
+    // blocks (0.85 - 0.95 at 256 tokens, 0.55 - 0.8 for shorter heads and three steps; longer heads at D = 32: 1.2 - 1.4
+    // below 64 heads; a single step of few heads: 1.03 - 1.23, they stay away).  Head dims up to 64: in the 128-column
+    // class the kernel holds heads of ~128 tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
+    if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= 96 || (p->T >= 2 && p->B <= 16 && Np <= 256)) && resident_head_fits(p)) return true;
+    // Heads of about twice that length (257 .. ~540 tokens at D = 64) keep the state and ONE input tile at a time in
+    // LDS.  A head has a compute unit to itself for its 2T phases, so the device has to be full of heads: from 192
+    // heads on (0.63 - 0.92 at 192 .. 768 heads with T = 2, 3; 0.71 - 1.02 with a single step), and with more than one
+    // step from 128 heads on for heads of 448 tokens and more that are a single strip one way (0.86 - 0.95; others
+    // 0.97 - 1.17; D = 48: 1.11 - 1.16).  Blocks and block counts of at most 32 (16 waves per workgroup).
+    const bool two_tiles = !resident_head_fits(p, 1) && resident_head_fits(p, 2);
+    if (two_tiles && p->B <= 32 && M <= 32) {
+        bool enough = heads >= 192 || (p->T >= 2 && heads >= 128 && Np >= 448 && (M <= 16 || p->B <= 16) && p->D > 48);
+        // head dims of 65 .. 80 (measured at 72): a single step 1.24 - 1.35, one and a half passes over the compute units 1.06 - 1.12
+        if (p->D > 64 && p->D <= 80 && (p->T == 1 || (heads > 256 && heads < 448))) enough = false;
+        // head dims above 80 (256 .. 288 tokens at D = 128): 256 tokens in 16-row blocks 0.79 - 0.87 for 192 .. 256 heads, else
+        // only where the heads come in whole passes over the compute units (0.82 - 0.97; 192 or 384 heads: 1.03 - 1.24)
+        if (p->D > 80) enough = (heads >= 192 && heads <= 256 && Np <= 256 && p->B <= 16) || (heads >= 224 && heads <= 256) || heads >= 448;
+        if (enough) return true;
+    }
+    // ... in blocks of 33 .. 64 rows (eight waves per workgroup: 0.89 - 1.22): one pass of 256 heads, 0.88 - 0.91 at T = 2, 3
+    if (two_tiles && p->D <= 80 && p->B <= 64 && M <= 64 && p->T >= 2 && heads >= 224 && heads <= 256) return true;
+    // Many short heads in 16-row blocks, whichever form takes them (D = 128: 1.07 - 1.37; D = 72: a single step
+    // 1.2 - 1.35, 128 heads 1.03 - 1.16)
+    if (p->D <= 80 && p->B <= 16 && M <= 32 && Np <= 288 && heads >= (p->D > 64 ? 192 : 128) && !(p->D > 64 && p->T == 1) &&
+        resident_fits(p, false))
+        return true;
+    // The one-tile form (aL and aR in one tile, inputs streamed, Y through the workspace) where the heads fill its
+    // one-workgroup-per-CU passes (D = 48: 1.12 - 1.19 of the chained kernel's time)
+    return heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D > 48 && p->D <= 64 &&
+           ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true);
+}
+
+// 16-bit: the team kernel - only for callers that own the device (its workgroups wait for each other).
+bool auto_fused(const ma_fwd_params* p, long long heads, long long M) {
+    if (!device_exclusive(p)) return false;
+    if (fused_full_width(p)) return true;
+    // Head dims of 65 .. 80 (the 80-column tile class; measured at 72) with 128-row problems - blocks or block counts of
+    // 97 .. 128 - and more than one step: 8 - 21 % ahead of the chained kernel for 6 .. 128 heads of thousands of tokens
+    // (from 2048 tokens on with 32 heads and more, 4096 below that)
+    const bool wide5 = p->D > 64 && p->D <= 80, class128 = (M > 96 || p->B > 96) && one_launch_tiles(p);
+    return wide5 && class128 && p->T >= 2 && heads >= 6 && heads <= 128 && p->N >= (heads >= 32 ? 2048 : 4096);
+}
+
+// 16-bit: do the per-stage launches beat the chained kernel?
+bool auto_staged(const ma_fwd_params* p, long long heads, long long M) {
+    // head dims of 65 .. 80 with 128-row blocks on 192 heads and more, T >= 2: 4 - 15 % ahead
+    if (p->D > 64 && p->D <= 80 && (M > 96 || p->B > 96) && one_launch_tiles(p) && p->T >= 2 && heads >= 192 && p->B > 96 && M >= 4) return true;
+    const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
+    // 128-row blocks in 33 .. 48 blocks (three-strip L / Z problems beside eight-strip R problems) on a head count that
+    // does not divide by 8, or on very many heads: 12 / 192 heads of 5000 tokens are 7 - 21 % behind the stage launches
+    // in the chained kernel (16 .. 96 heads: 9 - 23 % ahead)
+    const bool odd_mix = p->B > 96 && M > 32 && M <= 48 && (heads % 8 != 0 || heads >= 192);
+    // head dims above 80 (the 128-column class; measured at 96 and 128): many blocks of 64 rows and more, or 128-row
+    // problems on many tokens in total (4 - 16 % behind the stage launches there)
+    const bool wide_dim = p->D > 80 && ((M > 64 && p->B >= 64) || ((p->B > 96 || M > 96) && heads * p->N >= 393216));
+    // fewer than 8 long heads: a head is pinned to one XCD by the chained kernel
+    const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
+    // a single step: head counts that do not sit evenly on the XCDs, few very long heads, and at most 4 heads from 1024
+    // tokens on (two launches, 3 - 19 % ahead)
+    const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 7168) || (heads <= 4 && p->N >= 1024));
+    // launches that leave most of the device empty: the stage kernels run their 6- and 8-strip R and Z problems as two
+    // workgroups each then (halves_pay), which the one-launch kernels do not
+    const bool rows_halve = p->B > 64 && p->B <= 128, blocks_halve = M > 64 && M <= 128;
+    const long long r_problems = heads * M;
+    const bool underfilled = (rows_halve && (p->T == 1 ? (r_problems <= 160 || (heads <= 8 && r_problems <= 512))
+                                                       : p->B > 96 && (r_problems <= 48 || (heads <= 4 && p->N <= 4096)))) ||
+                             (blocks_halve && p->T == 1 && heads * p->B <= 128);
+    return uneven_128 || odd_mix || wide_dim || few_heads || one_step || underfilled || !chain_fits(p);
+}
+
 int select_variant(const ma_fwd_params* p) {
     const bool fast = mfma_supported(p);
-    const bool fast32 = mfma32_supported(p);   // fp32 operands: per-stage launches only
+    const bool fast32 = mfma32_supported(p);   // fp32 operands: per-stage launches and the one-launch head kernels
     const long long heads = static_cast<long long>(p->E) * p->H;
+    const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
     switch (p->variant) {
         case MA_VARIANT_GENERIC: return MA_VARIANT_GENERIC;
         case MA_VARIANT_STAGED: return fast || fast32 ? MA_VARIANT_STAGED : MA_ERR_UNSUPPORTED;
@@ -308,95 +402,11 @@ int select_variant(const ma_fwd_params* p) {
         case MA_VARIANT_CHAINED: return fast && chain_fits(p) ? MA_VARIANT_CHAINED : MA_ERR_UNSUPPORTED;
         case MA_VARIANT_RESIDENT: return (fast || fast32) && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_ERR_UNSUPPORTED;
         default:
-            // fp32: heads of up to 16 blocks of up to 16 rows can run whole in one workgroup each (one launch, no
-            // state in memory).  A head then has one compute unit to itself, which pays from 64 heads on
-            // (256 tokens x 64: 0.93 of the stage launches' time at 96 heads, 0.5 - 0.7 from 192 on, also
-            // beyond one pass over the compute units) and for any head count when the head is small
-            // (128 tokens x 32: 0.45 - 0.8); few large heads are faster spread over many compute units
-            // by the stage launches (one head of 256 x 64, two steps: 16.6 us against 20.4) - unless there is a
-            // single step: then a workgroup per (head, position) needs nothing from any other (one head of
-            // 256 x 64: 5.3 us against 7.9 as two launches; 16 heads: 6.7 against 10.3).
-            if (fast32) {
-                const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-                const bool single_step = p->T == 1 && heads * p->B <= kHead32T1MaxGroups;
-                const bool pays = heads >= 64 || M * p->B * p->D <= 4096 || single_step;
-                return pays && resident_fits(p, true) ? MA_VARIANT_RESIDENT : MA_VARIANT_STAGED;
-            }
+            if (fast32) return auto_fp32(p, heads, M);
             if (!fast) return MA_VARIANT_GENERIC;
-            {
-                const long long M = (static_cast<long long>(p->N) + p->B - 1) / p->B;
-                // heads that fit in LDS whole, in blocks and block counts of at most two strips (16 waves): every
-                // input is read once and no state leaves the compute unit.  From 96 heads on (0.63 - 0.93 of
-                // the next best variant's time at T = 1, 2, 3), and with more than one step also for any number of
-                // heads of at most 256 tokens in 16-row blocks (0.85 - 0.95 at 256 tokens, 0.55 - 0.8 for shorter heads
-                // and three steps; longer heads at D = 32: 1.2 - 1.4 below 64 heads; a single step of few heads: 1.03 -
-                // 1.23, they stay away).  Head dims up to 64: in the 128-column class the kernel holds heads of ~128
-                // tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
-                if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= 96 || (p->T >= 2 && p->B <= 16 && M * p->B <= 256)) && resident_head_fits(p))
-                    return MA_VARIANT_RESIDENT;
-                // Heads of about twice that length (257 .. ~540 tokens at D = 64) keep the state and ONE input tile at a
-                // time in LDS.  A head has a compute unit to itself for its 2T phases, so the device has to be full of
-                // heads: from 192 heads on (0.63 - 0.92 of the next best variant's time at 192 .. 768 heads with T = 2, 3;
-                // 0.71 - 1.02 with a single step), and with more than one step from 128 heads on for heads of 448 tokens
-                // and more that are a single strip one way (0.86 - 0.95; others 0.97 - 1.17).  Blocks and block counts
-                // of at most 32 (16 waves per workgroup; 64-row blocks at eight waves: 0.89 - 1.22).  Head dims above
-                // 80 (256 .. 320 tokens at D = 128): 16-row blocks of 256 tokens like the others (0.79 - 0.93), else only
-                // where the heads come in whole passes over the compute units (0.82 - 0.97; 192 or 384 heads: 1.03 - 1.24).
-                {
-                    const long long Np = M * p->B;
-                    bool enough = heads >= 192 || (p->T >= 2 && heads >= 128 && Np >= 448 && (M <= 16 || p->B <= 16) && p->D > 48);
-                    // (head dims of 65 .. 80, measured at 72: a single step 1.24 - 1.35, one and a half passes over the compute
-                    // units 1.06 - 1.12)
-                    if (p->D > 64 && p->D <= 80 && (p->T == 1 || (heads > 256 && heads < 448))) enough = false;
-                    if (p->D > 80) enough = (heads >= 192 && heads <= 256 && Np <= 256 && p->B <= 16) || (heads >= 224 && heads <= 256) || heads >= 448;
-                    if (p->B <= 32 && M <= 32 && enough && !resident_head_fits(p, 1) && resident_head_fits(p, 2)) return MA_VARIANT_RESIDENT;
-                    // (blocks of 33 .. 64 rows, eight waves per workgroup: one pass of 256 heads, 0.88 - 0.91 at T = 2, 3)
-                    if (p->D <= 80 && p->B <= 64 && M <= 64 && p->T >= 2 && heads >= 224 && heads <= 256 && !resident_head_fits(p, 1) &&
-                        resident_head_fits(p, 2))
-                        return MA_VARIANT_RESIDENT;
-                }
-                // (D = 128: 1.07 - 1.37; D = 72: a single step 1.2 - 1.35, 128 heads 1.03 - 1.16)
-                if (p->D <= 80 && p->B <= 16 && M <= 32 && M * p->B <= 288 && heads >= (p->D > 64 ? 192 : 128) && !(p->D > 64 && p->T == 1) &&
-                    resident_fits(p, false))
-                    return MA_VARIANT_RESIDENT;
-                if (heads >= 128 && (heads % 256 == 0 || heads % 256 >= 192) && p->D > 48 && p->D <= 64 &&   // (D = 48: 1.12 - 1.19 of the chained kernel's time)
-                    ((p->B <= 32 && M <= 16) || (p->B <= 16 && M <= 32)) && !resident_fits(p, false) && resident_fits(p, true))
-                    return MA_VARIANT_RESIDENT;
-                if (device_exclusive(p) && fused_full_width(p)) return MA_VARIANT_FUSED;
-                // Head dims of 65 .. 80 (the 80-column tile class; measured at 72) with 128-row problems - blocks or
-                // block counts of 97 .. 128 - and more than one step: the team kernel is 8 - 21 % ahead of the chained
-                // kernel for 6 .. 128 heads of thousands of tokens (from 2048 tokens on with 32 heads and more, 4096
-                // below that), the stage launches 4 - 15 % for 192 heads and more in 128-row blocks.
-                {
-                    const bool wide5 = p->D > 64 && p->D <= 80, class128 = (M > 96 || p->B > 96) && one_launch_tiles(p);
-                    if (wide5 && class128 && p->T >= 2) {
-                        if (device_exclusive(p) && heads >= 6 && heads <= 128 && p->N >= (heads >= 32 ? 2048 : 4096)) return MA_VARIANT_FUSED;
-                        if (heads >= 192 && p->B > 96 && M >= 4) return MA_VARIANT_STAGED;
-                    }
-                }
-                const bool uneven_128 = p->B > 96 && M > 96 && heads % 8 != 0;
-                // 128-row blocks in 33 .. 48 blocks (three-strip L / Z problems beside eight-strip R problems) on a head
-                // count that does not divide by 8, or on very many heads: 12 / 192 heads of 5000 tokens are 7 - 21 %
-                // behind the stage launches in the chained kernel (16 .. 96 heads: 9 - 23 % ahead)
-                const bool odd_mix = p->B > 96 && M > 32 && M <= 48 && (heads % 8 != 0 || heads >= 192);
-                // head dims above 80 (the 128-column class; measured at 96 and 128): many blocks of 64 rows and
-                // more, or 128-row problems on many tokens in total (4 - 16 % behind the stage launches there)
-                const bool wide_dim = p->D > 80 && ((M > 64 && p->B >= 64) || ((p->B > 96 || M > 96) && heads * p->N >= 393216));
-                const bool few_heads = heads < 8 && p->N > (heads <= 2 ? 2048 : 4096);
-                // (a single step of at most 4 heads from 1024 tokens on: two launches, 3 - 19 % ahead)
-                const bool one_step = p->T == 1 && ((heads % 8 != 0 && p->N >= 4096) || (heads < 16 && p->N >= 7168) || (heads <= 4 && p->N >= 1024));
-                // launches that leave most of the device empty: the stage kernels run their 6- and 8-strip R and Z
-                // problems as two workgroups each then (halves_pay), which the one-launch kernels do not
-                const bool rows_halve = p->B > 64 && p->B <= 128, blocks_halve = M > 64 && M <= 128;
-                const long long r_problems = heads * M;
-                const bool underfilled =
-                    (rows_halve && (p->T == 1 ? (r_problems <= 160 || (heads <= 8 && r_problems <= 512))
-                                              : p->B > 96 && (r_problems <= 48 || (heads <= 4 && p->N <= 4096)))) ||
-                    (blocks_halve && p->T == 1 && heads * p->B <= 128);
-                if (!uneven_128 && !odd_mix && !wide_dim && !few_heads && !one_step && !underfilled && chain_fits(p))
-                    return MA_VARIANT_CHAINED;
-            }
-            return MA_VARIANT_STAGED;
+            if (auto_resident(p, heads, M)) return MA_VARIANT_RESIDENT;
+            if (auto_fused(p, heads, M)) return MA_VARIANT_FUSED;
+            return auto_staged(p, heads, M) ? MA_VARIANT_STAGED : MA_VARIANT_CHAINED;
     }
 }
 
