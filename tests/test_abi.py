@@ -146,6 +146,41 @@ def test_select_variant_reports_a_known_variant():
     assert lib.ma_fwd_select_variant(p32) in (L.VARIANTS["generic"], L.VARIANTS["staged"], L.VARIANTS["resident"])
 
 
+def test_auto_resolves_to_a_variant_that_takes_the_problem():
+    """Over a random sample of problems: what AUTO resolves to is a variant that accepts the problem when it is asked for
+    by name, the answer does not depend on the device-ownership flag unless it is the team kernel, and a kernel name exists."""
+    import random
+    lib = L.load()
+    rnd = random.Random(11)
+    seen = set()
+    for _ in range(4000):
+        E, H = rnd.choice([1, 1, 2, 3, 4, 8, 16, 32, 64]), rnd.choice([1, 2, 3, 4, 6, 8, 12, 16])
+        B = rnd.choice([8, 14, 16, 24, 32, 45, 48, 64, 80, 96, 128, 160, 256])
+        M = rnd.choice([1, 2, 3, 4, 8, 13, 16, 24, 32, 46, 64, 90, 128, 200])
+        N = max(1, M * B - rnd.randint(0, B - 1))
+        D = rnd.choice([32, 40, 48, 60, 64, 72, 80, 96, 128])
+        if E * H * N * D > 3e8:
+            continue
+        p = good_params()
+        p.E, p.H, p.N, p.D, p.Dv, p.B, p.T = E, H, N, D, D, B, rnd.randint(1, 3)
+        p.dtype_qk = p.dtype_v = rnd.choice([L.MA_F16, L.MA_BF16, L.MA_F32])
+        for field in ("q_stride", "k_stride", "v_stride", "out_stride"):
+            setattr(p, field, (C.c_int64 * 3)(H * N * D, N * D, D))
+        p.variant, p.flags = L.VARIANTS["auto"], 0
+        shared = lib.ma_fwd_select_variant(p)
+        p.flags = L.MA_FLAG_DEVICE_EXCLUSIVE
+        owned = lib.ma_fwd_select_variant(p)
+        assert shared >= 0 and owned >= 0, (E, H, N, D, B)
+        assert shared != L.VARIANTS["fused"]
+        assert owned == shared or owned == L.VARIANTS["fused"], (E, H, N, D, B)
+        assert lib.ma_fwd_kernel_name(p) is not None
+        for v in (shared, owned):
+            p.variant = v
+            assert lib.ma_fwd_select_variant(p) == v, (E, H, N, D, B, v)
+            seen.add(v)
+    assert seen == {L.VARIANTS[n] for n in ("generic", "staged", "fused", "resident", "chained")}
+
+
 def test_kernel_name_follows_the_resolved_variant():
     lib = L.load()
 
