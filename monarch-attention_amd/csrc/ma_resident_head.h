@@ -578,7 +578,10 @@ __global__ __launch_bounds__(64 * W) void resident_head_mfma(Problem P) {
     // once per launch: zeros in the tiles (the gaps between the blocks' rows are never written again, and a
     // 16-row strip of a shorter block reads across them), in the row of zeros; the softmax bias of key
     // blocks that do not exist
-    for (unsigned i = c.tid * 16u; i < c.L.TR; i += HR::NT * 16u) *reinterpret_cast<u32x4*>(smem + i) = u32x4{0u, 0u, 0u, 0u};
+    // (with blocks of exactly 16, 32 or 64 rows no strip reaches across a gap or into the columns behind a row's last, and
+    // with a head dim that fills its tile columns every column a product reads is written first: only the row of zeros then)
+    const bool fill_tiles = HR::ROWSB != P.B || (DT & 1) != 0;   // uniform
+    for (unsigned i = (fill_tiles ? 0u : c.L.ZR) + c.tid * 16u; i < c.L.TR; i += HR::NT * 16u) *reinterpret_cast<u32x4*>(smem + i) = u32x4{0u, 0u, 0u, 0u};
     for (int i = c.tid; i < P.B * HR::ROWSM; i += HR::NT) c.fat(c.L.cb)[i] = kNegBig;
     // (the state rows are written 16*DT columns wide but read as GEMM operands over all 32*KS columns: for head
     // dims of 65..80 the columns in between are never written and keep those zeros)
