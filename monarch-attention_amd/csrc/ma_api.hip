@@ -193,7 +193,8 @@ bool resident_fits(const ma_fwd_params* p, bool one_tile) {
 }
 
 // Does the head fit in LDS whole (the head-resident forms of the resident kernel)?  forms = 1: Q, K, V and the
-// state in four tiles; 2: that, or the state and one input tile at a time.
+// state in four tiles; 2: that, or the state and one input tile at a time.  forms = 3 asks something else: would a
+// launch run the two-tile form in workgroups of 4 or 8 waves, several of them per compute unit (many short heads)?
 bool resident_head_fits(const ma_fwd_params* p, int forms = 1) {
     Problem P;
     std::memset(&P, 0, sizeof(P));
@@ -659,7 +660,9 @@ const char* ma_fwd_kernel_name(const ma_fwd_params* p) {
         case MA_VARIANT_FUSED: return "fused_fwd_mfma";
         case MA_VARIANT_CHAINED: return "chain_fwd_mfma";
         case MA_VARIANT_RESIDENT: {
-            if (!f32) return resident_head_fits(p, 1) ? "resident_head_mfma" : resident_head_fits(p, 2) ? "resident_head2_mfma" : "resident_fwd_mfma";
+            if (!f32)
+                return resident_head_fits(p, 3) ? "resident_head2_mfma"
+                       : resident_head_fits(p, 1) ? "resident_head_mfma" : resident_head_fits(p, 2) ? "resident_head2_mfma" : "resident_fwd_mfma";
             Problem P;
             std::memset(&P, 0, sizeof(P));
             P.E = p->E; P.H = p->H; P.N = p->N; P.D = p->D; P.Dv = p->Dv; P.B = p->B; P.T = p->T;

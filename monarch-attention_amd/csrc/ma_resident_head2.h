@@ -16,6 +16,9 @@
 // the K rows when it has formed aL, and the Z problems, which load their query rows a round ahead.
 // A head costs one read of Q, V and (T - 1) reads each of Q and K beyond the first (from L2), and one write of
 // the output; no state leaves the compute unit.
+// Two tiles of a SHORT head are small enough for several workgroups per compute unit: with more heads than compute
+// units the launcher runs this kernel in workgroups of 8 or 4 waves, two or four to a compute unit, each walking
+// its own heads - they are out of step and fill each other's barrier and load waits (ma_resident_launch.h).
 #pragma once
 
 #include "ma_resident_head.h"
@@ -63,7 +66,7 @@ struct HeadRes2 {
 };
 
 template <class T, int DT, int NTB, int NTM, int W, int NI>
-__global__ __launch_bounds__(64 * W) void resident_head2_mfma(Problem P) {
+__device__ __forceinline__ void resident_head2_body(const Problem& P) {
     using H2 = HeadRes2<T, DT, NTB, NTM, W, NI>;
     using HR = typename H2::HR;
     using V8 = typename H2::V8;
@@ -150,6 +153,12 @@ __global__ __launch_bounds__(64 * W) void resident_head2_mfma(Problem P) {
         }
         asm volatile("" ::"v"(warm));   // (keeps the loads)
     }
+}
+
+// WGS: the number of workgroups a compute unit is meant to hold (W * WGS = 16 waves; the register budget follows from it)
+template <class T, int DT, int NTB, int NTM, int W, int NI, int WGS = 1>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(W * WGS / 4))) void resident_head2_mfma(Problem P) {
+    resident_head2_body<T, DT, NTB, NTM, W, NI>(P);
 }
 
 }  // namespace mfma
