@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cM] [--T 1]
                     [--variant auto|generic|staged|fused|resident|chained] [--no-cpu] [--no-sdpa] [--no-sweep]
     python bench.py --sweep-n | --sweep-e        # the reference's own sweep protocol, against dense SDPA
-    python bench.py --sweep-variants [--T 2] [--head-dim 64] [--sweep-grid class96|fewheads]   # every variant over a grid of shapes: AUTO's choice vs the fastest
+    python bench.py --sweep-variants [--T 2] [--head-dim 64] [--sweep-grid class96|fewheads|ragged|mid|short]   # every variant over a grid of shapes: AUTO's choice vs the fastest
     python bench.py --record-traffic FETCH.csv WRITE.csv [--config cM --T 1 --variant auto]
 
 A step is ONE forward call of the hot path (monarch_attention, all T steps)
@@ -168,9 +168,10 @@ def main():
                          "N = 256 .. 8192, blocks of 16 .. 128 rows (T from --T, default 2; head dim from --head-dim); prints the rows "
                          "and how far AUTO's choice is from the fastest variant")
     ap.add_argument("--head-dim", type=int, default=64, help="head dim of --sweep-variants")
-    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96", "fewheads", "ragged", "mid"],
+    ap.add_argument("--sweep-grid", default="pow2", choices=["pow2", "class96", "fewheads", "ragged", "mid", "short"],
                     help="shapes of --sweep-variants: power-of-two lengths and blocks, blocks / block counts in the 96-row tile class, "
-                         "few heads of thousands of tokens, or lengths that are no multiple of the block (197, 500, 1000, 3000, 5000, 7600)")
+                         "few heads of thousands of tokens, lengths that are no multiple of the block (197, 500, 1000, 3000, 5000, 7600), "
+                         "heads of 256 .. 1000 tokens, or up to thousands of heads of at most 256 tokens")
     ap.add_argument("--sweep-dtype", default="f16", choices=["f16", "bf16", "f32"], help="operand dtype of --sweep-variants")
     ap.add_argument("--sweep-mask", action="store_true", help="--sweep-variants with a key / query mask (int64, ~10 %% of the tokens masked out in whole runs)")
     ap.add_argument("--sweep-pre-pad", action="store_true", help="--sweep-variants with the padding at the front")
@@ -307,6 +308,9 @@ def main():
             grid = [(h, N, B) for h in (4, 16, 32, 64, 96, 128, 192, 256, 384, 512, 768)
                     for (N, B) in ((256, 16), (256, 32), (288, 16), (320, 32), (384, 16), (384, 24), (384, 32), (400, 25), (448, 32), (448, 64),
                                    (500, 24), (512, 16), (512, 32), (512, 64), (540, 36), (768, 32), (1000, 32))]
+        elif args.sweep_grid == "short":      # hundreds to thousands of heads of at most 256 tokens (windows, patches): the narrow-workgroup forms
+            grid = [(h, N, B) for h in (64, 128, 256, 384, 512, 768, 1024, 1536, 3072)
+                    for (N, B) in ((49, 7), (64, 16), (96, 16), (128, 16), (128, 32), (160, 32), (197, 16), (224, 32), (256, 16))]
         elif args.sweep_grid == "fewheads":   # 8, 16, 24 heads of thousands of tokens: where the team kernel competes
             grid = [(h, N, B) for h in (8, 16, 24) for N in (2048, 4096, 5000, 6144, 8000, 8192) for B in (32, 64, 128)]
         else:   # blocks and / or block counts of 65 .. 96 rows (and two 128-row shapes with ragged block counts)

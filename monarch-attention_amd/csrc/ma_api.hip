@@ -324,7 +324,26 @@ bool auto_resident(const ma_fwd_params* p, long long heads, long long M) {
     // blocks (0.85 - 0.95 at 256 tokens, 0.55 - 0.8 for shorter heads and three steps; longer heads at D = 32: 1.2 - 1.4
     // below 64 heads; a single step of few heads: 1.03 - 1.23, they stay away).  Head dims up to 64: in the 128-column
     // class the kernel holds heads of ~128 tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
-    if (p->D <= 64 && p->B <= 32 && M <= 32 && (heads >= 96 || (p->T >= 2 && p->B <= 16 && Np <= 256)) && resident_head_fits(p)) return true;
+    // (64 heads of up to 192 tokens in longer blocks, more than one step: 0.84 - 0.95)
+    if (p->D <= 64 && p->B <= 32 && M <= 32 &&
+        (heads >= 96 || (p->T >= 2 && p->B <= 16 && Np <= 256) || (p->T >= 2 && heads >= 64 && Np <= 192)) && resident_head_fits(p))
+        return true;
+    // Head dims of 65 .. 80 (measured at 72), heads of at most 256 tokens that fit in four tiles or two: 0.48 - 0.95 from
+    // 192 heads on for any number of steps (one and a half heads per compute unit: up to 1.05), 0.8 - 1.0 for 128 heads
+    // (224 tokens in 32-row blocks: 1.04 - 1.15), and 0.6 - 0.78 for 64 heads of up to 128 tokens in 16-row blocks with
+    // more than one step
+    if (p->D > 64 && p->D <= 80 && p->B <= 32 && M <= 32 && Np <= 256 && resident_head_fits(p, 2) &&
+        (heads >= 192 || (heads >= 128 && (p->B <= 16 || Np <= 192)) || (heads >= 64 && p->T >= 2 && p->B <= 16 && Np <= 128)))
+        return true;
+    // Head dims above 80 (measured at 96 and 128), more short heads than compute units, in narrow workgroups that share
+    // a compute unit, more than one step: 16-row blocks from 512 heads of 96 tokens and more (0.63 - 0.94) and from 1024
+    // shorter heads (0.69 - 1.04); longer blocks from 1536 heads (0.78 - 1.04).  A single step: 0.84 - 1.3, they stay away.
+    // (D = 128: from 384 heads of 96 tokens and more, 0.87 - 0.93)
+    if (p->D > 80 && p->T >= 2 && resident_head_fits(p, 3) &&
+        (p->B <= 16 ? (heads >= 1024 || (heads >= (p->D > 96 ? 384 : 512) && Np >= 96)) : heads >= 1536))
+        return true;
+    // ... and with three steps and more any 64 .. 256 heads of at most 128 tokens in 16-row blocks (four tiles, 0.79 - 0.87)
+    if (p->D > 80 && p->T >= 3 && p->B <= 16 && Np <= 128 && heads >= 64 && heads <= 256 && resident_head_fits(p)) return true;
     // Heads of about twice that length (257 .. ~540 tokens at D = 64) keep the state and ONE input tile at a time in
     // LDS.  A head has a compute unit to itself for its 2T phases, so the device has to be full of heads: from 192
     // heads on (0.63 - 0.92 at 192 .. 768 heads with T = 2, 3; 0.71 - 1.02 with a single step), and with more than one
@@ -337,7 +356,13 @@ bool auto_resident(const ma_fwd_params* p, long long heads, long long M) {
         if (p->D > 64 && p->D <= 80 && (p->T == 1 || (heads > 256 && heads < 448))) enough = false;
         // head dims above 80 (256 .. 288 tokens at D = 128): 256 tokens in 16-row blocks 0.79 - 0.87 for 192 .. 256 heads, else
         // only where the heads come in whole passes over the compute units (0.82 - 0.97; 192 or 384 heads: 1.03 - 1.24)
-        if (p->D > 80) enough = (heads >= 192 && heads <= 256 && Np <= 256 && p->B <= 16) || (heads >= 224 && heads <= 256) || heads >= 448;
+        if (p->D > 80)
+            enough = (heads >= 192 && heads <= 256 && Np <= 256 && p->B <= 16) || (heads >= 224 && heads <= 256) || heads >= 448 ||
+                     (heads >= 384 && p->T >= 2 && Np <= 256 && p->B <= 16);   // (narrow workgroups: 0.84 - 0.97)
+        // ... a single step of such heads in longer blocks (160 / 224 tokens, 32-row blocks): 1.04 - 1.21
+        if (p->D > 80 && p->T == 1 && p->B > 16) enough = false;
+        // ... and at D = 96 any number of steps of 160 tokens in 32-row blocks: 1.05 - 1.38
+        if (p->D > 80 && p->D <= 96 && p->B > 16 && Np < 224) enough = false;
         if (enough) return true;
     }
     // ... in blocks of 33 .. 64 rows (eight waves per workgroup: 0.89 - 1.22): one pass of 256 heads, 0.88 - 0.91 at T = 2, 3
