@@ -193,8 +193,9 @@ bool resident_fits(const ma_fwd_params* p, bool one_tile) {
 }
 
 // Does the head fit in LDS whole (the head-resident forms of the resident kernel)?  forms = 1: Q, K, V and the
-// state in four tiles; 2: that, or the state and one input tile at a time.  forms = 3 asks something else: would a
-// launch run the two-tile form in workgroups of 4 or 8 waves, several of them per compute unit (many short heads)?
+// state in four tiles; 2: that, or the state and one input tile at a time.  forms = 3, 4 ask something else: would a
+// launch run a head-resident form (4: the four-tile one) in workgroups of 4 or 8 waves, several of them per compute
+// unit (more short heads than compute units)?
 bool resident_head_fits(const ma_fwd_params* p, int forms = 1) {
     Problem P;
     std::memset(&P, 0, sizeof(P));
@@ -686,7 +687,7 @@ const char* ma_fwd_kernel_name(const ma_fwd_params* p) {
         case MA_VARIANT_CHAINED: return "chain_fwd_mfma";
         case MA_VARIANT_RESIDENT: {
             if (!f32)
-                return resident_head_fits(p, 3) ? "resident_head2_mfma"
+                return resident_head_fits(p, 4) ? "resident_head_mfma" : resident_head_fits(p, 3) ? "resident_head2_mfma"
                        : resident_head_fits(p, 1) ? "resident_head_mfma" : resident_head_fits(p, 2) ? "resident_head2_mfma" : "resident_fwd_mfma";
             Problem P;
             std::memset(&P, 0, sizeof(P));

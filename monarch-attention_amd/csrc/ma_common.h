@@ -42,7 +42,7 @@ struct Problem {
     int one_tile_ok;
     // Query only: does a head-resident form of the resident kernel take this head?  1: the one that keeps Q, K and V
     // in LDS beside the state; 2: that one or the two-tile form (the state and one input tile at a time); 3: would a
-    // launch run the two-tile form in narrow workgroups, several to a compute unit?
+    // launch run a head-resident form in narrow workgroups, several to a compute unit?  4: ... the four-tile form?
     int resident_head_only;
     int test_no_spin;    // waits between workgroups give up at once (failure-path tests)
     // Copy of the error word in host memory the device can write (or null): a workgroup that raises the

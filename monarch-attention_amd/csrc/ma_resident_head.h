@@ -554,8 +554,8 @@ struct HeadRes {
     }
 };
 
-template <class T, int DT, int NTB, int NTM, int W, int NI>
-__global__ __launch_bounds__(64 * W) void resident_head_mfma(Problem P) {
+template <class T, int DT, int NTB, int NTM, int W, int NI, int WGS = 1>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(W * WGS / 4))) void resident_head_mfma(Problem P) {
     using HR = HeadRes<T, DT, NTB, NTM, W, NI>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int Np = P.M * P.B;

@@ -199,7 +199,8 @@ def test_kernel_name_follows_the_resolved_variant():
     assert name(64, 12, 256, 64, 16) == "resident_head_mfma"      # the head fits in LDS with its inputs
     assert name(64, 4, 197, 64, 16) == "resident_head_mfma"       # ... a head per compute unit: the widest workgroup
     assert name(64, 12, 197, 64, 16) == "resident_head2_mfma"     # three short heads per compute unit: narrow workgroups, two tiles each
-    assert name(128, 12, 64, 64, 16, T=1) == "resident_head2_mfma"
+    assert name(128, 12, 64, 64, 16, T=1) == "resident_head_mfma"    # ... and four tiles where four fit a share of the LDS
+    assert name(128, 12, 64, 128, 16) == "resident_head2_mfma"        # (not in the 128-column class)
     assert name(16, 12, 512, 64, 32) == "resident_head2_mfma"     # twice that length: the state and one input tile at a time
     assert name(16, 12, 512, 64, 32, T=1) == "resident_head2_mfma"
     assert name(8, 12, 512, 64, 32) == "chain_fwd_mfma"           # ... 96 heads do not fill the device

@@ -249,12 +249,18 @@ TWO_TILE = [  # E, H, N, D, B, T, pre, dt, masked: heads too long for Q, K, V an
     (16, 12, 512, 64, 32, 2, False, "bf16", False), (16, 16, 512, 64, 32, 1, True, "f16", True),   # what 'auto' sends there
 ]
 
-PACKED = [  # E, H, N, D, B, T, pre, dt, masked: more short heads than compute units: the two-tile form in workgroups of 8 or 4 waves
-    (65, 4, 64, 64, 16, 1, False, "f16", False), (130, 6, 64, 64, 16, 2, True, "bf16", True), (200, 4, 96, 32, 16, 3, False, "f16", True),
-    (70, 4, 197, 64, 16, 2, False, "f16", True), (192, 4, 197, 64, 16, 2, True, "f16", False),   # (the second: the ViT shape)
-    (66, 4, 100, 72, 10, 2, False, "f16", True), (65, 4, 60, 128, 12, 3, True, "bf16", True), (260, 4, 50, 128, 10, 1, False, "f16", False),
-    (65, 5, 130, 48, 26, 2, False, "f16", True), (80, 4, 90, 40, 30, 1, True, "bf16", True), (200, 4, 64, 32, 32, 2, False, "f16", False),
-    (210, 4, 100, 32, 5, 2, True, "f16", True), (300, 4, 33, 64, 11, 3, False, "bf16", True),
+PACKED = [  # E, H, N, D, B, T, pre, dt, masked, kernel: more short heads than compute units: a head-resident form in workgroups of 8 or 4 waves
+    # four tiles (head dims of up to 80, heads whose four tiles fit half or a quarter of the LDS)
+    (65, 4, 64, 64, 16, 1, False, "f16", False, "resident_head_mfma"), (130, 6, 64, 64, 16, 2, True, "bf16", True, "resident_head_mfma"),
+    (200, 4, 96, 32, 16, 3, False, "f16", True, "resident_head_mfma"), (80, 4, 90, 40, 30, 1, True, "bf16", True, "resident_head_mfma"),
+    (200, 4, 64, 32, 32, 2, False, "f16", False, "resident_head_mfma"), (210, 4, 100, 32, 5, 2, True, "f16", True, "resident_head_mfma"),
+    (300, 4, 33, 64, 11, 3, False, "bf16", True, "resident_head_mfma"), (300, 4, 96, 64, 16, 2, False, "f16", True, "resident_head_mfma"),
+    (100, 4, 128, 32, 32, 1, True, "bf16", False, "resident_head_mfma"), (70, 4, 80, 72, 16, 3, False, "f16", True, "resident_head_mfma"),
+    (200, 4, 40, 80, 8, 2, True, "f16", False, "resident_head_mfma"),
+    # two tiles (longer heads, and every head dim above 80)
+    (70, 4, 197, 64, 16, 2, False, "f16", True, "resident_head2_mfma"), (192, 4, 197, 64, 16, 2, True, "f16", False, "resident_head2_mfma"),   # (the second: the ViT shape)
+    (66, 4, 100, 72, 10, 2, False, "f16", True, "resident_head2_mfma"), (65, 4, 60, 128, 12, 3, True, "bf16", True, "resident_head2_mfma"),
+    (260, 4, 50, 128, 10, 1, False, "f16", False, "resident_head2_mfma"), (65, 5, 130, 48, 26, 2, False, "f16", True, "resident_head2_mfma"),
 ]
 
 ONE_TILE = [  # heads beyond that whose aL / aR / Y do not fit in LDS as three (or two) tiles either
@@ -289,17 +295,17 @@ def test_resident_kernel_with_the_state_and_one_input_tile(E, H, N, D, B, T, pre
         assert torch.equal(out, auto)
 
 
-@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked", PACKED)
-def test_resident_kernel_in_narrow_workgroups(E, H, N, D, B, T, pre, dt, masked):
-    """Many short heads: the two-tile form of the resident kernel in workgroups of 4 or 8 waves that share a compute
-    unit (and walk several heads each)."""
+@pytest.mark.parametrize("E,H,N,D,B,T,pre,dt,masked,kernel", PACKED)
+def test_resident_kernel_in_narrow_workgroups(E, H, N, D, B, T, pre, dt, masked, kernel):
+    """Many short heads: the head-resident forms of the resident kernel in workgroups of 4 or 8 waves that share a
+    compute unit (and walk several heads each)."""
     q, k, v = seeded_qkv(E, H, N, D, DT[dt], seed=N + B)
     mask = block_safe_mask(E, N, B, seed=B) if masked else None
     ref = monarch_attention_oracle(q, k, v, mask, T, B, pre, upcast=True)
     dev = to_dev(q, k, v, mask)
-    assert resident_kernel_name(dev, T, B, pre) == "resident_head2_mfma"
+    assert resident_kernel_name(dev, T, B, pre) == kernel
     out = monarch_attention_hip(*dev, T, B, pre, variant="resident")
-    assert_parity(out.cpu(), ref, dt, f"packed two-tile resident {(E, H, N, D, B, T, pre, dt, masked)}")
+    assert_parity(out.cpu(), ref, dt, f"narrow-workgroup resident {(E, H, N, D, B, T, pre, dt, masked)}")
     again = monarch_attention_hip(*dev, T, B, pre, variant="resident")
     assert torch.equal(out, again)
 
