@@ -353,6 +353,8 @@ bool auto_resident(const ma_fwd_params* p, long long heads, long long M) {
     const bool two_tiles = !resident_head_fits(p, 1) && resident_head_fits(p, 2);
     if (two_tiles && p->B <= 32 && M <= 32) {
         bool enough = heads >= 192 || (p->T >= 2 && heads >= 128 && Np >= 448 && (M <= 16 || p->B <= 16) && p->D > 48);
+        // ... in 16-row blocks from 384 tokens on for any number of steps (0.83 - 0.95)
+        if (heads >= 128 && p->B <= 16 && Np >= 384 && p->D > 48 && p->D <= 64) enough = true;
         // head dims of 65 .. 80 (measured at 72): a single step 1.24 - 1.35, one and a half passes over the compute units 1.06 - 1.12
         if (p->D > 64 && p->D <= 80 && (p->T == 1 || (heads > 256 && heads < 448))) enough = false;
         // head dims above 80 (256 .. 288 tokens at D = 128): 256 tokens in 16-row blocks 0.79 - 0.87 for 192 .. 256 heads, else
