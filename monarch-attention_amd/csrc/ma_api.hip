@@ -368,8 +368,12 @@ bool auto_resident(const ma_fwd_params* p, long long heads, long long M) {
         if (p->D > 80 && p->D <= 96 && p->B > 16 && Np < 224) enough = false;
         if (enough) return true;
     }
-    // ... in blocks of 33 .. 64 rows (eight waves per workgroup: 0.89 - 1.22): one pass of 256 heads, 0.88 - 0.91 at T = 2, 3
-    if (two_tiles && p->D <= 80 && p->B <= 64 && M <= 64 && p->T >= 2 && heads >= 224 && heads <= 256) return true;
+    // ... in blocks of 33 .. 64 rows (eight waves per workgroup: 0.84 - 1.22): whole passes over the compute units only - one
+    // pass of 256 heads 0.84 - 0.91 at T = 2, 3 and (D <= 64) 0.87 - 0.96 with a single step, two or three passes 0.90 - 0.97
+    // with more than one step (one and a half: 1.09 - 1.22)
+    if (two_tiles && p->D <= 80 && p->B <= 64 && M <= 64 && heads >= 224 && heads <= 256 && (p->T >= 2 || p->D <= 64)) return true;
+    if (two_tiles && p->D <= 64 && p->B <= 64 && M <= 64 && p->T >= 2 && heads >= 448 && heads <= 768 && (heads % 256 == 0 || heads % 256 >= 224))
+        return true;
     // Many short heads in 16-row blocks, whichever form takes them (D = 128: 1.07 - 1.37; D = 72: a single step
     // 1.2 - 1.35, 128 heads 1.03 - 1.16)
     if (p->D <= 80 && p->B <= 16 && M <= 32 && Np <= 288 && heads >= (p->D > 64 ? 192 : 128) && !(p->D > 64 && p->T == 1) &&
