@@ -74,10 +74,13 @@ typedef enum ma_variant {
                             /* of the flag a workgroup waits for, 0.1 - 0.5 s) makes */
                             /* the call fail loudly (NaN rows + error word).  Only   */
                             /* for callers that own the device while the call runs   */
-    MA_VARIANT_RESIDENT = 4,/* MFMA, ONE launch, one workgroup per head with the     */
-                            /* per-head state resident in LDS (heads of up to ~256   */
-                            /* tokens at d = 64; up to ~512 with Y passed through    */
-                            /* the workspace)                                        */
+    MA_VARIANT_RESIDENT = 4,/* MFMA, ONE launch, a workgroup runs whole heads with   */
+                            /* the per-head state resident in LDS: with Q, K, V      */
+                            /* beside it for heads of up to ~256 tokens at d = 64,   */
+                            /* with one input tile at a time up to ~540, with the    */
+                            /* inputs streamed (and Y through the workspace) up to   */
+                            /* ~1000; several narrow workgroups per compute unit     */
+                            /* when there are more short heads than compute units    */
     MA_VARIANT_CHAINED = 5  /* MFMA, ONE launch, one workgroup per block problem of  */
                             /* every phase; a problem starts when its head's         */
                             /* previous phase has released it through the workspace. */
