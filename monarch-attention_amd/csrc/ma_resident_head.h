@@ -141,6 +141,13 @@ struct HeadRes {
             off[i] = ok ? static_cast<unsigned>(t) * st + ch * 16 : kOob;
         }
     }
+    // POL: the cache policy of the row loads (compile time: a run-time choice between two runs of loads into the same
+    // registers measured 1.02 - 1.18 of the time - the merged registers cost the prefetch its head start).  The four-tile
+    // kernel reads every input exactly once and streams them (kPolStream), which leaves the L2 to the rows other compute
+    // units are waiting for: 0.91 - 0.98 for 192 heads and more of 224 .. 256 tokens (the ViT shape at N = 256: 34.7 -> 33.3 us),
+    // 1.02 - 1.04 for 64 .. 128 such heads with more than one step, +-1 % elsewhere.  The two-tile kernel reads Q and K
+    // again later and keeps the ordinary policy (streamed: the ViT shape 28.2 -> 29.8 us).
+    template <int POL = 0>
     static __device__ __forceinline__ void issue_q(const Problem& P, const Ctx& c, const Head& hd, Pre& pre, bool live = true) {
         if (P.mask != nullptr) {   // uniform; first: whoever looks at it waits for nothing issued behind it
             // the thread's entry of tokb: block tid / ROWSB, row tid % ROWSB
@@ -154,19 +161,21 @@ struct HeadRes {
         unsigned off[NI];
         chunk_offsets(P, c, c.qst, off, live);
 #pragma unroll
-        for (int i = 0; i < NI; ++i) pre.q[i] = bload16<false>(hd.q, off[i]);
+        for (int i = 0; i < NI; ++i) pre.q[i] = bload16<POL>(hd.q, off[i]);
     }
+    template <int POL = 0>
     static __device__ __forceinline__ void issue_k(const Problem& P, const Ctx& c, const Head& hd, Pre& pre) {
         unsigned off[NI];
         chunk_offsets(P, c, c.kst, off);
 #pragma unroll
-        for (int i = 0; i < NI; ++i) pre.k[i] = bload16<false>(hd.k, off[i]);
+        for (int i = 0; i < NI; ++i) pre.k[i] = bload16<POL>(hd.k, off[i]);
     }
+    template <int POL = 0>
     static __device__ __forceinline__ void issue_v(const Problem& P, const Ctx& c, const Head& hd, Pre& pre) {
         unsigned off[NI];
         chunk_offsets(P, c, c.vst, off);
 #pragma unroll
-        for (int i = 0; i < NI; ++i) pre.v[i] = bload16<false>(hd.v, off[i]);
+        for (int i = 0; i < NI; ++i) pre.v[i] = bload16<POL>(hd.v, off[i]);
     }
     // write a thread's chunks to the tile at byte offset `tile` (chunks beyond the tile go to the row nobody reads)
     static __device__ __forceinline__ void commit_tile(const Problem& P, const Ctx& c, unsigned tile, const u32x4 (&val)[NI]) {
@@ -592,9 +601,9 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(W * WGS 
     if (head >= heads) return;
     typename HR::Pre pre = {};
     typename HR::Head hd = HR::head_of(P, c, head);
-    HR::issue_q(P, c, hd, pre);
-    HR::issue_k(P, c, hd, pre);
-    HR::issue_v(P, c, hd, pre);
+    HR::template issue_q<kPolStream>(P, c, hd, pre);
+    HR::template issue_k<kPolStream>(P, c, hd, pre);
+    HR::template issue_v<kPolStream>(P, c, hd, pre);
     HR::commit_tile(P, c, c.L.Q, pre.q);
     HR::commit_tile(P, c, c.L.K, pre.k);
     HR::commit_tile(P, c, c.L.V, pre.v);
@@ -613,9 +622,9 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(W * WGS 
         // starting them in front of a later phase, or a tile per phase, measured 1 - 2 us slower per forward.)
         if (more) {
             hn = HR::head_of(P, c, next);
-            HR::issue_q(P, c, hn, pre);
-            HR::issue_k(P, c, hn, pre);
-            HR::issue_v(P, c, hn, pre);
+            HR::template issue_q<kPolStream>(P, c, hn, pre);
+            HR::template issue_k<kPolStream>(P, c, hn, pre);
+            HR::template issue_v<kPolStream>(P, c, hn, pre);
         }
         for (int ph = 0; ph < nph - 1; ++ph) {
             if (ph & 1) {
