@@ -325,16 +325,18 @@ bool auto_resident(const ma_fwd_params* p, long long heads, long long M) {
     // blocks (0.85 - 0.95 at 256 tokens, 0.55 - 0.8 for shorter heads and three steps; longer heads at D = 32: 1.2 - 1.4
     // below 64 heads; a single step of few heads: 1.03 - 1.23, they stay away).  Head dims up to 64: in the 128-column
     // class the kernel holds heads of ~128 tokens and takes 1.0 - 1.35 of the chained kernel's time on them.
-    // (64 heads of up to 192 tokens in longer blocks, more than one step: 0.84 - 0.95)
+    // (64 heads in longer blocks, more than one step: 0.84 - 0.96; D = 48 at 256 tokens: 1.02)
     if (p->D <= 64 && p->B <= 32 && M <= 32 &&
-        (heads >= 96 || (p->T >= 2 && p->B <= 16 && Np <= 256) || (p->T >= 2 && heads >= 64 && Np <= 192)) && resident_head_fits(p))
+        (heads >= 96 || (p->T >= 2 && p->B <= 16 && Np <= 256) || (p->T >= 2 && heads >= 64 && Np <= 256) ||
+         (heads >= 64 && Np <= 128 && p->B <= 16 && p->D > 32)) &&   // (a single step of 64 short heads: 0.88 - 0.91; D = 32: 1.0)
+        resident_head_fits(p))
         return true;
     // Head dims of 65 .. 80 (measured at 72), heads of at most 256 tokens that fit in four tiles or two: 0.48 - 0.95 from
     // 192 heads on for any number of steps (one and a half heads per compute unit: up to 1.05), 0.8 - 1.0 for 128 heads
     // (224 tokens in 32-row blocks: 1.04 - 1.15), and 0.6 - 0.78 for 64 heads of up to 128 tokens in 16-row blocks with
     // more than one step
     if (p->D > 64 && p->D <= 80 && p->B <= 32 && M <= 32 && Np <= 256 && resident_head_fits(p, 2) &&
-        (heads >= 192 || (heads >= 128 && (p->B <= 16 || Np <= 192)) || (heads >= 64 && p->T >= 2 && p->B <= 16 && Np <= 128)))
+        (heads >= 192 || (heads >= 128 && (p->B <= 16 || Np <= 192)) || (heads >= 64 && p->B <= 16 && Np <= (p->T >= 2 ? 128 : 64))))
         return true;
     // Head dims above 80 (measured at 96 and 128), more short heads than compute units, in narrow workgroups that share
     // a compute unit, more than one step: 16-row blocks from 512 heads of 96 tokens and more (0.63 - 0.94) and from 1024
