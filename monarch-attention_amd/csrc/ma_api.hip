@@ -343,8 +343,12 @@ bool auto_resident(const ma_fwd_params* p, long long heads, long long M) {
     // shorter heads (0.69 - 1.04); longer blocks from 1536 heads (0.78 - 1.04).  A single step: 0.84 - 1.3, they stay away.
     // (D = 128: from 384 heads of 96 tokens and more, 0.87 - 0.93)
     if (p->D > 80 && p->T >= 2 && resident_head_fits(p, 3) &&
-        (p->B <= 16 ? (heads >= 1024 || (heads >= (p->D > 96 ? 384 : 512) && Np >= 96)) : heads >= 1536))
+        (p->B <= 16 ? (heads >= (p->D > 96 ? 768 : 1024) || (heads >= (p->D > 96 ? 384 : 512) && Np >= 96)) : heads >= (p->D > 96 ? 1024 : 1536)))
         return true;
+    // ... D = 128 beyond that: a single step of 1024 heads and more of 96 tokens and more in 16-row blocks (0.84 - 0.97), and
+    // with more than one step 192 .. 256 heads of 96 .. 128 tokens (four tiles, one workgroup each: 0.87 - 0.94)
+    if (p->D > 96 && p->T == 1 && p->B <= 16 && Np >= 96 && heads >= 1024 && resident_head_fits(p, 3)) return true;
+    if (p->D > 96 && p->T >= 2 && p->B <= 16 && Np >= 96 && Np <= 128 && heads >= 192 && heads <= 256 && resident_head_fits(p)) return true;
     // ... and with three steps and more any 64 .. 256 heads of at most 128 tokens in 16-row blocks (four tiles, 0.79 - 0.87)
     if (p->D > 80 && p->T >= 3 && p->B <= 16 && Np <= 128 && heads >= 64 && heads <= 256 && resident_head_fits(p)) return true;
     // Heads of about twice that length (257 .. ~540 tokens at D = 64) keep the state and ONE input tile at a time in
